@@ -1,0 +1,127 @@
+"""Typed model descriptions.
+
+Two layers of description live here:
+
+* ``ModelPlan`` is what the engine runs: which parts make each layer (mixer,
+  feed-forward, norms, block arrangement), in which order layers are called and
+  which cache slot each call uses.  It is pure data; nothing in it names an
+  architecture.
+* An architecture's own frozen config dataclass (``Qwen3Config`` in
+  ``tokamak_amd.models.qwen3``) is parsed from the keys of its ``config.json``
+  and turned into a plan by the architecture entry in the registry.
+
+The reference keeps one flat ``ModelConfig`` for three architectures
+(reference: src/tokamak/config.py:29-126); here every number a part needs is a
+parameter of that part's ``PartSpec``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any
+
+
+def _freeze(value: Any) -> Any:
+    if isinstance(value, dict):
+        return tuple(sorted((k, _freeze(v)) for k, v in value.items()))
+    if isinstance(value, (list, tuple)):
+        return tuple(_freeze(v) for v in value)
+    return value
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """Name of a registered part plus its constructor parameters."""
+
+    kind: str
+    params: tuple[tuple[str, Any], ...] = ()
+
+    @classmethod
+    def of(cls, kind: str, **params: Any) -> PartSpec:
+        return cls(kind, tuple(sorted((k, _freeze(v)) for k, v in params.items())))
+
+    def as_dict(self) -> dict[str, Any]:
+        return dict(self.params)
+
+    def __getitem__(self, key: str) -> Any:
+        for k, v in self.params:
+            if k == key:
+                return v
+        raise KeyError(key)
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One layer: two sub-layers (mixer, feed-forward), each behind a norm.
+
+    ``block`` names the arrangement (residual topology) that puts them together.
+    """
+
+    mixer: PartSpec
+    feed_forward: PartSpec
+    mixer_norm: PartSpec
+    feed_forward_norm: PartSpec
+    block: PartSpec = field(default_factory=lambda: PartSpec.of("pre_norm"))
+    # checkpoint sub-prefix of each part inside the layer's own prefix
+    mixer_prefix: str = "self_attn."
+    feed_forward_prefix: str = "mlp."
+    mixer_norm_prefix: str = "input_layernorm."
+    feed_forward_norm_prefix: str = "post_attention_layernorm."
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    """One entry of the run order.
+
+    ``layer`` indexes ``ModelPlan.layers`` (the weights); the same layer may be
+    called more than once.  ``cache`` is the cache slot the call's mixer uses;
+    two calls with the same slot share what is stored there.  A call with
+    ``writes_cache=False`` only reads the slot (it attends over keys and values
+    another call stored) and stores nothing itself.
+    """
+
+    layer: int
+    cache: int
+    writes_cache: bool = True
+
+
+@dataclass(frozen=True)
+class ModelPlan:
+    """Everything the engine needs to build and run a model."""
+
+    vocab_size: int
+    hidden_size: int
+    max_position_embeddings: int
+    tie_word_embeddings: bool
+    embedding: PartSpec
+    layers: tuple[LayerSpec, ...]
+    order: tuple[LayerCall, ...]
+    final_norm: PartSpec
+    head: PartSpec
+    eos_token_ids: tuple[int, ...] = ()
+    # checkpoint names; ``layer_prefix`` is formatted with the layer index
+    embedding_prefix: str = "model.embed_tokens."
+    layer_prefix: str = "model.layers.{}."
+    final_norm_prefix: str = "model.norm."
+    head_prefix: str = "lm_head."
+
+    def __post_init__(self) -> None:
+        for call in self.order:
+            if not 0 <= call.layer < len(self.layers):
+                raise ValueError(f"run order names layer {call.layer}, model has {len(self.layers)}")
+        writers: dict[int, int] = {}
+        for call in self.order:
+            if call.writes_cache:
+                writers[call.cache] = writers.get(call.cache, 0) + 1
+        for call in self.order:
+            if not call.writes_cache and call.cache not in writers:
+                raise ValueError(f"cache slot {call.cache} is read but never written")
+
+    @property
+    def num_cache_slots(self) -> int:
+        return 1 + max((c.cache for c in self.order), default=-1)
+
+
+def default_order(num_layers: int) -> tuple[LayerCall, ...]:
+    """Each layer once, in index order, each with a cache slot of its own."""
+    return tuple(LayerCall(i, i) for i in range(num_layers))

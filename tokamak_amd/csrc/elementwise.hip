@@ -1,0 +1,240 @@
+// Memory-bound kernels of one step: embedding gather, residual add + RMSNorm,
+// rotary tables, per-head q/k norm + rotation + cache write, SiLU-gate product.
+// The residual stream is float32 in both dtypes; norm statistics, rotation
+// angles and the residual sum are float32.
+#include "common.h"
+
+using namespace tk;
+
+// ---------------------------------------------------------------------------
+// embedding: resid[n, :] = float(table[ids[n], :]); an id outside [0, V) gives NaN
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_gather_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ resid, int H, int V) {
+  const int n = blockIdx.x;
+  const int id = ids[n];
+  float* out = resid + (size_t)n * H;
+  if (id < 0 || id >= V) {
+    for (int d = threadIdx.x; d < H; d += blockDim.x) out[d] = __uint_as_float(0x7fc00000u);
+    return;
+  }
+  const T* row = table + (size_t)id * H;
+  for (int d = threadIdx.x; d < H; d += blockDim.x) out[d] = Elem<T>::load(row + d);
+}
+
+TK_API int tk_embed_gather(int dtype, const void* table, const int* ids, float* resid, int N, int H,
+                           int V, hipStream_t stream) {
+  if (N <= 0) return 0;
+  if (dtype == 0)
+    embed_gather_kernel<float><<<N, 256, 0, stream>>>((const float*)table, ids, resid, H, V);
+  else
+    embed_gather_kernel<bf16_t><<<N, 256, 0, stream>>>((const bf16_t*)table, ids, resid, H, V);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// residual add + RMSNorm over rows of width H.
+//   x = resid[row] (+ delta[row]);  if write_resid: resid[row] = x
+//   out[m] = x * rsqrt(mean(x^2) + eps) * weight
+// row = rows ? rows[m] : m.  With `rows`, write_resid must be 0 (a row could be
+// named twice).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
+                                   const int* __restrict__ rows, const float* __restrict__ weight,
+                                   T* __restrict__ out, int H, float eps, int write_resid) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  const size_t row = rows ? (size_t)rows[m] : (size_t)m;
+  float* x = resid + row * H;
+  const T* dl = delta ? delta + row * H : nullptr;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < H; d += blockDim.x) {
+    float v = x[d];
+    if (dl) {
+      v += Elem<T>::load(dl + d);
+      if (write_resid) x[d] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float rstd = rsqrtf(ss / (float)H + eps);
+  T* o = out + (size_t)m * H;
+  for (int d = threadIdx.x; d < H; d += blockDim.x) {
+    float v = x[d];
+    if (dl && !write_resid) v += Elem<T>::load(dl + d);
+    Elem<T>::store(o + d, v * rstd * weight[d]);
+  }
+}
+
+TK_API int tk_add_rmsnorm(int dtype, float* resid, const void* delta, const int* rows,
+                          const float* weight, void* out, int M, int H, float eps, int write_resid,
+                          hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (rows && write_resid) return -1;
+  if (dtype == 0)
+    add_rmsnorm_kernel<float><<<M, 256, 0, stream>>>(resid, (const float*)delta, rows, weight,
+                                                     (float*)out, H, eps, write_resid);
+  else
+    add_rmsnorm_kernel<bf16_t><<<M, 256, 0, stream>>>(resid, (const bf16_t*)delta, rows, weight,
+                                                      (bf16_t*)out, H, eps, write_resid);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// rotary tables: angle = float(pos) * inv_freq[j]  (one float32 product, as the
+// formula is written), cos/sin [N, half]
+// ---------------------------------------------------------------------------
+__global__ void rope_tables_kernel(const int* __restrict__ positions,
+                                   const float* __restrict__ inv_freq, float* __restrict__ cos_t,
+                                   float* __restrict__ sin_t, int N, int half) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N * half) return;
+  const int n = i / half, j = i - n * half;
+  const float angle = __fmul_rn((float)positions[n], inv_freq[j]);
+  cos_t[i] = cosf(angle);
+  sin_t[i] = sinf(angle);
+}
+
+TK_API int tk_rope_tables(const int* positions, const float* inv_freq, float* cos_t, float* sin_t,
+                          int N, int half, hipStream_t stream) {
+  const int total = N * half;
+  if (total <= 0) return 0;
+  rope_tables_kernel<<<(total + 255) / 256, 256, 0, stream>>>(positions, inv_freq, cos_t, sin_t, N,
+                                                               half);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// per-head RMSNorm of q and k, half-split rotation of the first `rot` dims,
+// q written out, k and v written into the paged cache.
+//
+// qkv: [N, (nh + 2*nkv) * hd] (q heads, then k heads, then v heads); with
+// nkv_in == 0 the input holds q heads only and nothing is stored.
+// Cache pages (page_elems = nkv * hd * ps elements each):
+//   K page: [nkv][hd/8][ps][8]   (8 consecutive dims of one token are adjacent,
+//                                 then tokens, so lanes that hold consecutive
+//                                 tokens read consecutive 16-byte pieces)
+//   V page: [nkv][hd][ps]        (tokens of one dim adjacent)
+// One 64-lane block per (token, head).
+// ---------------------------------------------------------------------------
+constexpr int kMaxHeadDim = 512;
+
+template <typename T>
+__global__ void qknorm_rope_store_kernel(
+    const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions, const int* __restrict__ req_of_token,
+    const int* __restrict__ block_tables, T* __restrict__ q_out, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, int nh, int nkv_in, int nkv, int hd, int rot, int ps, int max_pages,
+    float eps) {
+  __shared__ float vec[kMaxHeadDim];
+  const int n = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int row_width = (nh + 2 * nkv_in) * hd;
+  const T* src = qkv + (size_t)n * row_width + (size_t)head * hd;
+  const bool is_q = head < nh;
+  const bool is_k = !is_q && head < nh + nkv_in;
+  const float* w = is_q ? q_weight : (is_k ? k_weight : nullptr);
+
+  float ss = 0.f;
+  for (int d = lane; d < hd; d += kWave) {
+    const float v = Elem<T>::load(src + d);
+    vec[d] = v;
+    ss += v * v;
+  }
+  if (is_q || is_k) {
+    if (w) {
+      ss = wave_sum(ss);
+      const float rstd = rsqrtf(ss / (float)hd + eps);
+      __syncthreads();
+      for (int d = lane; d < hd; d += kWave) vec[d] = vec[d] * rstd * w[d];
+    }
+    __syncthreads();
+    // out[j] = x[j] cos_j - x[j+half] sin_j ; out[j+half] = x[j+half] cos_j + x[j] sin_j
+    const int half = rot / 2;
+    float lo[kMaxHeadDim / 2 / kWave], hi[kMaxHeadDim / 2 / kWave];
+    int cnt = 0;
+    for (int j = lane; j < half; j += kWave, ++cnt) {
+      const float c = cos_t[(size_t)n * half + j], s = sin_t[(size_t)n * half + j];
+      const float a = vec[j], b = vec[j + half];
+      lo[cnt] = a * c - b * s;
+      hi[cnt] = b * c + a * s;
+    }
+    __syncthreads();
+    cnt = 0;
+    for (int j = lane; j < half; j += kWave, ++cnt) {
+      vec[j] = lo[cnt];
+      vec[j + half] = hi[cnt];
+    }
+  }
+  __syncthreads();
+
+  if (is_q) {
+    T* dst = q_out + ((size_t)n * nh + head) * hd;
+    for (int d = lane; d < hd; d += kWave) Elem<T>::store(dst + d, vec[d]);
+    return;
+  }
+  const int pos = positions[n];
+  const int page = block_tables[(size_t)req_of_token[n] * max_pages + pos / ps];
+  const int off = pos % ps;
+  const size_t page_elems = (size_t)nkv * hd * ps;
+  if (is_k) {
+    const int kvh = head - nh;
+    T* base = k_cache + (size_t)page * page_elems + (size_t)kvh * hd * ps;
+    for (int d = lane; d < hd; d += kWave)
+      Elem<T>::store(base + ((size_t)(d >> 3) * ps + off) * 8 + (d & 7), vec[d]);
+  } else {
+    const int kvh = head - nh - nkv_in;
+    T* base = v_cache + (size_t)page * page_elems + (size_t)kvh * hd * ps;
+    for (int d = lane; d < hd; d += kWave) Elem<T>::store(base + (size_t)d * ps + off, vec[d]);
+  }
+}
+
+TK_API int tk_qknorm_rope_store(int dtype, const void* qkv, const float* q_weight,
+                                const float* k_weight, const float* cos_t, const float* sin_t,
+                                const int* positions, const int* req_of_token,
+                                const int* block_tables, void* q_out, void* k_cache, void* v_cache,
+                                int N, int nh, int nkv_in, int nkv, int hd, int rot, int ps,
+                                int max_pages, float eps, hipStream_t stream) {
+  if (N <= 0) return 0;
+  if (hd > kMaxHeadDim || hd % 8 != 0 || rot > hd || rot % 2 != 0) return -1;
+  if (nkv_in != 0 && nkv_in != nkv) return -1;
+  dim3 grid(N, nh + 2 * nkv_in);
+  if (dtype == 0)
+    qknorm_rope_store_kernel<float><<<grid, kWave, 0, stream>>>(
+        (const float*)qkv, q_weight, k_weight, cos_t, sin_t, positions, req_of_token, block_tables,
+        (float*)q_out, (float*)k_cache, (float*)v_cache, nh, nkv_in, nkv, hd, rot, ps, max_pages,
+        eps);
+  else
+    qknorm_rope_store_kernel<bf16_t><<<grid, kWave, 0, stream>>>(
+        (const bf16_t*)qkv, q_weight, k_weight, cos_t, sin_t, positions, req_of_token, block_tables,
+        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv_in, nkv, hd, rot, ps, max_pages,
+        eps);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// out[n, i] = silu(gu[n, i]) * gu[n, I + i],  silu(z) = z / (1 + exp(-z))
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t n = idx / I;
+  const int i = (int)(idx - n * I);
+  const float g = Elem<T>::load(gu + n * 2 * I + i);
+  const float u = Elem<T>::load(gu + n * 2 * I + I + i);
+  Elem<T>::store(out + idx, g / (1.f + expf(-g)) * u);
+}
+
+TK_API int tk_silu_mul(int dtype, const void* gu, void* out, int N, int I, hipStream_t stream) {
+  if (N <= 0 || I <= 0) return 0;
+  const size_t total = (size_t)N * I;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == 0)
+    silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
+  else
+    silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
+  return launch_status();
+}

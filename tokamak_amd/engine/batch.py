@@ -1,0 +1,101 @@
+"""The step descriptor: one flat batch of tokens from several requests.
+
+The reference runs either one whole sequence or B single tokens, in a padded
+[batch, seq] layout (src/tokamak/engine/llm.py:347-388).  Here a step is N
+tokens from R requests; request r contributes ``q_len[r]`` consecutive tokens
+that start at absolute position ``ctx_len[r]`` (what its cache already holds).
+A decode token is a span of length one, a prompt portion a longer one; any
+mixture is one batch.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepSpan:
+    """One request's share of a step."""
+
+    request: object
+    tokens: list[int]
+    ctx_len: int                 # tokens of this request already in the cache
+    state_slot: int
+    tables: list[list[int]]      # block table per cache group
+    want: list[int] = field(default_factory=list)  # offsets within ``tokens`` whose logits are wanted
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_requests: int
+    num_logit_rows: int
+    token_ids: torch.Tensor      # [N] int32
+    positions: torch.Tensor      # [N] int32
+    req_of_token: torch.Tensor   # [N] int32, row of the request in this batch
+    q_start: torch.Tensor        # [R+1] int32, first token of each request
+    ctx_len: torch.Tensor        # [R] int32, cached tokens before this step
+    state_slots: torch.Tensor    # [R] int32
+    logit_rows: torch.Tensor     # [M] int32, token rows whose logits are wanted
+    block_tables: list[torch.Tensor]  # per cache group [R, max_pages] int32
+    # host copies, for choosing kernels and grids
+    q_lens: list[int] = field(default_factory=list)
+    ctx_lens: list[int] = field(default_factory=list)
+    max_q_len: int = 0
+    max_seq_len: int = 0
+    memo: dict = field(default_factory=dict)  # per-step data shared between layers
+
+
+def build_batch(spans: list[StepSpan], num_groups: int, device) -> StepBatch:
+    """Pack the descriptor into one host buffer and copy it to the device once."""
+    r = len(spans)
+    n = sum(len(s.tokens) for s in spans)
+    widths = []
+    for g in range(num_groups):
+        w = max((len(s.tables[g]) for s in spans), default=0)
+        widths.append(max(4, -(-w // 4) * 4))
+    m = sum(len(s.want) for s in spans)
+    sizes = [n, n, n, r + 1, r, r, m] + [r * w for w in widths]
+    offsets = np.concatenate([[0], np.cumsum(sizes)])
+    buf = np.zeros(int(offsets[-1]), dtype=np.int32)
+    tok, pos, req, qs, ctx, slots, rows = (buf[offsets[i]:offsets[i + 1]] for i in range(7))
+    tabs = [buf[offsets[7 + g]:offsets[8 + g]].reshape(r, widths[g]) for g in range(num_groups)]
+    at = 0
+    mi = 0
+    for i, s in enumerate(spans):
+        q = len(s.tokens)
+        tok[at:at + q] = s.tokens
+        pos[at:at + q] = np.arange(s.ctx_len, s.ctx_len + q, dtype=np.int32)
+        req[at:at + q] = i
+        qs[i] = at
+        ctx[i] = s.ctx_len
+        slots[i] = s.state_slot
+        for w in s.want:
+            if not 0 <= w < q:
+                raise ValueError(f"wanted offset {w} is outside a span of {q} tokens")
+            rows[mi] = at + w
+            mi += 1
+        for g in range(num_groups):
+            t = s.tables[g]
+            # entries released behind a window are never read; keep them in range
+            tabs[g][i, :len(t)] = [p if p >= 0 else 0 for p in t]
+        at += q
+    qs[r] = at
+    host = torch.from_numpy(buf)
+    if torch.device(device).type == "cuda":
+        dev = host.pin_memory().to(device, non_blocking=True)
+    else:
+        dev = host.to(device)
+    parts = [dev[int(offsets[i]):int(offsets[i + 1])] for i in range(7 + num_groups)]
+    return StepBatch(
+        num_tokens=n, num_requests=r, num_logit_rows=m,
+        token_ids=parts[0], positions=parts[1], req_of_token=parts[2], q_start=parts[3],
+        ctx_len=parts[4], state_slots=parts[5], logit_rows=parts[6],
+        block_tables=[parts[7 + g].view(r, widths[g]) for g in range(num_groups)],
+        q_lens=[len(s.tokens) for s in spans], ctx_lens=[s.ctx_len for s in spans],
+        max_q_len=max((len(s.tokens) for s in spans), default=0),
+        max_seq_len=max((s.ctx_len + len(s.tokens) for s in spans), default=0),
+    )

@@ -1,0 +1,130 @@
+"""The step function: run a batch of (request, its next tokens) from the cache.
+
+One ``ModelRunner`` owns the model, the cache manager and the cache memory.
+``step`` runs only the tokens it is given, as one batch, against what earlier
+steps left in the cache, and returns float32 logits at the wanted places.
+Generation (``LLM``), the scheduler and trace replay all drive this one
+function.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from pathlib import Path
+
+import torch
+
+from tokamak_amd.cache.manager import CacheManager
+from tokamak_amd.config.registry import load_model_description
+from tokamak_amd.engine.batch import StepBatch, StepSpan, build_batch
+from tokamak_amd.engine.model import LayeredModel
+from tokamak_amd.engine.storage import CacheStorage
+from tokamak_amd.weights.loader import load_weights
+from tokamak_amd.weights.sources import SafetensorsSource
+
+DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32,
+          torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def resolve_dtype(dtype) -> torch.dtype:
+    try:
+        return DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}") from None
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens, and the offsets among them whose logits are wanted."""
+
+    request: object
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)
+
+
+class ModelRunner:
+    def __init__(self, plan, source, *, dtype="bfloat16", page_size: int = 16,
+                 kv_pool_tokens: int, max_requests: int = 64,
+                 device: str | torch.device = "cuda:0") -> None:
+        self.dtype = resolve_dtype(dtype)
+        self.device = torch.device(device)
+        if self.device.type != "cuda" or not torch.cuda.is_available():
+            raise RuntimeError("tokamak_amd runs on a GPU only; no GPU is visible")
+        if page_size < 8 or page_size % 8:
+            raise ValueError(f"page_size must be a multiple of 8, got {page_size}")
+        self.plan = plan
+        self.page_size = page_size
+        self.model = LayeredModel(plan, dtype=self.dtype, device=self.device)
+        load_weights(self.model, source, dtype=self.dtype, device=self.device)
+        groups, _ = self.model.cache_layout()
+        num_pages = max(1, -(-int(kv_pool_tokens) // page_size))
+        self.manager = CacheManager(groups, num_pages, page_size, max_requests)
+        self.storage = CacheStorage(self.model, [num_pages] * len(groups), page_size, max_requests,
+                                    dtype=self.dtype, device=self.device)
+        self.num_groups = len(groups)
+        self._ctx_len: dict[object, int] = {}
+
+    @classmethod
+    def from_folder(cls, folder: str | Path, **kwargs) -> ModelRunner:
+        _, _, plan = load_model_description(folder)
+        return cls(plan, SafetensorsSource(folder), **kwargs)
+
+    # -- request lifetime ------------------------------------------------------
+    def cached_tokens(self, request) -> int:
+        return self._ctx_len.get(request, 0)
+
+    def is_live(self, request) -> bool:
+        return request in self._ctx_len
+
+    def end(self, request) -> None:
+        """The request is finished (or preempted): give back what it holds."""
+        self._ctx_len.pop(request, None)
+        self.manager.free(request)
+
+    def end_all(self) -> None:
+        for request in list(self._ctx_len):
+            self.end(request)
+
+    # -- the step --------------------------------------------------------------
+    def prepare(self, entries: list[StepEntry]) -> StepBatch:
+        spans = []
+        vocab = self.plan.vocab_size
+        for e in entries:
+            if not e.tokens:
+                raise ValueError(f"request {e.request!r} brings no tokens to this step")
+            if min(e.tokens) < 0 or max(e.tokens) >= vocab:
+                raise ValueError(f"request {e.request!r} has a token id outside [0, {vocab})")
+            ctx = self._ctx_len.get(e.request)
+            if ctx is None:
+                slot = self.manager.admit(e.request)
+                self.storage.reset_state(slot)
+                ctx = 0
+                self._ctx_len[e.request] = 0
+            total = ctx + len(e.tokens)
+            if total > self.plan.max_position_embeddings:
+                raise ValueError(
+                    f"request {e.request!r} would reach {total} tokens; the model's limit is "
+                    f"{self.plan.max_position_embeddings}")
+            self.manager.release_behind_window(e.request, ctx)
+            self.manager.ensure_capacity(e.request, total)
+            spans.append(StepSpan(
+                request=e.request, tokens=list(e.tokens), ctx_len=ctx,
+                state_slot=self.manager.slots.slot_of(e.request),
+                tables=[self.manager.block_table(e.request, g) for g in range(self.num_groups)],
+                want=list(e.want)))
+        if len({id(s.request) if not isinstance(s.request, (int, str)) else s.request for s in spans}) != len(spans):
+            raise ValueError("a request appears twice in one step")
+        return build_batch(spans, self.num_groups, self.device)
+
+    @torch.inference_mode()
+    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+        """Run the entries as one batch; logits float32 [wanted, vocab], in the
+        order of the entries and of each entry's ``want``."""
+        if not entries:
+            return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
+        batch = self.prepare(entries)
+        with torch.cuda.device(self.device):
+            logits = self.model.forward(batch, self.storage)
+        for e in entries:
+            self._ctx_len[e.request] += len(e.tokens)
+        return logits

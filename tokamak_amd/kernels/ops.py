@@ -1,0 +1,253 @@
+"""Python face of the HIP kernels.
+
+Every function checks on the host that shapes, dtypes and devices match what
+the kernel and its grid assume, then launches on torch's current stream.  There
+is no CPU path and no library fallback: without a GPU tensor or without the
+compiled library the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+
+import torch
+
+from tokamak_amd.kernels.build import load_library
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DT[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16, not {dtype}") from None
+
+
+def _p(t: torch.Tensor | None) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(*tensors: torch.Tensor | None) -> None:
+    for t in tensors:
+        if t is None:
+            continue
+        _need(t.is_cuda, "kernel arguments must live on the GPU (there is no CPU path)")
+        _need(t.is_contiguous(), "kernel arguments must be contiguous")
+
+
+def _check(status: int, name: str) -> None:
+    if status != 0:
+        raise KernelError(f"{name} failed with status {status}")
+
+
+_SIGS = {
+    "elementwise": {
+        "tk_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "tk_add_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                           c_float, c_int, c_void_p],
+        "tk_rope_tables": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+        "tk_qknorm_rope_store": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+        "tk_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    },
+    "gemm_tiled": {
+        "tk_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long,
+                          c_long, c_long, c_void_p],
+    },
+    "attention_generic": {
+        "tk_paged_attention_generic": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                       c_float, c_int, c_void_p],
+    },
+    "sampling": {
+        "tk_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+        "tk_sample": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                      c_void_p, c_void_p, c_void_p, c_void_p],
+    },
+}
+_fns: dict[str, ctypes._CFuncPtr] = {}
+
+
+def _fn(library: str, name: str):
+    fn = _fns.get(name)
+    if fn is None:
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: tokamak_amd runs on an MI355X only")
+        lib = load_library(library)
+        fn = getattr(lib, name)
+        fn.argtypes = _SIGS[library][name]
+        fn.restype = c_int
+        _fns[name] = fn
+    return fn
+
+
+# ---------------------------------------------------------------------------
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, resid: torch.Tensor) -> None:
+    """resid[n] = float(table[ids[n]]); resid is float32 [N, H]."""
+    _gpu(table, ids, resid)
+    n = ids.numel()
+    v, h = table.shape
+    _need(ids.dtype == torch.int32, "token ids must be int32")
+    _need(resid.dtype == torch.float32 and resid.shape[-1] == h and resid.numel() >= n * h,
+          "residual buffer must be float32 [>=N, H]")
+    _check(_fn("elementwise", "tk_embed_gather")(_code(table.dtype), _p(table), _p(ids), _p(resid),
+                                                 n, h, v, _stream()), "embed_gather")
+
+
+def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: torch.Tensor | None = None,
+                write_resid: bool = True) -> None:
+    """x = resid[row] (+ delta[row]); optionally stored back; out = rmsnorm(x) * weight."""
+    _gpu(resid, delta, weight, out, rows)
+    h = resid.shape[-1]
+    m = out.shape[0] if rows is None else rows.numel()
+    _need(resid.dtype == torch.float32 and weight.dtype == torch.float32, "residual and norm weight are float32")
+    _need(weight.numel() == h and out.shape[-1] == h and out.shape[0] >= m, "rmsnorm shapes disagree")
+    if rows is None:
+        _need(resid.shape[0] >= m, "residual has fewer rows than the output")
+    else:
+        _need(rows.dtype == torch.int32 and not (write_resid and delta is not None),
+              "row-indexed rmsnorm cannot write the residual")
+        write_resid = False
+    if delta is not None:
+        _need(delta.dtype == out.dtype and delta.shape == resid.shape, "delta must match the residual's shape")
+    _check(_fn("elementwise", "tk_add_rmsnorm")(_code(out.dtype), _p(resid), _p(delta), _p(rows),
+                                                _p(weight), _p(out), m, h, float(eps),
+                                                int(bool(write_resid)), _stream()), "add_rmsnorm")
+
+
+def rope_tables(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor,
+                sin: torch.Tensor) -> None:
+    _gpu(positions, inv_freq, cos, sin)
+    n, half = positions.numel(), inv_freq.numel()
+    _need(positions.dtype == torch.int32 and inv_freq.dtype == torch.float32, "positions int32, inv_freq float32")
+    _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.numel() >= n * half
+          and sin.numel() >= n * half, "cos/sin tables must be float32 [N, half]")
+    _check(_fn("elementwise", "tk_rope_tables")(_p(positions), _p(inv_freq), _p(cos), _p(sin), n,
+                                                half, _stream()), "rope_tables")
+
+
+def qknorm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor | None,
+                      k_weight: torch.Tensor | None, cos: torch.Tensor, sin: torch.Tensor,
+                      positions: torch.Tensor, req_of_token: torch.Tensor,
+                      block_tables: torch.Tensor, q_out: torch.Tensor,
+                      k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, *, num_heads: int,
+                      num_kv_heads: int, head_dim: int, rotary_dim: int, page_size: int, eps: float,
+                      store: bool = True) -> None:
+    """Per-head norm + rotation of q (and k), q written to q_out, k/v into pages."""
+    _gpu(qkv, q_weight, k_weight, cos, sin, positions, req_of_token, block_tables, q_out, k_cache, v_cache)
+    n = positions.numel()
+    nkv_in = num_kv_heads if store else 0
+    width = (num_heads + 2 * nkv_in) * head_dim
+    _need(qkv.shape[-1] == width and qkv.shape[0] >= n, f"qkv must be [N, {width}]")
+    _need(q_out.dtype == qkv.dtype and q_out.numel() >= n * num_heads * head_dim, "q_out too small")
+    _need(head_dim % 8 == 0 and head_dim <= 512, "head_dim must be a multiple of 8, at most 512")
+    _need(rotary_dim % 2 == 0 and rotary_dim <= head_dim, "rotary_dim must be even and <= head_dim")
+    _need(cos.numel() >= n * (rotary_dim // 2) and sin.numel() >= n * (rotary_dim // 2), "rotary tables too small")
+    for w in (q_weight, k_weight):
+        _need(w is None or (w.dtype == torch.float32 and w.numel() == head_dim), "q/k norm weights are float32 [head_dim]")
+    _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32
+          and block_tables.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
+    _need(req_of_token.numel() >= n, "req_of_token shorter than positions")
+    max_pages = block_tables.shape[1]
+    if store:
+        page_elems = num_kv_heads * head_dim * page_size
+        _need(k_cache is not None and v_cache is not None and k_cache.dtype == qkv.dtype
+              and v_cache.dtype == qkv.dtype, "cache dtype must match activations")
+        _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
+    _check(_fn("elementwise", "tk_qknorm_rope_store")(
+        _code(qkv.dtype), _p(qkv), _p(q_weight), _p(k_weight), _p(cos), _p(sin), _p(positions),
+        _p(req_of_token), _p(block_tables), _p(q_out), _p(k_cache), _p(v_cache), n, num_heads,
+        nkv_in, num_kv_heads, head_dim, rotary_dim, page_size, max_pages, float(eps), _stream()),
+        "qknorm_rope_store")
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
+    _gpu(gate_up, out)
+    n, two_i = gate_up.shape
+    _need(two_i % 2 == 0 and out.shape == (n, two_i // 2) and out.dtype == gate_up.dtype, "silu_mul shapes disagree")
+    _check(_fn("elementwise", "tk_silu_mul")(_code(out.dtype), _p(gate_up), _p(out), n, two_i // 2,
+                                             _stream()), "silu_mul")
+
+
+def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out[M, N] = a[M, K] @ w[N, K]^T, float32 multiply-add (rows may be strided)."""
+    for t in (a, w, out):
+        _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and out.shape == (m, n), f"gemm shapes disagree: {tuple(a.shape)} x {tuple(w.shape)}^T -> {tuple(out.shape)}")
+    _need(a.dtype == w.dtype, "gemm inputs must share a dtype")
+    _need(m <= 64 * 65535, "too many rows for one launch")
+    _check(_fn("gemm_tiled", "tk_gemm_tiled")(_code(a.dtype), _code(out.dtype), _p(a), _p(w), _p(out),
+                                              m, n, k, a.stride(0), w.stride(0), out.stride(0),
+                                              _stream()), "gemm_tiled")
+
+
+def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                            block_tables: torch.Tensor, positions: torch.Tensor,
+                            req_of_token: torch.Tensor, out: torch.Tensor, *, num_heads: int,
+                            num_kv_heads: int, head_dim: int, page_size: int, scale: float,
+                            window: int | None = None) -> None:
+    """Causal attention of each query token over its request's pages."""
+    _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, out)
+    n = positions.numel()
+    _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "attention tensors must share a dtype")
+    _need(q.numel() >= n * num_heads * head_dim and out.numel() >= n * num_heads * head_dim, "q/out too small")
+    _need(head_dim % 8 == 0 and head_dim <= 512, "head_dim must be a multiple of 8, at most 512")
+    _need(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
+    page_elems = num_kv_heads * head_dim * page_size
+    _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
+    _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32
+          and block_tables.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
+    _check(_fn("attention_generic", "tk_paged_attention_generic")(
+        _code(q.dtype), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(positions),
+        _p(req_of_token), _p(out), n, num_heads, num_kv_heads, head_dim, page_size,
+        block_tables.shape[1], float(scale), int(window or 0), _stream()), "paged_attention_generic")
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    """out[m] = index of the first maximum of logits[m]."""
+    _need(logits.is_cuda and logits.dim() == 2 and logits.stride(1) == 1 and logits.dtype == torch.float32,
+          "logits are float32 [M, V] on the GPU")
+    _gpu(out)
+    m, v = logits.shape
+    _need(out.dtype == torch.int32 and out.numel() >= m, "argmax output is int32 [M]")
+    _check(_fn("sampling", "tk_argmax")(_p(logits), _p(out), m, v, logits.stride(0), _stream()), "argmax")
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
+           top_p: torch.Tensor, seeds: torch.Tensor, counters: torch.Tensor, out: torch.Tensor,
+           probs_out: torch.Tensor | None = None) -> None:
+    """Temperature / top-k / top-p sampling, one row per request."""
+    _need(logits.is_cuda and logits.dim() == 2 and logits.stride(1) == 1 and logits.dtype == torch.float32,
+          "logits are float32 [M, V] on the GPU")
+    _gpu(temperature, top_k, top_p, seeds, counters, out, probs_out)
+    m, v = logits.shape
+    _need(temperature.dtype == torch.float32 and top_p.dtype == torch.float32 and top_k.dtype == torch.int32,
+          "temperature/top_p float32, top_k int32")
+    _need(seeds.dtype == torch.int64 and counters.dtype == torch.int64, "seeds and counters are int64")
+    for t in (temperature, top_k, top_p, seeds, counters, out):
+        _need(t.numel() >= m, "one sampling parameter per row is required")
+    _need(out.dtype == torch.int32, "sample output is int32")
+    _need(probs_out is None or (probs_out.dtype == torch.float32 and probs_out.shape == (m, v)), "probs_out is float32 [M, V]")
+    _check(_fn("sampling", "tk_sample")(_p(logits), logits.stride(0), m, v, _p(temperature), _p(top_k),
+                                        _p(top_p), _p(seeds), _p(counters), _p(out), _p(probs_out),
+                                        _stream()), "sample")

@@ -1,0 +1,90 @@
+"""Grouped-query attention over a paged cache."""
+
+from __future__ import annotations
+
+import torch
+
+from tokamak_amd.config.registry import get_part, register_part
+from tokamak_amd.kernels import ops
+from tokamak_amd.kernels.attention import paged_attention
+from tokamak_amd.kernels.linear import linear
+from tokamak_amd.parts.base import CacheRequest, Fetch, Mixer
+from tokamak_amd.weights.spec import TensorSpec
+
+
+class GQAAttention(Mixer):
+    """q/k/v projections, optional per-head RMSNorm of q and k, position
+    encoding, causal softmax attention over the request's pages, o projection
+    (reference: src/tokamak/model/transformer.py:22-86).
+
+    Query head a reads kv head a // (num_heads / num_kv_heads).  Keys are cached
+    after norm and rotation, values as projected (transformer.py:71-82).  The
+    three projections are held as one [(nh + 2 nkv) hd, H] matrix.
+    ``window``: None for full causal attention, W to see the last W positions.
+    """
+
+    def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 qk_norm_eps: float | None, softmax_scale: float, position, window: int | None,
+                 dtype, device) -> None:
+        super().__init__(dtype=dtype, device=device)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"num_heads ({num_heads}) must be divisible by num_kv_heads ({num_kv_heads})")
+        if head_dim % 8 or head_dim > 512:
+            raise ValueError(f"head_dim must be a multiple of 8 and at most 512, got {head_dim}")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim = int(head_dim)
+        self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
+        self.softmax_scale = float(softmax_scale)
+        self.window = None if window is None else int(window)
+        kind, params = position
+        self.position = get_part("position", kind)(**dict(params), dtype=dtype, device=device)
+        self.qkv: torch.Tensor | None = None
+        self.o: torch.Tensor | None = None
+        self.q_norm: torch.Tensor | None = None
+        self.k_norm: torch.Tensor | None = None
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        h, nh, nkv, hd = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim
+        out = {
+            prefix + "q_proj.weight": TensorSpec((nh * hd, h)),
+            prefix + "k_proj.weight": TensorSpec((nkv * hd, h)),
+            prefix + "v_proj.weight": TensorSpec((nkv * hd, h)),
+            prefix + "o_proj.weight": TensorSpec((h, nh * hd)),
+        }
+        if self.qk_norm_eps is not None:
+            out[prefix + "q_norm.weight"] = TensorSpec((hd,), role="vector")
+            out[prefix + "k_norm.weight"] = TensorSpec((hd,), role="vector")
+        return out
+
+    def bind(self, prefix: str, fetch: Fetch) -> None:
+        self.qkv = torch.cat([fetch(prefix + n + "_proj.weight") for n in "qkv"], dim=0).contiguous()
+        self.o = fetch(prefix + "o_proj.weight")
+        if self.qk_norm_eps is not None:
+            self.q_norm = fetch(prefix + "q_norm.weight")
+            self.k_norm = fetch(prefix + "k_norm.weight")
+
+    def cache_request(self) -> CacheRequest:
+        return CacheRequest(arrays=("k", "v"), elems_per_token=self.num_kv_heads * self.head_dim,
+                            window=self.window)
+
+    def forward(self, h: torch.Tensor, batch, store, writes_cache: bool = True) -> torch.Tensor:
+        nh, nkv, hd = self.num_heads, self.num_kv_heads, self.head_dim
+        n = h.shape[0]
+        weight = self.qkv if writes_cache else self.qkv[: nh * hd]
+        qkv = linear(h, weight)
+        cos, sin = self.position.prepare(batch)
+        tables = batch.block_tables[store.group]
+        q = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
+        ops.qknorm_rope_store(
+            qkv, self.q_norm, self.k_norm, cos, sin, batch.positions, batch.req_of_token, tables, q,
+            store.arrays["k"], store.arrays["v"], num_heads=nh, num_kv_heads=nkv, head_dim=hd,
+            rotary_dim=self.position.rotary_dim, page_size=store.page_size,
+            eps=self.qk_norm_eps or 0.0, store=writes_cache)
+        attended = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
+        paged_attention(q, store.arrays["k"], store.arrays["v"], tables, batch, attended,
+                        num_heads=nh, num_kv_heads=nkv, head_dim=hd, page_size=store.page_size,
+                        scale=self.softmax_scale, window=self.window)
+        return linear(attended, self.o)
+
+
+register_part("mixer", "gqa_attention", GQAAttention)
