@@ -1,0 +1,120 @@
+"""Configuration and registry (scenarios of reference tests/unit/test_config.py:29-138)."""
+
+import json
+
+import pytest
+
+from tokamak_amd.config import (
+    Architecture, LayerCall, ModelPlan, PartSpec, get_architecture, get_part,
+    load_model_description, register_architecture, supported_architectures,
+)
+from tokamak_amd.models import qwen3
+
+
+def raw(**over):
+    d = {
+        "architectures": ["Qwen3ForCausalLM"], "vocab_size": 1000, "hidden_size": 64,
+        "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 2,
+        "head_dim": 32, "intermediate_size": 128, "rms_norm_eps": 1e-6, "rope_theta": 1e6,
+        "max_position_embeddings": 512, "tie_word_embeddings": True,
+    }
+    d.update(over)
+    return {k: v for k, v in d.items() if v is not ...}
+
+
+def test_qwen3_sample_parses():
+    cfg = qwen3.parse(raw(), (7,))
+    assert cfg.architecture == "Qwen3ForCausalLM"
+    assert cfg.head_dim == 32  # decoupled from hidden_size / num_heads
+    assert cfg.rope_theta == 1e6
+    assert cfg.tie_word_embeddings
+    assert cfg.num_kv_groups == 2
+    assert cfg.eos_token_ids == (7,)
+
+
+def test_defaults_when_keys_absent():
+    cfg = qwen3.parse(raw(head_dim=..., num_key_value_heads=..., tie_word_embeddings=...))
+    assert cfg.head_dim == 16           # hidden_size // num_heads
+    assert cfg.num_kv_heads == 4        # = num_attention_heads
+    assert cfg.tie_word_embeddings is False
+
+
+def test_rope_theta_in_rope_parameters_layout():
+    cfg = qwen3.parse(raw(rope_theta=..., rope_parameters={"rope_type": "default", "rope_theta": 5e5}))
+    assert cfg.rope_theta == 5e5
+
+
+@pytest.mark.parametrize("over, match", [
+    (dict(rope_theta=...), "rope_theta"),
+    (dict(rope_scaling={"type": "linear", "factor": 2.0}), "scaling"),
+    (dict(rope_theta=..., rope_parameters={"rope_type": "yarn", "rope_theta": 1e6}), "yarn"),
+    (dict(num_attention_heads=6, num_key_value_heads=4), "divisible"),
+    (dict(architectures=["LlamaForCausalLM"]), "Unsupported architecture"),
+    (dict(attention_bias=True), "attention_bias"),
+    (dict(use_sliding_window=True), "sliding"),
+    (dict(hidden_act="gelu"), "hidden_act"),
+    (dict(head_dim=15), "even"),
+    (dict(vocab_size=...), "vocab_size"),
+])
+def test_bad_configs_raise(over, match):
+    with pytest.raises(ValueError, match=match):
+        qwen3.parse(raw(**over))
+
+
+def test_registry_rejects_unknown_names_and_lists_supported():
+    with pytest.raises(ValueError, match="Unsupported architecture 'NopeForCausalLM'; supported: .*Qwen3ForCausalLM"):
+        get_architecture("NopeForCausalLM")
+    assert "Qwen3ForCausalLM" in supported_architectures()
+    with pytest.raises(ValueError, match="unknown mixer part"):
+        get_part("mixer", "does_not_exist")
+    with pytest.raises(ValueError, match="already registered"):
+        register_architecture(Architecture("Qwen3ForCausalLM", qwen3.parse, qwen3.plan))
+
+
+def test_config_json_round_trip(tmp_path):
+    cfg = qwen3.parse(raw(), ())
+    (tmp_path / "config.json").write_text(json.dumps(qwen3.to_config_json(cfg)))
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": [3, 9]}))
+    arch, parsed, plan = load_model_description(tmp_path)
+    assert arch.name == "Qwen3ForCausalLM"
+    assert parsed == qwen3.parse(raw(), (3, 9))
+    assert plan.eos_token_ids == (3, 9)
+
+
+def test_eos_as_single_int(tmp_path):
+    cfg = qwen3.parse(raw(), ())
+    (tmp_path / "config.json").write_text(json.dumps(qwen3.to_config_json(cfg)))
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": 5}))
+    assert load_model_description(tmp_path)[2].eos_token_ids == (5,)
+
+
+def test_plan_carries_every_number_as_part_parameters():
+    cfg = qwen3.parse(raw(), ())
+    plan = qwen3.plan(cfg)
+    assert len(plan.layers) == 2 and [c.layer for c in plan.order] == [0, 1]
+    mixer = plan.layers[0].mixer
+    assert mixer.kind == "gqa_attention"
+    assert mixer["head_dim"] == 32 and mixer["num_kv_heads"] == 2
+    assert mixer["softmax_scale"] == 32 ** -0.5   # the configured head_dim, not hidden/heads
+    assert mixer["qk_norm_eps"] == 1e-6
+    kind, params = mixer["position"]
+    assert kind == "rotary_half" and dict(params) == {"rotary_dim": 32, "theta": 1e6}
+    assert plan.layers[0].feed_forward["intermediate_size"] == 128
+    assert plan.head["tied"] is True
+
+
+def test_run_order_is_validated_data():
+    spec = qwen3.plan(qwen3.parse(raw(), ()))
+    kw = dict(vocab_size=10, hidden_size=8, max_position_embeddings=16, tie_word_embeddings=False,
+              embedding=spec.embedding, layers=spec.layers, final_norm=spec.final_norm, head=spec.head)
+    ModelPlan(order=(LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2), LayerCall(1, 0, writes_cache=False)), **kw)
+    with pytest.raises(ValueError, match="names layer 5"):
+        ModelPlan(order=(LayerCall(5, 0),), **kw)
+    with pytest.raises(ValueError, match="never written"):
+        ModelPlan(order=(LayerCall(0, 0), LayerCall(1, 3, writes_cache=False)), **kw)
+
+
+def test_partspec_is_hashable_and_frozen():
+    a = PartSpec.of("x", b=2, a=[1, 2])
+    assert a == PartSpec.of("x", a=(1, 2), b=2) and hash(a) == hash(PartSpec.of("x", a=(1, 2), b=2))
+    assert a.as_dict() == {"a": (1, 2), "b": 2}

@@ -1,0 +1,131 @@
+"""Generation through the entry point: greedy equals the plain implementation,
+lengths and stop rules, seeded sampling, preemption is invisible."""
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from replay_util import random_ids
+from tiny import TINIES, make_folder
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("gen")
+    return {k: make_folder(root, k) for k in TINIES}
+
+
+@pytest.mark.parametrize("which, lengths, new", [("A", [5, 17, 33], 8), ("B", [1, 9, 40, 70], 12)])
+def test_greedy_generation_matches_plain(folders, which, lengths, new):
+    from tokamak_amd import LLM, SamplingParams
+
+    folder = folders[which]
+    cfg, w = plain.read_folder(folder)
+    prompts = [random_ids(cfg["vocab_size"], n, 40 + i) for i, n in enumerate(lengths)]
+    llm = LLM(folder, dtype="float32", block_size=TINIES[which]["page_size"], kv_pool_tokens=512,
+              max_batch_size=4, max_num_batched_tokens=32, prefill_chunk=16)
+    outs = llm.generate(prompt_token_ids=prompts,
+                        sampling_params=SamplingParams(temperature=0.0, max_new_tokens=new, ignore_eos=True))
+    assert [o.request_id for o in outs] == list(range(len(prompts)))
+    for o, p in zip(outs, prompts):
+        assert o.prompt_token_ids == p
+        assert o.output_token_ids == plain.greedy(p, new, cfg, w)
+        assert o.finish_reason.value == "length" and len(o.output_token_ids) == new
+        assert o.ttft_s is not None and o.latency_s >= o.ttft_s
+    llm.runner.manager.check()
+    assert llm.runner.manager.num_free_pages() == llm.runner.manager.num_pages()
+
+
+def test_bfloat16_greedy_runs_and_mostly_agrees(folders):
+    from tokamak_amd import LLM, SamplingParams
+
+    folder = folders["C"]
+    cfg, w = plain.read_folder(folder)
+    prompts = [random_ids(cfg["vocab_size"], n, 70 + i) for i, n in enumerate([12, 50])]
+    llm = LLM(folder, dtype="bfloat16", kv_pool_tokens=1024)
+    outs = llm.generate(prompt_token_ids=prompts, sampling_params=SamplingParams(temperature=0.0, max_new_tokens=4, ignore_eos=True))
+    for o, p in zip(outs, prompts):
+        # the first token is decided by logits within bf16 distance of the plain ones
+        logits = plain.logits(p, cfg, w)[-1]
+        top = float(logits.max())
+        assert float(logits[o.output_token_ids[0]]) > top - 0.05 * float(logits.abs().max())
+
+
+def test_stop_rules(folders, tmp_path):
+    from tokamak_amd import LLM, SamplingParams
+    import json, shutil
+
+    folder = tmp_path / "with_eos"
+    shutil.copytree(folders["A"], folder)
+    cfg, w = plain.read_folder(folder)
+    prompt = random_ids(cfg["vocab_size"], 9, 5)
+    free_run = plain.greedy(prompt, 6, cfg, w)
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": [free_run[2]]}))
+    llm = LLM(folder, dtype="float32", max_seq_len=64)
+    first_stop = free_run.index(free_run[2])
+    out = llm.generate(prompt_token_ids=[prompt], sampling_params=SamplingParams(temperature=0.0, max_new_tokens=6))[0]
+    assert out.finish_reason.value == "stop" and out.output_token_ids == free_run[:first_stop + 1]  # EOS included
+    out = llm.generate(prompt_token_ids=[prompt], sampling_params=SamplingParams(temperature=0.0, max_new_tokens=6, ignore_eos=True))[0]
+    assert out.finish_reason.value == "length" and out.output_token_ids == free_run
+    # the context limit ends a request too
+    long_prompt = random_ids(cfg["vocab_size"], 60, 6)
+    out = llm.generate(prompt_token_ids=[long_prompt], sampling_params=SamplingParams(temperature=0.0, max_new_tokens=50, ignore_eos=True))[0]
+    assert out.finish_reason.value == "length" and len(out.output_token_ids) == 4
+    with pytest.raises(ValueError, match="does not fit"):
+        llm.generate(prompt_token_ids=[random_ids(cfg["vocab_size"], 64, 7)])
+    with pytest.raises(ValueError, match="exactly one"):
+        llm.generate()
+    with pytest.raises(ValueError, match="SamplingParams for"):
+        llm.generate(prompt_token_ids=[prompt], sampling_params=[SamplingParams(), SamplingParams()])
+    with pytest.raises(ValueError, match="tokenizer"):
+        llm.generate("text without a tokenizer")
+
+
+def test_seeded_sampling_is_reproducible_and_independent_of_batching(folders):
+    from tokamak_amd import LLM, SamplingParams
+
+    folder = folders["B"]
+    cfg, _ = plain.read_folder(folder)
+    prompts = [random_ids(cfg["vocab_size"], n, 90 + i) for i, n in enumerate([1, 9, 40, 70])]
+    params = [SamplingParams(temperature=0.8, top_p=0.95, max_new_tokens=12, seed=100 + i, ignore_eos=True) for i in range(4)]
+    llm = LLM(folder, dtype="float32", block_size=8, kv_pool_tokens=512, max_batch_size=4,
+              max_num_batched_tokens=32, prefill_chunk=16)
+    a = llm.generate(prompt_token_ids=prompts, sampling_params=params)
+    b = llm.generate(prompt_token_ids=prompts, sampling_params=params)
+    assert [o.output_token_ids for o in a] == [o.output_token_ids for o in b]
+    alone = [llm.generate(prompt_token_ids=[p], sampling_params=q)[0] for p, q in zip(prompts, params)]
+    assert [o.output_token_ids for o in a] == [o.output_token_ids for o in alone]
+    other = llm.generate(prompt_token_ids=prompts, sampling_params=[
+        SamplingParams(temperature=0.8, top_p=0.95, max_new_tokens=12, seed=7 + i, ignore_eos=True) for i in range(4)])
+    assert [o.output_token_ids for o in a] != [o.output_token_ids for o in other]
+
+
+def test_preemption_is_invisible(folders):
+    """A pool of three pages for two requests (reference
+    tests/integration/test_generate_e2e.py:180-213): outputs equal a roomy run."""
+    from tokamak_amd import LLM, SamplingParams
+
+    folder = folders["A"]
+    cfg, _ = plain.read_folder(folder)
+    prompts = [random_ids(cfg["vocab_size"], n, 20 + i) for i, n in enumerate([14, 13])]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=20, ignore_eos=True),
+              SamplingParams(temperature=0.9, top_k=20, max_new_tokens=20, seed=3, ignore_eos=True)]
+    roomy = LLM(folder, dtype="float32", max_seq_len=48, kv_pool_tokens=256, max_batch_size=2)
+    tight = LLM(folder, dtype="float32", max_seq_len=48, kv_pool_tokens=48, max_batch_size=2)
+    want = roomy.generate(prompt_token_ids=prompts, sampling_params=params)
+    got = tight.generate(prompt_token_ids=prompts, sampling_params=params)
+    assert tight.num_preemptions > 0 and roomy.num_preemptions == 0
+    assert [o.output_token_ids for o in got] == [o.output_token_ids for o in want]
+    tight.runner.manager.check()
+    assert tight.runner.manager.num_free_pages() == 3
+
+
+def test_command_line(folders, capsys):
+    from tokamak_amd import cli
+
+    assert cli.main(["--model", str(folders["A"]), "--prompt-ids", "5,6,7", "--max-new-tokens", "5",
+                     "--temperature", "0", "--dtype", "float32"]) == 0
+    out = capsys.readouterr().out
+    assert "[completion (length)]" in out and "[prompt ids]" in out

@@ -1,0 +1,199 @@
+"""Pins of the plain implementation beside the reference's text: vectors the
+reference's own tests hold, special cases that reduce to a library routine, and
+invariants, each chosen so that a plausible mistake fails it."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_qwen3 as plain
+from tiny import TINIES, make_folder
+
+
+# -- RMSNorm (reference tests/unit/test_layers.py:11-27) ----------------------
+def test_rmsnorm_formula_and_unit_rms():
+    torch.manual_seed(0)
+    w = torch.randn(64)
+    x = torch.randn(2, 5, 64)
+    expected = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+    torch.testing.assert_close(plain.rmsnorm(x, w, 1e-6), expected, rtol=1e-5, atol=1e-6)
+    out = plain.rmsnorm(torch.randn(10, 128) * 3.0, torch.ones(128), 1e-8)
+    torch.testing.assert_close(out.pow(2).mean(-1).sqrt(), torch.ones(10), rtol=1e-3, atol=1e-3)
+    # scale invariance (eps -> 0): a norm that forgot the rsqrt, or used the mean, fails
+    torch.testing.assert_close(plain.rmsnorm(7.0 * x, w, 1e-12), plain.rmsnorm(x, w, 1e-12), rtol=1e-5, atol=1e-6)
+
+
+# -- RoPE (reference tests/unit/test_layers.py:30-68) -------------------------
+def test_rope_position_zero_is_identity_and_norm_is_kept():
+    cos, sin = plain.rope_tables(torch.tensor([0]), 32, 10000.0)
+    q = torch.randn(1, 4, 32)
+    torch.testing.assert_close(plain.apply_rope(q, cos, sin), q)
+    cos, sin = plain.rope_tables(torch.arange(10), 64, 1e6)
+    q = torch.randn(10, 4, 64)
+    torch.testing.assert_close(plain.apply_rope(q, cos, sin).norm(dim=-1), q.norm(dim=-1), rtol=1e-4, atol=1e-4)
+
+
+def test_rope_dot_depends_on_distance_only():
+    torch.manual_seed(3)
+    q, k = torch.randn(1, 1, 32), torch.randn(1, 1, 32)
+
+    def dot(m, n):
+        cq, sq = plain.rope_tables(torch.tensor([m]), 32, 10000.0)
+        ck, sk = plain.rope_tables(torch.tensor([n]), 32, 10000.0)
+        return float((plain.apply_rope(q, cq, sq) * plain.apply_rope(k, ck, sk)).sum())
+
+    assert abs(dot(5, 3) - dot(9, 7)) < 1e-4
+    assert abs(dot(10, 0) - dot(15, 5)) < 1e-4
+    assert abs(dot(5, 3) - dot(3, 5)) > 1e-3      # the sign of the distance matters
+
+
+def test_rope_pairs_halves_not_neighbours_and_turns_the_right_way():
+    hd, theta, pos = 8, 10000.0, 3
+    cos, sin = plain.rope_tables(torch.tensor([pos]), hd, theta)
+    x = torch.zeros(1, 1, hd)
+    x[0, 0, 1] = 1.0                                # unit vector on dim 1
+    out = plain.apply_rope(x, cos, sin)[0, 0]
+    angle = pos * theta ** (-2.0 / hd)              # frequency index 1
+    expected = torch.zeros(hd)
+    expected[1] = math.cos(angle)                   # stays on dim 1 ...
+    expected[1 + hd // 2] = math.sin(angle)         # ... and leaks into dim 1 + hd/2 with a plus sign
+    torch.testing.assert_close(out, expected, rtol=1e-5, atol=1e-6)
+
+
+# -- attention core ------------------------------------------------------------
+def test_attention_equals_library_sdpa_with_gqa():
+    torch.manual_seed(1)
+    T, nh, nkv, hd = 11, 6, 3, 16
+    q, k, v = torch.randn(T, nh, hd), torch.randn(T, nkv, hd), torch.randn(T, nkv, hd)
+    ours = plain.causal_gqa_attention(q, k, v, hd ** -0.5)
+    rep = nh // nkv
+    lib = F.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.transpose(0, 1).repeat_interleave(rep, 0)[None],
+        v.transpose(0, 1).repeat_interleave(rep, 0)[None], is_causal=True)[0].transpose(0, 1)
+    torch.testing.assert_close(ours, lib, rtol=1e-5, atol=1e-5)
+
+
+def test_attention_special_cases():
+    torch.manual_seed(2)
+    nh, nkv, hd = 4, 2, 8
+    q, k, v = torch.randn(1, nh, hd), torch.randn(1, nkv, hd), torch.randn(1, nkv, hd)
+    out = plain.causal_gqa_attention(q, k, v, hd ** -0.5)
+    # one token: softmax over one key is 1, the output is v of head a // G (not a % nkv)
+    torch.testing.assert_close(out[0, 0], v[0, 0])
+    torch.testing.assert_close(out[0, 1], v[0, 0])
+    torch.testing.assert_close(out[0, 2], v[0, 1])
+    torch.testing.assert_close(out[0, 3], v[0, 1])
+    # all keys equal: output is the mean of the visible values
+    T = 6
+    q, v = torch.randn(T, nh, hd), torch.randn(T, nkv, hd)
+    k = torch.randn(1, nkv, hd).expand(T, nkv, hd)
+    out = plain.causal_gqa_attention(q, k, v, hd ** -0.5)
+    for t in range(T):
+        torch.testing.assert_close(out[t, 3], v[: t + 1, 1].mean(0), rtol=1e-5, atol=1e-6)
+
+
+def test_attention_scale_is_applied_to_scores():
+    torch.manual_seed(4)
+    T, hd = 5, 8
+    q, k, v = torch.randn(T, 1, hd), torch.randn(T, 1, hd), torch.randn(T, 1, hd)
+    a = plain.causal_gqa_attention(q, k, v, 0.5)
+    b = plain.causal_gqa_attention(q * 0.5, k, v, 1.0)
+    torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-6)
+
+
+# -- SwiGLU (reference tests/unit/test_layers.py:71-79) -----------------------
+def test_swiglu_zero_gate_and_library_silu():
+    torch.manual_seed(5)
+    w = {"gate_proj.weight": torch.randn(32, 16), "up_proj.weight": torch.randn(32, 16),
+         "down_proj.weight": torch.randn(16, 32)}
+    x = torch.randn(3, 16)
+    lib = (F.silu(x @ w["gate_proj.weight"].T) * (x @ w["up_proj.weight"].T)) @ w["down_proj.weight"].T
+    torch.testing.assert_close(plain.swiglu(x, w, ""), lib, rtol=1e-5, atol=1e-5)
+    w["gate_proj.weight"] = torch.zeros(32, 16)
+    torch.testing.assert_close(plain.swiglu(x, w, ""), torch.zeros(3, 16))
+
+
+# -- whole model -----------------------------------------------------------------
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("plain")
+    return {k: plain.read_folder(make_folder(root, k)) for k in ("A", "B")}
+
+
+def test_layers_switched_off_leave_head_of_norm_of_embedding(folders):
+    cfg, w = folders["B"]
+    w = dict(w)
+    for i in range(cfg["num_hidden_layers"]):
+        w[f"model.layers.{i}.self_attn.o_proj.weight"] = torch.zeros_like(w[f"model.layers.{i}.self_attn.o_proj.weight"])
+        w[f"model.layers.{i}.mlp.down_proj.weight"] = torch.zeros_like(w[f"model.layers.{i}.mlp.down_proj.weight"])
+    ids = [3, 1, 4, 1, 5]
+    emb = w["model.embed_tokens.weight"][torch.tensor(ids)]
+    expected = plain.rmsnorm(emb, w["model.norm.weight"], cfg["rms_norm_eps"]) @ w["lm_head.weight"].T
+    torch.testing.assert_close(plain.logits(ids, cfg, w), expected, rtol=1e-5, atol=1e-6)
+
+
+def test_causality(folders):
+    cfg, w = folders["A"]
+    ids = [5, 9, 2, 7, 11, 3, 8]
+    base = plain.logits(ids, cfg, w)
+    changed = plain.logits(ids[:-1] + [200], cfg, w)
+    torch.testing.assert_close(base[:-1], changed[:-1], rtol=0, atol=0)
+    assert (base[-1] - changed[-1]).abs().max() > 1e-4
+
+
+def test_shift_of_all_positions_changes_nothing(folders):
+    # only distances count: a rotation with the wrong sign on k, or applied to v, fails this
+    for key in ("A", "B"):
+        cfg, w = folders[key]
+        ids = list(range(10, 22))
+        a = plain.logits(ids, cfg, w, start_position=0)
+        b = plain.logits(ids, cfg, w, start_position=37)
+        torch.testing.assert_close(a, b, rtol=1e-4, atol=2e-5)
+
+
+def test_tied_head_uses_the_embedding(folders):
+    cfg, w = folders["A"]
+    assert cfg["tie_word_embeddings"] and "lm_head.weight" not in w
+    h = plain.hidden_states([1, 2, 3], cfg, w)
+    torch.testing.assert_close(plain.logits([1, 2, 3], cfg, w), h @ w["model.embed_tokens.weight"].T)
+
+
+def test_qk_norm_comes_before_rotation_and_v_is_untouched(folders):
+    cfg, w = folders["B"]
+    s = plain.sizes(cfg)
+    torch.manual_seed(6)
+    h = torch.randn(4, s["H"])
+    p = "model.layers.0.self_attn."
+    w1 = dict(w)
+    w1[p + "q_norm.weight"] = torch.ones(s["hd"])
+    q = (h @ w1[p + "q_proj.weight"].T).view(4, s["nh"], s["hd"])
+    qn = plain.rmsnorm(q, w1[p + "q_norm.weight"], 0.0)
+    cos, sin = plain.rope_tables(torch.arange(4), s["hd"], s["theta"])
+    rotated = plain.apply_rope(qn, cos, sin)
+    torch.testing.assert_close(rotated.norm(dim=-1), torch.full((4, s["nh"]), math.sqrt(s["hd"])), rtol=1e-4, atol=1e-4)
+
+
+def test_float64_agrees_with_float32(folders):
+    cfg, w = folders["B"]
+    ids = list(range(1, 40))
+    w64 = {k: v.double() for k, v in w.items()}
+    torch.testing.assert_close(plain.logits(ids, cfg, w), plain.logits(ids, cfg, w64), rtol=0, atol=2e-5)
+
+
+# -- sampler vectors (reference tests/unit/test_sampler.py:12-56) ----------------
+def test_sampler_vectors():
+    p = plain.sampling_probs(torch.tensor([1.0, 2.0, 3.0, 4.0, 5.0]), 1.0, 2, 1.0)
+    assert set(torch.nonzero(p).flatten().tolist()) == {3, 4}
+    p = plain.sampling_probs(torch.tensor([0.5, 0.3, 0.2]).log(), 1.0, 0, 0.7)
+    assert set(torch.nonzero(p).flatten().tolist()) == {0, 1}
+    torch.testing.assert_close(p[:2], torch.tensor([0.625, 0.375], dtype=torch.float64), rtol=1e-6, atol=1e-6)
+    p = plain.sampling_probs(torch.tensor([0.9, 0.06, 0.04]).log(), 1.0, 0, 0.05)
+    assert torch.nonzero(p).flatten().tolist() == [0]
+    torch.manual_seed(0)
+    logits = torch.randn(100)
+    p = plain.sampling_probs(logits, 2.0, 1, 1.0)     # top_k = 1 is greedy at any temperature
+    assert int(p.argmax()) == int(logits.argmax()) and p.max() == 1.0
+    p = plain.sampling_probs(logits, 0.5, 0, 1.0)
+    torch.testing.assert_close(p, torch.softmax(logits.double() / 0.5, -1))

@@ -1,0 +1,73 @@
+"""Command line: generate from one prompt.
+
+    python -m tokamak_amd.cli --model DIR --prompt-ids 1,2,3 --max-new-tokens 16
+    python -m tokamak_amd.cli --random-weights tiny-a --prompt-ids 5,6,7 --temperature 0
+
+Options ``--model --prompt --max-new-tokens --temperature --top-p`` and their
+defaults are those of the reference's example (examples/basic_generation.py:14-20);
+the chat template is applied only when the folder has a tokenizer.
+"""
+
+from __future__ import annotations
+
+import argparse
+import sys
+import tempfile
+
+
+def main(argv: list[str] | None = None) -> int:
+    parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    parser.add_argument("--model", default=None, help="model folder (config.json + safetensors)")
+    parser.add_argument("--prompt", default="What does an LLM inference engine do?")
+    parser.add_argument("--prompt-ids", default=None, help="comma-separated token ids (no tokenizer needed)")
+    parser.add_argument("--max-new-tokens", type=int, default=256)
+    parser.add_argument("--temperature", type=float, default=0.7)
+    parser.add_argument("--top-p", type=float, default=0.95)
+    parser.add_argument("--top-k", type=int, default=0)
+    parser.add_argument("--seed", type=int, default=None)
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--page-size", type=int, default=16)
+    parser.add_argument("--max-seq-len", type=int, default=None)
+    parser.add_argument("--random-weights", default=None, metavar="PRESET",
+                        help="write a folder of seeded random weights of this shape and use it")
+    parser.add_argument("--weights-seed", type=int, default=0)
+    args = parser.parse_args(argv)
+
+    from tokamak_amd import LLM, SamplingParams
+
+    if (args.model is None) == (args.random_weights is None):
+        parser.error("give exactly one of --model and --random-weights")
+    tmp = None
+    folder = args.model
+    if args.random_weights is not None:
+        from tokamak_amd.models.qwen3 import PRESETS
+        from tokamak_amd.weights import write_random_model
+
+        if args.random_weights not in PRESETS:
+            parser.error(f"unknown preset {args.random_weights!r}; presets: {sorted(PRESETS)}")
+        tmp = tempfile.TemporaryDirectory(prefix="tokamak_amd_")
+        folder = write_random_model(tmp.name, PRESETS[args.random_weights], args.weights_seed)
+
+    llm = LLM(folder, dtype=args.dtype, block_size=args.page_size, max_seq_len=args.max_seq_len)
+    params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k,
+                            max_new_tokens=args.max_new_tokens, seed=args.seed)
+    if args.prompt_ids is not None:
+        ids = [int(t) for t in args.prompt_ids.split(",") if t.strip()]
+        outputs = llm.generate(prompt_token_ids=[ids], sampling_params=params)
+        print(f"\n[prompt ids]\n{ids}\n")
+    else:
+        if llm.tokenizer is None:
+            parser.error("the model folder has no tokenizer.json: use --prompt-ids")
+        text = f"<|im_start|>user\n{args.prompt}<|im_end|>\n<|im_start|>assistant\n<think>\n\n</think>\n\n"
+        outputs = llm.generate(text, params)
+        print(f"\n[prompt]\n{args.prompt}\n")
+    out = outputs[0]
+    print(f"[completion ({out.finish_reason.value})]")
+    print(out.output_text if out.output_text is not None else out.output_token_ids)
+    if tmp is not None:
+        tmp.cleanup()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

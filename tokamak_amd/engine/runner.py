@@ -76,8 +76,13 @@ class ModelRunner:
     def is_live(self, request) -> bool:
         return request in self._ctx_len
 
+    def forget(self, request) -> None:
+        """Drop the record of what the cache holds for ``request`` (its pages were
+        already given back by whoever preempted it)."""
+        self._ctx_len.pop(request, None)
+
     def end(self, request) -> None:
-        """The request is finished (or preempted): give back what it holds."""
+        """The request is finished: give back what it holds."""
         self._ctx_len.pop(request, None)
         self.manager.free(request)
 

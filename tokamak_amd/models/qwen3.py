@@ -175,4 +175,18 @@ def plan(cfg: Qwen3Config) -> ModelPlan:
     )
 
 
+def _shape(vocab, hidden, layers, heads, kv, hd, inter, theta, max_pos, tied, eps=1e-6) -> Qwen3Config:
+    return Qwen3Config(NAME, vocab, hidden, layers, heads, kv, hd, inter, eps, theta, max_pos, tied)
+
+
+# Shapes for the random-weights mode (sizes only; no trained weights exist here).
+PRESETS = {
+    "tiny-a": _shape(256, 64, 2, 4, 2, 16, 128, 10000.0, 128, True),
+    "tiny-b": _shape(384, 96, 3, 6, 3, 32, 200, 1000000.0, 256, False, eps=1e-5),
+    "qwen3-0.6b": _shape(151936, 1024, 28, 16, 8, 128, 3072, 1000000.0, 40960, True),
+    "qwen3-8b": _shape(151936, 4096, 36, 32, 8, 128, 12288, 1000000.0, 40960, False),
+    "qwen3-32b": _shape(151936, 5120, 64, 64, 8, 128, 25600, 1000000.0, 40960, False),
+}
+
+
 register_architecture(Architecture(name=NAME, parse=parse, plan=plan, to_json=to_config_json))

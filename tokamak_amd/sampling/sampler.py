@@ -1,0 +1,49 @@
+"""Choose next tokens from float32 logits on the GPU.
+
+Greedy rows take the first maximum (reference: src/tokamak/sampling/sampler.py:58-59).
+Other rows go through temperature -> top-k -> top-p -> softmax -> one draw
+(sampler.py:34-39,61).  The draw uses a counter-based generator keyed by the
+request's seed and the number of draws it has made, so a request's stream does
+not depend on what else is in the batch and survives preemption.  The
+reference draws with ``torch.multinomial``; the same distribution is sampled
+here, not the same stream.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from tokamak_amd.kernels import ops
+from tokamak_amd.sampling.params import SamplingParams
+
+
+def greedy_tokens(logits: torch.Tensor) -> torch.Tensor:
+    """int32 [M]: argmax of every row."""
+    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+    ops.argmax(logits, out)
+    return out
+
+
+def sample_tokens(logits: torch.Tensor, params: list[SamplingParams], seeds: list[int],
+                  draws: list[int], *, return_probs: bool = False):
+    """One token per row of ``logits`` [M, V].
+
+    ``seeds[i]`` and ``draws[i]``: row i's request seed and how many tokens it
+    has drawn before.  Returns int32 [M] (and the post-filter distributions
+    [M, V] when ``return_probs``; greedy rows have none and stay zero).
+    """
+    m = logits.shape[0]
+    if not (len(params) == len(seeds) == len(draws) == m):
+        raise ValueError("one SamplingParams, seed and draw count per logits row is required")
+    if all(p.is_greedy for p in params) and not return_probs:
+        return greedy_tokens(logits)
+    dev = logits.device
+    temperature = torch.tensor([p.temperature for p in params], dtype=torch.float32).to(dev)
+    top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32).to(dev)
+    top_p = torch.tensor([p.top_p for p in params], dtype=torch.float32).to(dev)
+    seed_t = torch.tensor([s & 0x7FFFFFFFFFFFFFFF for s in seeds], dtype=torch.int64).to(dev)
+    draw_t = torch.tensor(draws, dtype=torch.int64).to(dev)
+    out = torch.empty((m,), dtype=torch.int32, device=dev)
+    probs = torch.zeros_like(logits) if return_probs else None
+    ops.sample(logits, temperature, top_k, top_p, seed_t, draw_t, out, probs)
+    return (out, probs) if return_probs else out
