@@ -1,0 +1,54 @@
+"""Test-side helpers for kernel tests: page packing written independently of the
+kernels (from the documented layout), and float64 reference attention."""
+
+from __future__ import annotations
+
+import torch
+
+from tokamak_amd.engine.batch import StepSpan, build_batch
+
+
+def pack_pages(k_cache, v_cache, k_seq, v_seq, table, ps):
+    """Write a request's keys/values ([T, nkv, hd]) into its pages.
+    K page: [nkv][hd/8][ps][8]; V page: [nkv][hd][ps]."""
+    T, nkv, hd = k_seq.shape
+    for t in range(T):
+        page, off = table[t // ps], t % ps
+        kp = k_cache[page].view(nkv, hd // 8, ps, 8)
+        vp = v_cache[page].view(nkv, hd, ps)
+        kp[:, :, off, :] = k_seq[t].view(nkv, hd // 8, 8).to(k_cache.dtype)
+        vp[:, :, off] = v_seq[t].to(v_cache.dtype)
+
+
+def unpack_pages(k_cache, v_cache, table, T, nkv, hd, ps):
+    k = torch.empty(T, nkv, hd, dtype=k_cache.dtype)
+    v = torch.empty(T, nkv, hd, dtype=v_cache.dtype)
+    for t in range(T):
+        page, off = table[t // ps], t % ps
+        k[t] = k_cache[page].view(nkv, hd // 8, ps, 8)[:, :, off, :].reshape(nkv, hd).cpu()
+        v[t] = v_cache[page].view(nkv, hd, ps)[:, :, off].cpu()
+    return k, v
+
+
+def reference_attention(q, k, v, positions, scale, window=None):
+    """float64, explicit softmax.  q [Tq, nh, hd] at absolute ``positions``;
+    k, v [Tk, nkv, hd] (position = index).  Query head a uses kv head a // G."""
+    q, k, v = q.double(), k.double(), v.double()
+    Tq, nh, hd = q.shape
+    group = nh // k.shape[1]
+    out = torch.zeros(Tq, nh, hd, dtype=torch.float64)
+    for i, p in enumerate(positions):
+        lo = 0 if window is None else max(0, p - window + 1)
+        for a in range(nh):
+            kv = a // group
+            s = (k[lo:p + 1, kv] @ q[i, a]) * scale
+            w = torch.softmax(s, dim=0)
+            out[i, a] = w @ v[lo:p + 1, kv]
+    return out
+
+
+def make_batch(spans, device="cuda"):
+    """spans: list of (tokens_count, ctx_len, table) -> StepBatch with one cache group."""
+    ss = [StepSpan(request=i, tokens=[0] * n, ctx_len=ctx, state_slot=i, tables=[table])
+          for i, (n, ctx, table) in enumerate(spans)]
+    return build_batch(ss, 1, device)

@@ -1,0 +1,297 @@
+"""Each kernel alone against a plain float32/float64 reference, at sizes other
+than the engine's tiny models, with inputs made so that faults show."""
+
+import math
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from kernel_util import make_batch, pack_pages, reference_attention, unpack_pages
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=2e-2, atol=1e-2)}
+
+
+def rand(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+# ---------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------
+def run_attention(dtype, nh, nkv, hd, ps, requests, *, window=None, poison=True, force_generic=False,
+                  seed=0, boost=None):
+    """requests: list of (ctx_len, q_len).  Builds scattered tables, fills pages,
+    runs the dispatcher (or the generic kernel) and returns (got, want) lists."""
+    from tokamak_amd.kernels import ops
+    from tokamak_amd.kernels.attention import paged_attention
+
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum(-(-(c + q) // ps) for c, q in requests) + 5
+    order = torch.randperm(total_pages, generator=g).tolist()
+    fill = float("nan") if poison else 0.0
+    k_cache = torch.full((total_pages, nkv * hd * ps), fill, dtype=dtype)
+    v_cache = torch.full((total_pages, nkv * hd * ps), fill, dtype=dtype)
+    spans, seqs, qs = [], [], []
+    for ctx, qlen in requests:
+        T = ctx + qlen
+        npages = -(-T // ps)
+        table, order = order[:npages], order[npages:]
+        k = torch.randn(T, nkv, hd, generator=g).to(dtype)
+        v = torch.randn(T, nkv, hd, generator=g).to(dtype)
+        q = torch.randn(qlen, nh, hd, generator=g).to(dtype)
+        if boost is not None:
+            boost(q, k, v, ctx, qlen)
+        pack_pages(k_cache, v_cache, k, v, table, ps)
+        spans.append((qlen, ctx, table))
+        seqs.append((k, v))
+        qs.append(q)
+    batch = make_batch(spans)
+    q_all = torch.cat(qs).reshape(-1, nh * hd).to(DEV)
+    out = torch.full_like(q_all, float("nan"))
+    scale = hd ** -0.5
+    kc, vc = k_cache.to(DEV), v_cache.to(DEV)
+    if force_generic:
+        ops.paged_attention_generic(q_all, kc, vc, batch.block_tables[0], batch.positions, batch.req_of_token,
+                                    out, num_heads=nh, num_kv_heads=nkv, head_dim=hd, page_size=ps,
+                                    scale=scale, window=window)
+    else:
+        paged_attention(q_all, kc, vc, batch.block_tables[0], batch, out, num_heads=nh, num_kv_heads=nkv,
+                        head_dim=hd, page_size=ps, scale=scale, window=window)
+    out = out.cpu().float().reshape(-1, nh, hd)
+    got, want, at = [], [], 0
+    for (ctx, qlen), (k, v), q in zip(requests, seqs, qs):
+        got.append(out[at:at + qlen])
+        want.append(reference_attention(q.float(), k.float(), v.float(), range(ctx, ctx + qlen), scale, window).float())
+        at += qlen
+    return got, want
+
+
+SHAPES = [
+    (4, 2, 16, 8), (7, 1, 16, 16), (16, 8, 128, 16), (32, 8, 128, 16), (8, 2, 64, 32), (5, 5, 48, 16),
+    (6, 2, 256, 16), (24, 2, 64, 16), (3, 1, 128, 16), (14, 2, 128, 16),
+]
+MIXES = {
+    "decode": [(48, 1), (15, 1), (0, 1), (300, 1), (16, 1)],
+    "prefill": [(0, 33), (0, 1), (0, 16), (0, 70)],
+    "portions": [(17, 2), (30, 19), (64, 32), (5, 40)],
+    "mixed": [(100, 1), (0, 50), (31, 1), (47, 18), (16, 1)],
+}
+
+
+@pytest.mark.parametrize("mix", list(MIXES))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("nh, nkv, hd, ps", SHAPES)
+def test_attention_matches_reference(nh, nkv, hd, ps, dtype, mix):
+    got, want = run_attention(dtype, nh, nkv, hd, ps, MIXES[mix], seed=hd + nh)
+    for g, w in zip(got, want):
+        assert torch.isfinite(g).all(), "a page that the request does not own, or a slot past its end, was read"
+        torch.testing.assert_close(g, w, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_generic_kernel_at_mfma_shapes(dtype):
+    got, want = run_attention(dtype, 16, 4, 128, 16, MIXES["mixed"], force_generic=True)
+    for g, w in zip(got, want):
+        torch.testing.assert_close(g, w, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("hd", [64, 128, 80])
+def test_long_context_over_shuffled_pages(dtype, hd):
+    """4,089 tokens over 256 scattered pages (reference
+    tests/unit/test_paged_attention_kernel.py:108-124), decoded and as a portion."""
+    got, want = run_attention(dtype, 4, 2, hd, 16, [(4088, 1), (4000, 89)], seed=2)
+    for g, w in zip(got, want):
+        torch.testing.assert_close(g, w, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("far", [0, 3, 255, 256, 511, 777])
+def test_a_far_key_among_hundreds_is_found(dtype, far):
+    """One key (position ``far``) and the query are scaled so that its score
+    stands out: the output must be that key's value.  Random weights alone would
+    spread the softmax so thin that a skipped key could not be seen."""
+    hd = 128
+
+    def boost(q, k, v, ctx, qlen):
+        direction = torch.nn.functional.normalize(torch.randn(hd, generator=torch.Generator().manual_seed(9)), dim=0)
+        k[far, :, :] = (direction * 12.0).to(k.dtype)
+        q[-1, :, :] = (direction * 12.0).to(q.dtype)
+
+    got, want = run_attention(dtype, 8, 2, hd, 16, [(1023, 1), (1000, 24)], boost=boost, seed=4)
+    for g, w in zip(got, want):
+        torch.testing.assert_close(g, w, **TOL[dtype])
+        # and the reference itself says: the last query sees essentially one key
+        assert (w[-1] - w[-1]).abs().max() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_window_edge(dtype):
+    """Keys just inside and just outside a window of 24; the key right outside is
+    made enormous, so reading it would show."""
+    window = 24
+
+    def boost(q, k, v, ctx, qlen):
+        p = ctx + qlen - 1          # last query's position
+        outside = p - window        # first position it must not see
+        k[outside] = q[-1, :1].expand_as(k[outside]) * 30
+        v[outside] = 1000.0
+
+    for hd, nh, nkv in [(16, 4, 2), (128, 8, 2)]:
+        got, want = run_attention(dtype, nh, nkv, hd, 16, [(40, 1), (10, 30), (100, 7)], window=window, boost=boost, seed=5)
+        for g, w in zip(got, want):
+            torch.testing.assert_close(g, w, **TOL[dtype])
+            assert g[-1].abs().max() < 50
+
+
+def test_unsupported_sizes_are_refused_not_wrong():
+    from tokamak_amd.kernels import ops
+
+    q = torch.zeros(1, 4 * 12, device=DEV)
+    cache = torch.zeros(2, 2 * 12 * 16, device=DEV)
+    tables = torch.zeros(1, 4, dtype=torch.int32, device=DEV)
+    idx = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(ops.KernelError, match="multiple of 8"):
+        ops.paged_attention_generic(q, cache, cache, tables, idx, idx, q.clone(), num_heads=4, num_kv_heads=2,
+                                    head_dim=12, page_size=16, scale=1.0)
+    with pytest.raises(ops.KernelError, match="GPU"):
+        ops.silu_mul(torch.zeros(2, 8), torch.zeros(2, 4))
+
+
+# ---------------------------------------------------------------------------
+# per-head norm + rotation + cache write
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("nh, nkv, hd, ps, rot", [(4, 2, 16, 8, 16), (5, 1, 48, 16, 48), (8, 2, 128, 16, 128), (3, 3, 64, 32, 32)])
+def test_qknorm_rope_store(dtype, nh, nkv, hd, ps, rot):
+    from tokamak_amd.kernels import ops
+
+    eps, theta = 1e-5, 50000.0
+    spans = [(5, 11, [3, 0]), (1, 16, [6, 2]), (20, 0, [5, 1])]      # (tokens, ctx, table)
+    if ps == 8:
+        spans = [(5, 11, [3, 0]), (1, 16, [6, 2, 7]), (20, 0, [5, 1, 4])]
+    batch = make_batch(spans)
+    N = batch.num_tokens
+    qkv = rand(N, (nh + 2 * nkv) * hd, seed=1).to(dtype)
+    qw, kw = 1 + 0.3 * rand(hd, seed=2), 1 + 0.3 * rand(hd, seed=3)
+    positions = batch.positions.cpu()
+    inv_freq = 1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
+    cos = torch.empty(N, rot // 2, device=DEV)
+    sin = torch.empty(N, rot // 2, device=DEV)
+    ops.rope_tables(batch.positions, inv_freq.to(DEV), cos, sin)
+    want_cos, want_sin = plain.rope_tables(positions, rot, theta)
+    torch.testing.assert_close(cos.cpu(), want_cos[:, : rot // 2], rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(sin.cpu(), want_sin[:, : rot // 2], rtol=1e-5, atol=1e-6)
+
+    k_cache = torch.full((8, nkv * hd * ps), 7.0, dtype=dtype, device=DEV)
+    v_cache = torch.full((8, nkv * hd * ps), 7.0, dtype=dtype, device=DEV)
+    q_out = torch.empty(N, nh * hd, dtype=dtype, device=DEV)
+    ops.qknorm_rope_store(qkv.to(DEV), qw.to(DEV), kw.to(DEV), cos, sin, batch.positions, batch.req_of_token,
+                          batch.block_tables[0], q_out, k_cache, v_cache, num_heads=nh, num_kv_heads=nkv,
+                          head_dim=hd, rotary_dim=rot, page_size=ps, eps=eps)
+    x = qkv.float().view(N, nh + 2 * nkv, hd)
+    q, k, v = x[:, :nh], x[:, nh:nh + nkv], x[:, nh + nkv:]
+
+    def expect(t, w, rows=slice(None)):
+        t = plain.rmsnorm(t, w, eps)
+        rotated = plain.apply_rope(t[..., :rot], want_cos[rows], want_sin[rows])
+        return torch.cat([rotated, t[..., rot:]], dim=-1)
+
+    tol = TOL[dtype]
+    torch.testing.assert_close(q_out.cpu().float().view(N, nh, hd), expect(q, qw), **tol)
+    at = 0
+    for n, ctx, table in spans:
+        kk, vv = unpack_pages(k_cache.cpu(), v_cache.cpu(), table, ctx + n, nkv, hd, ps)
+        torch.testing.assert_close(kk[ctx:].float(), expect(k[at:at + n], kw, slice(at, at + n)), **tol)
+        torch.testing.assert_close(vv[ctx:].float(), v[at:at + n].to(dtype).float(), rtol=0, atol=0)  # v untouched
+        assert (kk[:ctx] == 7.0).all() and (vv[:ctx] == 7.0).all()   # earlier positions are not written
+        at += n
+
+
+# ---------------------------------------------------------------------------
+# norms, activation, embedding, matrix product
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("H", [64, 200, 4096, 5120 + 24])
+def test_add_rmsnorm(dtype, H):
+    from tokamak_amd.kernels import ops
+
+    M, eps = 7, 1e-5
+    resid, delta, w = rand(M, H, seed=1, scale=3.0), rand(M, H, seed=2).to(dtype), 1 + 0.2 * rand(H, seed=3)
+    r = resid.to(DEV)
+    out = torch.empty(M, H, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(r, delta.to(DEV), w.to(DEV), eps, out)
+    x = resid + delta.float()
+    torch.testing.assert_close(r.cpu(), x, rtol=0, atol=0)                      # the sum is float32 and stored
+    torch.testing.assert_close(out.cpu().float(), plain.rmsnorm(x, w, eps), **TOL[dtype])
+    # no delta; and row-indexed without touching the residual
+    out2 = torch.empty(M, H, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(r, None, w.to(DEV), eps, out2)
+    torch.testing.assert_close(out2.cpu().float(), plain.rmsnorm(x, w, eps), **TOL[dtype])
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    out3 = torch.empty(3, H, dtype=dtype, device=DEV)
+    before = r.clone()
+    ops.add_rmsnorm(r, delta.to(DEV), w.to(DEV), eps, out3, rows=rows, write_resid=False)
+    torch.testing.assert_close(out3.cpu().float(), plain.rmsnorm(x[[5, 0, 5]] + delta.float()[[5, 0, 5]], w, eps), **TOL[dtype])
+    assert torch.equal(r, before)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_silu_mul_and_embedding(dtype):
+    from tokamak_amd.kernels import ops
+
+    N, I = 5, 200
+    gu = rand(N, 2 * I, seed=1, scale=4.0).to(dtype)
+    out = torch.empty(N, I, dtype=dtype, device=DEV)
+    ops.silu_mul(gu.to(DEV), out)
+    g, u = gu.float()[:, :I], gu.float()[:, I:]
+    torch.testing.assert_close(out.cpu().float(), plain.silu(g) * u, **TOL[dtype])
+
+    table = rand(331, 120, seed=2).to(dtype)
+    ids = torch.tensor([0, 330, 17, 17, 5], dtype=torch.int32)
+    resid = torch.empty(5, 120, device=DEV)
+    ops.embed_gather(table.to(DEV), ids.to(DEV), resid)
+    torch.testing.assert_close(resid.cpu(), table.float()[ids.long()], rtol=0, atol=0)
+    bad = torch.tensor([331, -1], dtype=torch.int32, device=DEV)
+    resid2 = torch.zeros(2, 120, device=DEV)
+    ops.embed_gather(table.to(DEV), bad, resid2)
+    assert torch.isnan(resid2).all()        # an id outside the table never reads memory
+
+
+@pytest.mark.parametrize("M, N, K", [(1, 64, 64), (5, 200, 96), (70, 331, 120), (3, 1000, 4096), (129, 65, 17)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_linear(dtype, M, N, K):
+    from tokamak_amd.kernels.linear import linear
+
+    x, w = rand(M, K, seed=1).to(dtype), rand(N, K, seed=2, scale=K ** -0.5).to(dtype)
+    want = x.double() @ w.double().T
+    for out_dtype in (dtype, torch.float32):
+        got = linear(x.to(DEV), w.to(DEV), out_dtype=out_dtype).cpu()
+        assert got.dtype == out_dtype
+        tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else (
+            dict(rtol=2e-2, atol=1e-2) if out_dtype == torch.bfloat16 else dict(rtol=1e-3, atol=1e-3))
+        torch.testing.assert_close(got.double(), want, **tol)
+
+
+def test_float32_product_is_true_32_bit_and_row_independent():
+    """Values that a reduced-precision matrix mode would round away survive, and
+    a row's result does not depend on which rows are beside it."""
+    from tokamak_amd.kernels.linear import linear
+
+    K = 512
+    x = torch.ones(4, K)
+    x[:, 0] = 1.0 + 2.0 ** -20                 # lost in bf16, tf32 and fp16 inputs
+    w = torch.zeros(3, K)
+    w[:, 0] = 1.0
+    w[1, 1] = -1.0 + 2.0 ** -18
+    got = linear(x.to(DEV), w.to(DEV)).cpu()
+    assert got[0, 0].item() == 1.0 + 2.0 ** -20
+    assert got[0, 1].item() == pytest.approx(2.0 ** -20 + 2.0 ** -18, rel=1e-6)
+    big = rand(100, 300, seed=5)
+    wt = rand(77, 300, seed=6)
+    whole = linear(big.to(DEV), wt.to(DEV)).cpu()
+    one = linear(big[41:42].to(DEV), wt.to(DEV)).cpu()
+    assert torch.equal(whole[41:42], one)

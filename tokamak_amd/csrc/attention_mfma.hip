@@ -1,0 +1,309 @@
+// Paged causal attention on the matrix cores (bf16 in, float32 softmax and
+// accumulation) for head sizes 64 and 128 and page sizes that are multiples of 16.
+//
+// One 64-lane wave owns a work item: up to 16 "columns" per column set that share
+// one kv head and one request, and a range of that request's keys (a split).
+//   heads mode  (decode):  the columns of set s are query heads s*16 .. s*16+15 of
+//                          the group, all of one token;
+//   tokens mode (prefill): the columns are 16 consecutive tokens of one request,
+//                          set s is query head s of the group.
+// Keys are taken 16 at a time (one MFMA tile, never across a page edge):
+//   S^T[key][col] = K[key][:] . Q[col][:]      v_mfma_f32_16x16x32_bf16, K rows as A
+//   P^T = exp2(S^T * c - m[col])               float32, one column per lane
+//   O^T[d][col] += V^T[d][key] * P^T[key][col] v_mfma_f32_16x16x16_bf16, V^T rows as A
+// The result layout of the first product is exactly the B operand layout of the
+// second, so probabilities never leave registers, and both K and V^T operands
+// are loaded straight from the pages (K page [nkv][hd/8][ps][8], V page
+// [nkv][hd][ps]) in contiguous 16- and 8-byte pieces: no LDS is used.
+//
+// With more than one split the wave writes an unnormalised partial (o, m, l) and
+// a second kernel merges the splits of each (token, head).
+#include "common.h"
+
+using namespace tk;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+union Frag8 {
+  uint4 u;
+  bf16x8 v;
+};
+union Frag4 {
+  uint2 u;
+  short4v v;
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+template <int HD, int NSETS, bool TOKENS>
+__global__ __launch_bounds__(64) void attention_mfma_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
+    const int* __restrict__ positions, const int* __restrict__ req_of_token,
+    const int* __restrict__ item_token, const int* __restrict__ item_count,
+    bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int nsplit,
+    int split_keys, int nh, int nkv, int ps, float scale_log2) {
+  constexpr int KCH = HD / 32;  // 32-wide chunks of the head dim (QK^T steps)
+  constexpr int DBL = HD / 16;  // 16-wide blocks of the head dim (PV outputs)
+  const int lane = threadIdx.x, col = lane & 15, kb = lane >> 4;
+  const int split = blockIdx.x, item = blockIdx.z;
+  const int G = nh / nkv;
+  const int sets_per_group = TOKENS ? G / NSETS : 1;
+  const int kvh = blockIdx.y / sets_per_group;
+  const int set0 = (blockIdx.y % sets_per_group) * NSETS;  // first head of the group (tokens mode)
+
+  const int n0 = item_token[item];
+  const int count = TOKENS ? item_count[item] : 1;
+  const int pos0 = positions[n0];
+  const int last_pos = pos0 + count - 1;
+  const int k_begin = split * split_keys;
+  const int k_end = min(last_pos + 1, k_begin + split_keys);
+  if (k_begin >= k_end) return;
+  const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
+  const size_t page_elems = (size_t)nkv * HD * ps;
+  const size_t head_off = (size_t)kvh * HD * ps;
+
+  // which (token, head) this lane's column is, per set
+  int c_token[NSETS], c_head[NSETS];
+  bool c_valid[NSETS];
+  const int c_pos = TOKENS ? pos0 + col : pos0;
+#pragma unroll
+  for (int s = 0; s < NSETS; ++s) {
+    if (TOKENS) {
+      c_token[s] = n0 + col;
+      c_head[s] = kvh * G + set0 + s;
+      c_valid[s] = col < count;
+    } else {
+      c_token[s] = n0;
+      c_head[s] = kvh * G + s * 16 + col;
+      c_valid[s] = s * 16 + col < G;
+    }
+  }
+
+  // Q as B operand: lane (col, kb) holds Q[col][c*32 + kb*8 .. +8]
+  bf16x8 qreg[NSETS][KCH];
+#pragma unroll
+  for (int s = 0; s < NSETS; ++s) {
+    const bf16_t* qp = q + ((size_t)c_token[s] * nh + c_head[s]) * HD + kb * 8;
+#pragma unroll
+    for (int c = 0; c < KCH; ++c) {
+      Frag8 f;
+      f.u = c_valid[s] ? *reinterpret_cast<const uint4*>(qp + c * 32) : make_uint4(0, 0, 0, 0);
+      qreg[s][c] = f.v;
+    }
+  }
+
+  float m_run[NSETS], l_run[NSETS];
+  float4v acc[NSETS][DBL];
+#pragma unroll
+  for (int s = 0; s < NSETS; ++s) {
+    m_run[s] = -INFINITY;
+    l_run[s] = 0.f;
+#pragma unroll
+    for (int d = 0; d < DBL; ++d) acc[s][d] = float4v{0.f, 0.f, 0.f, 0.f};
+  }
+
+  Frag8 kreg[KCH];
+  Frag4 vreg[DBL];
+  auto load_tile = [&](int c0) {
+    const int page = table[c0 / ps];
+    const int off = c0 % ps;
+    const bf16_t* kp = k_cache + (size_t)page * page_elems + head_off + (size_t)(off + col) * 8;
+#pragma unroll
+    for (int c = 0; c < KCH; ++c)
+      kreg[c].u = *reinterpret_cast<const uint4*>(kp + (size_t)(c * 4 + kb) * ps * 8);
+    const bf16_t* vp = v_cache + (size_t)page * page_elems + head_off + (size_t)col * ps + off + kb * 4;
+#pragma unroll
+    for (int d = 0; d < DBL; ++d)
+      vreg[d].u = *reinterpret_cast<const uint2*>(vp + (size_t)d * 16 * ps);
+  };
+
+  load_tile(k_begin);
+  for (int c0 = k_begin; c0 < k_end; c0 += 16) {
+    Frag8 kc[KCH];
+    Frag4 vc[DBL];
+#pragma unroll
+    for (int c = 0; c < KCH; ++c) kc[c] = kreg[c];
+#pragma unroll
+    for (int d = 0; d < DBL; ++d) vc[d] = vreg[d];
+    if (c0 + 16 < k_end) load_tile(c0 + 16);  // next tile's loads fly while this one computes
+
+    const bool edge = c0 + 15 > pos0;  // some key of this tile is hidden from some column
+    if (c0 + 15 > last_pos) {
+      // keys past the request's end may hold anything (NaN included): zero their values
+#pragma unroll
+      for (int d = 0; d < DBL; ++d) {
+        short4v t = vc[d].v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (c0 + kb * 4 + i > last_pos) t[i] = 0;
+        vc[d].v = t;
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < NSETS; ++s) {
+      float4v sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < KCH; ++c)
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc[c].v, qreg[s][c], sc, 0, 0, 0);
+      float sv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        sv[i] = sc[i] * scale_log2;
+        if (edge) {
+          const int key = c0 + kb * 4 + i;
+          if (key > c_pos || key > last_pos) sv[i] = -INFINITY;
+        }
+      }
+      float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+      const float m_new = fmaxf(m_run[s], tmax);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run[s] - m_safe);
+      m_run[s] = m_new;
+      float p[4];
+      float psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[i] = fast_exp2(sv[i] - m_safe);
+        psum += p[i];
+      }
+      l_run[s] = l_run[s] * alpha + psum;
+      Frag4 pb;
+      pb.v = short4v{(short)float_to_bf16(p[0]), (short)float_to_bf16(p[1]),
+                     (short)float_to_bf16(p[2]), (short)float_to_bf16(p[3])};
+#pragma unroll
+      for (int d = 0; d < DBL; ++d) {
+        float4v a = acc[s][d];
+        a[0] *= alpha;
+        a[1] *= alpha;
+        a[2] *= alpha;
+        a[3] *= alpha;
+        acc[s][d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vc[d].v, pb.v, a, 0, 0, 0);
+      }
+    }
+  }
+
+  // acc[s][d][i] = O^T[dim = d*16 + kb*4 + i][col]
+#pragma unroll
+  for (int s = 0; s < NSETS; ++s) {
+    float l = l_run[s];
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if (!c_valid[s]) continue;
+    const size_t row = (size_t)c_token[s] * nh + c_head[s];
+    const size_t prow = (size_t)item * nh + c_head[s];  // partials are indexed by item, not token
+    if (nsplit == 1) {
+      const float inv = 1.f / l;
+      bf16_t* op = out + row * HD + kb * 4;
+#pragma unroll
+      for (int d = 0; d < DBL; ++d) {
+        Frag4 o;
+        o.v = short4v{(short)float_to_bf16(acc[s][d][0] * inv), (short)float_to_bf16(acc[s][d][1] * inv),
+                      (short)float_to_bf16(acc[s][d][2] * inv), (short)float_to_bf16(acc[s][d][3] * inv)};
+        *reinterpret_cast<uint2*>(op + d * 16) = o.u;
+      }
+    } else {
+      float* po = part_o + (prow * nsplit + split) * HD + kb * 4;
+#pragma unroll
+      for (int d = 0; d < DBL; ++d)
+        *reinterpret_cast<float4*>(po + d * 16) =
+            make_float4(acc[s][d][0], acc[s][d][1], acc[s][d][2], acc[s][d][3]);
+      if (kb == 0) {
+        part_ml[(prow * nsplit + split) * 2] = m_run[s];
+        part_ml[(prow * nsplit + split) * 2 + 1] = l;
+      }
+    }
+  }
+}
+
+// Merge the splits of every (token, head): out = sum_s w_s o_s / sum_s w_s l_s,
+// w_s = exp2(m_s - max m).  Splits that hold no key of the token are skipped by
+// the token's position, so they need not have been written.
+template <int HD>
+__global__ __launch_bounds__(64) void attention_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    const int* __restrict__ positions, const int* __restrict__ tokens, bf16_t* __restrict__ out,
+    int nsplit, int split_keys, int nh) {
+  const int n = tokens[blockIdx.x], head = blockIdx.y, lane = threadIdx.x;
+  const size_t row = (size_t)blockIdx.x * nh + head;  // partial row (by item)
+  const size_t orow = (size_t)n * nh + head;          // output row (by token)
+  const int used = min(nsplit, positions[n] / split_keys + 1);
+  float mx = -INFINITY;
+  for (int s = 0; s < used; ++s) mx = fmaxf(mx, part_ml[(row * nsplit + s) * 2]);
+  float denom = 0.f;
+  float o[HD / 64];
+#pragma unroll
+  for (int i = 0; i < HD / 64; ++i) o[i] = 0.f;
+  for (int s = 0; s < used; ++s) {
+    const float w = fast_exp2(part_ml[(row * nsplit + s) * 2] - mx);
+    denom += w * part_ml[(row * nsplit + s) * 2 + 1];
+    const float* po = part_o + (row * nsplit + s) * HD;
+#pragma unroll
+    for (int i = 0; i < HD / 64; ++i) o[i] += w * po[lane + i * 64];
+  }
+  const float inv = 1.f / denom;
+#pragma unroll
+  for (int i = 0; i < HD / 64; ++i) out[orow * HD + lane + i * 64] = float_to_bf16(o[i] * inv);
+}
+
+template <int HD, int NSETS, bool TOKENS>
+static int launch(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
+                  int max_pages, const int* positions, const int* req_of_token,
+                  const int* item_token, const int* item_count, int num_items, void* out,
+                  float* part_o, float* part_ml, int nsplit, int split_keys, int nh, int nkv, int ps,
+                  float scale, hipStream_t stream) {
+  const int G = nh / nkv;
+  dim3 grid(nsplit, TOKENS ? nkv * (G / NSETS) : nkv, num_items);
+  attention_mfma_kernel<HD, NSETS, TOKENS><<<grid, 64, 0, stream>>>(
+      (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
+      positions, req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit,
+      split_keys, nh, nkv, ps, scale * 1.4426950408889634f);
+  if (nsplit > 1) {
+    dim3 mgrid(num_items, nh);
+    attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token,
+                                                         (bf16_t*)out, nsplit, split_keys, nh);
+  }
+  return launch_status();
+}
+
+// mode 0: heads (every item is one decode token; item_count is ignored)
+// mode 1: tokens (item = up to 16 consecutive tokens of one request; nsplit must be 1)
+// Returns -2 if this shape is not instantiated (the caller uses the generic kernel).
+TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const void* v_cache,
+                             const int* block_tables, int max_pages, const int* positions,
+                             const int* req_of_token, const int* item_token, const int* item_count,
+                             int num_items, void* out, float* part_o, float* part_ml, int nsplit,
+                             int split_keys, int nh, int nkv, int hd, int ps, float scale,
+                             hipStream_t stream) {
+  if (num_items <= 0) return 0;
+  if (nkv <= 0 || nh % nkv != 0 || ps % 16 != 0 || split_keys % 16 != 0 || nsplit < 1) return -1;
+  if (num_items > 65535 || nh > 65535) return -1;
+  const int G = nh / nkv;
+#define TK_ARGS                                                                                   \
+  q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
+      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream
+  if (mode == 0) {
+    if (G > 16) return -2;
+    if (hd == 128) return launch<128, 1, false>(TK_ARGS);
+    if (hd == 64) return launch<64, 1, false>(TK_ARGS);
+    return -2;
+  }
+  if (nsplit != 1) return -1;
+  const int nsets = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
+  if (hd == 128) {
+    if (nsets == 4) return launch<128, 4, true>(TK_ARGS);
+    if (nsets == 2) return launch<128, 2, true>(TK_ARGS);
+    return launch<128, 1, true>(TK_ARGS);
+  }
+  if (hd == 64) {
+    if (nsets == 4) return launch<64, 4, true>(TK_ARGS);
+    if (nsets == 2) return launch<64, 2, true>(TK_ARGS);
+    return launch<64, 1, true>(TK_ARGS);
+  }
+#undef TK_ARGS
+  return -2;
+}

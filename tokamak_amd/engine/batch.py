@@ -41,12 +41,24 @@ class StepBatch:
     state_slots: torch.Tensor    # [R] int32
     logit_rows: torch.Tensor     # [M] int32, token rows whose logits are wanted
     block_tables: list[torch.Tensor]  # per cache group [R, max_pages] int32
+    # work lists for the attention kernels: single (decode) tokens, and tiles of up to
+    # 16 consecutive tokens of the longer spans
+    decode_tokens: torch.Tensor | None = None   # [num_decode] int32 token rows
+    tile_first: torch.Tensor | None = None      # [num_tiles] int32 first token row
+    tile_count: torch.Tensor | None = None      # [num_tiles] int32 tokens in the tile
+    num_decode: int = 0
+    num_tiles: int = 0
+    max_decode_len: int = 0                     # longest context among the decode tokens
     # host copies, for choosing kernels and grids
     q_lens: list[int] = field(default_factory=list)
     ctx_lens: list[int] = field(default_factory=list)
     max_q_len: int = 0
     max_seq_len: int = 0
     memo: dict = field(default_factory=dict)  # per-step data shared between layers
+
+
+TILE_TOKENS = 16   # tokens per attention tile of a prompt portion
+NUM_FIXED = 10     # arrays in the packed buffer before the block tables
 
 
 def build_batch(spans: list[StepSpan], num_groups: int, device) -> StepBatch:
@@ -58,11 +70,26 @@ def build_batch(spans: list[StepSpan], num_groups: int, device) -> StepBatch:
         w = max((len(s.tables[g]) for s in spans), default=0)
         widths.append(max(4, -(-w // 4) * 4))
     m = sum(len(s.want) for s in spans)
-    sizes = [n, n, n, r + 1, r, r, m] + [r * w for w in widths]
+    decode_rows, tiles = [], []
+    at = 0
+    for s in spans:
+        q = len(s.tokens)
+        if q == 1:
+            decode_rows.append(at)
+        else:
+            tiles.extend((at + t, min(TILE_TOKENS, q - t)) for t in range(0, q, TILE_TOKENS))
+        at += q
+    nd, nt = len(decode_rows), len(tiles)
+    sizes = [n, n, n, r + 1, r, r, m, nd, nt, nt] + [r * w for w in widths]
     offsets = np.concatenate([[0], np.cumsum(sizes)])
     buf = np.zeros(int(offsets[-1]), dtype=np.int32)
-    tok, pos, req, qs, ctx, slots, rows = (buf[offsets[i]:offsets[i + 1]] for i in range(7))
-    tabs = [buf[offsets[7 + g]:offsets[8 + g]].reshape(r, widths[g]) for g in range(num_groups)]
+    tok, pos, req, qs, ctx, slots, rows, dec, tfirst, tcount = (
+        buf[offsets[i]:offsets[i + 1]] for i in range(NUM_FIXED))
+    tabs = [buf[offsets[NUM_FIXED + g]:offsets[NUM_FIXED + 1 + g]].reshape(r, widths[g])
+            for g in range(num_groups)]
+    dec[:] = decode_rows
+    tfirst[:] = [t[0] for t in tiles]
+    tcount[:] = [t[1] for t in tiles]
     at = 0
     mi = 0
     for i, s in enumerate(spans):
@@ -89,12 +116,14 @@ def build_batch(spans: list[StepSpan], num_groups: int, device) -> StepBatch:
         dev = host.pin_memory().to(device, non_blocking=True)
     else:
         dev = host.to(device)
-    parts = [dev[int(offsets[i]):int(offsets[i + 1])] for i in range(7 + num_groups)]
+    parts = [dev[int(offsets[i]):int(offsets[i + 1])] for i in range(NUM_FIXED + num_groups)]
     return StepBatch(
         num_tokens=n, num_requests=r, num_logit_rows=m,
         token_ids=parts[0], positions=parts[1], req_of_token=parts[2], q_start=parts[3],
         ctx_len=parts[4], state_slots=parts[5], logit_rows=parts[6],
-        block_tables=[parts[7 + g].view(r, widths[g]) for g in range(num_groups)],
+        block_tables=[parts[NUM_FIXED + g].view(r, widths[g]) for g in range(num_groups)],
+        decode_tokens=parts[7], tile_first=parts[8], tile_count=parts[9], num_decode=nd, num_tiles=nt,
+        max_decode_len=max((s.ctx_len + 1 for s in spans if len(s.tokens) == 1), default=0),
         q_lens=[len(s.tokens) for s in spans], ctx_lens=[s.ctx_len for s in spans],
         max_q_len=max((len(s.tokens) for s in spans), default=0),
         max_seq_len=max((s.ctx_len + len(s.tokens) for s in spans), default=0),

@@ -75,6 +75,11 @@ _SIGS = {
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                        c_float, c_int, c_void_p],
     },
+    "attention_mfma": {
+        "tk_attention_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                              c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                              c_int, c_int, c_int, c_int, c_float, c_void_p],
+    },
     "sampling": {
         "tk_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
         "tk_sample": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -221,6 +226,46 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         _code(q.dtype), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(positions),
         _p(req_of_token), _p(out), n, num_heads, num_kv_heads, head_dim, page_size,
         block_tables.shape[1], float(scale), int(window or 0), _stream()), "paged_attention_generic")
+
+
+NOT_INSTANTIATED = -2
+
+
+def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   block_tables: torch.Tensor, positions: torch.Tensor, req_of_token: torch.Tensor,
+                   item_token: torch.Tensor, item_count: torch.Tensor | None, num_items: int,
+                   out: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int,
+                   page_size: int, scale: float, split_keys: int = 256, num_splits: int = 1) -> bool:
+    """bf16 attention on the matrix cores.  ``mode`` "heads": every item is one
+    decode token; "tokens": every item is up to 16 consecutive tokens of one
+    request.  Returns False (nothing launched) if the shape is not instantiated."""
+    _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, item_token, item_count, out)
+    n = positions.numel()
+    _need(q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
+          and out.dtype == torch.bfloat16, "the MFMA attention kernel takes bfloat16")
+    _need(q.numel() >= n * num_heads * head_dim and out.numel() >= n * num_heads * head_dim, "q/out too small")
+    _need(num_heads % num_kv_heads == 0 and page_size % 16 == 0 and split_keys % 16 == 0, "bad head counts, page size or split")
+    page_elems = num_kv_heads * head_dim * page_size
+    _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
+    _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32 and block_tables.dtype == torch.int32
+          and item_token.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
+    _need(item_token.numel() >= num_items and 0 < num_items <= 65535, "bad item list")
+    if mode == "tokens":
+        _need(item_count is not None and item_count.dtype == torch.int32 and item_count.numel() >= num_items
+              and num_splits == 1, "tokens mode needs item counts and one split")
+    part_o = part_ml = None
+    if num_splits > 1:
+        part_o = torch.empty((num_items * num_heads * num_splits, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((num_items * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
+    status = _fn("attention_mfma", "tk_attention_mfma")(
+        0 if mode == "heads" else 1, _p(q), _p(k_cache), _p(v_cache), _p(block_tables),
+        block_tables.shape[1], _p(positions), _p(req_of_token), _p(item_token), _p(item_count),
+        num_items, _p(out), _p(part_o), _p(part_ml), num_splits, split_keys, num_heads, num_kv_heads,
+        head_dim, page_size, float(scale), _stream())
+    if status == NOT_INSTANTIATED:
+        return False
+    _check(status, "attention_mfma")
+    return True
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
