@@ -129,3 +129,44 @@ def test_command_line(folders, capsys):
                      "--temperature", "0", "--dtype", "float32"]) == 0
     out = capsys.readouterr().out
     assert "[completion (length)]" in out and "[prompt ids]" in out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_equal_eager_ones_on_every_replay(folders, dtype):
+    """The same decode steps through replayed HIP graphs and eagerly, with the
+    program's own eager work (prefill of other requests) and synchronisations
+    between the replays; every replay is checked."""
+    from tokamak_amd.engine.runner import ModelRunner, StepEntry
+
+    folder = folders["C"]
+    cfg, _ = plain.read_folder(folder)
+    kw = dict(dtype=dtype, page_size=16, kv_pool_tokens=2048, max_requests=8)
+    graphed = ModelRunner.from_folder(folder, use_graphs=True, **kw)
+    eager = ModelRunner.from_folder(folder, use_graphs=False, **kw)
+    prompts = {r: random_ids(cfg["vocab_size"], n, 300 + r) for r, n in enumerate([30, 7, 250])}
+    last = {}
+    for r, p in prompts.items():
+        a = graphed.step([StepEntry(r, p, [len(p) - 1])])
+        b = eager.step([StepEntry(r, p, [len(p) - 1])])
+        assert torch.equal(a, b)
+        last[r] = int(a.argmax())
+    for i in range(40):
+        if i == 7:      # a newcomer's prefill between replays, and a request that ends
+            p = random_ids(cfg["vocab_size"], 19, 999)
+            a = graphed.step([StepEntry(9, p, [18])])
+            b = eager.step([StepEntry(9, p, [18])])
+            assert torch.equal(a, b)
+            last[9] = int(a.argmax())
+        if i == 20:
+            graphed.end(1)
+            eager.end(1)
+            del last[1]
+        entries = [StepEntry(r, [t], [0]) for r, t in last.items()]
+        a = graphed.step(entries).clone()
+        torch.cuda.synchronize()
+        b = eager.step(entries)
+        assert torch.equal(a, b), f"replay {i} differs from the eager step"
+        for row, r in enumerate(list(last)):
+            last[r] = int(a[row].argmax())
+    assert sum(g.replays for g in graphed._graphs.values()) == 40
+    assert len(graphed._graphs) >= 2     # batch sizes 3, 4 and 3 again; lengths crossing 256

@@ -61,14 +61,38 @@ TILE_TOKENS = 16   # tokens per attention tile of a prompt portion
 NUM_FIXED = 10     # arrays in the packed buffer before the block tables
 
 
-def build_batch(spans: list[StepSpan], num_groups: int, device) -> StepBatch:
-    """Pack the descriptor into one host buffer and copy it to the device once."""
+@dataclass
+class PackedBatch:
+    """The descriptor packed into one host int32 buffer, plus what is needed to
+    cut the device copy of that buffer back into arrays."""
+
+    buf: np.ndarray
+    offsets: list[int]
+    widths: list[int]
+    num_tokens: int
+    num_requests: int
+    num_logit_rows: int
+    num_decode: int
+    num_tiles: int
+    q_lens: list[int]
+    ctx_lens: list[int]
+    max_decode_len: int
+
+
+def table_width(longest: int, fixed: int | None = None) -> int:
+    if fixed is not None:
+        if longest > fixed:
+            raise ValueError(f"a block table of {longest} pages does not fit the fixed width {fixed}")
+        return fixed
+    return max(4, -(-longest // 4) * 4)
+
+
+def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] | None = None) -> PackedBatch:
     r = len(spans)
     n = sum(len(s.tokens) for s in spans)
-    widths = []
-    for g in range(num_groups):
-        w = max((len(s.tables[g]) for s in spans), default=0)
-        widths.append(max(4, -(-w // 4) * 4))
+    widths = [table_width(max((len(s.tables[g]) for s in spans), default=0),
+                          None if fixed_widths is None else fixed_widths[g])
+              for g in range(num_groups)]
     m = sum(len(s.want) for s in spans)
     decode_rows, tiles = [], []
     at = 0
@@ -81,8 +105,10 @@ def build_batch(spans: list[StepSpan], num_groups: int, device) -> StepBatch:
         at += q
     nd, nt = len(decode_rows), len(tiles)
     sizes = [n, n, n, r + 1, r, r, m, nd, nt, nt] + [r * w for w in widths]
-    offsets = np.concatenate([[0], np.cumsum(sizes)])
-    buf = np.zeros(int(offsets[-1]), dtype=np.int32)
+    offsets = [0]
+    for size in sizes:
+        offsets.append(offsets[-1] + size)
+    buf = np.zeros(offsets[-1], dtype=np.int32)
     tok, pos, req, qs, ctx, slots, rows, dec, tfirst, tcount = (
         buf[offsets[i]:offsets[i + 1]] for i in range(NUM_FIXED))
     tabs = [buf[offsets[NUM_FIXED + g]:offsets[NUM_FIXED + 1 + g]].reshape(r, widths[g])
@@ -111,20 +137,36 @@ def build_batch(spans: list[StepSpan], num_groups: int, device) -> StepBatch:
             tabs[g][i, :len(t)] = [p if p >= 0 else 0 for p in t]
         at += q
     qs[r] = at
-    host = torch.from_numpy(buf)
+    return PackedBatch(
+        buf=buf, offsets=offsets, widths=widths, num_tokens=n, num_requests=r, num_logit_rows=m,
+        num_decode=nd, num_tiles=nt, q_lens=[len(s.tokens) for s in spans],
+        ctx_lens=[s.ctx_len for s in spans],
+        max_decode_len=max((s.ctx_len + 1 for s in spans if len(s.tokens) == 1), default=0))
+
+
+def batch_from_device(packed: PackedBatch, dev: torch.Tensor) -> StepBatch:
+    """Cut the device copy ``dev`` of ``packed.buf`` into the descriptor's arrays."""
+    o, r, widths = packed.offsets, packed.num_requests, packed.widths
+    parts = [dev[o[i]:o[i + 1]] for i in range(len(o) - 1)]
+    return StepBatch(
+        num_tokens=packed.num_tokens, num_requests=r, num_logit_rows=packed.num_logit_rows,
+        token_ids=parts[0], positions=parts[1], req_of_token=parts[2], q_start=parts[3],
+        ctx_len=parts[4], state_slots=parts[5], logit_rows=parts[6],
+        block_tables=[parts[NUM_FIXED + g].view(r, widths[g]) for g in range(len(widths))],
+        decode_tokens=parts[7], tile_first=parts[8], tile_count=parts[9],
+        num_decode=packed.num_decode, num_tiles=packed.num_tiles,
+        max_decode_len=packed.max_decode_len, q_lens=packed.q_lens, ctx_lens=packed.ctx_lens,
+        max_q_len=max(packed.q_lens, default=0),
+        max_seq_len=max((c + q for c, q in zip(packed.ctx_lens, packed.q_lens)), default=0),
+    )
+
+
+def build_batch(spans: list[StepSpan], num_groups: int, device) -> StepBatch:
+    """Pack the descriptor into one host buffer and copy it to the device once."""
+    packed = pack_batch(spans, num_groups)
+    host = torch.from_numpy(packed.buf)
     if torch.device(device).type == "cuda":
         dev = host.pin_memory().to(device, non_blocking=True)
     else:
         dev = host.to(device)
-    parts = [dev[int(offsets[i]):int(offsets[i + 1])] for i in range(NUM_FIXED + num_groups)]
-    return StepBatch(
-        num_tokens=n, num_requests=r, num_logit_rows=m,
-        token_ids=parts[0], positions=parts[1], req_of_token=parts[2], q_start=parts[3],
-        ctx_len=parts[4], state_slots=parts[5], logit_rows=parts[6],
-        block_tables=[parts[NUM_FIXED + g].view(r, widths[g]) for g in range(num_groups)],
-        decode_tokens=parts[7], tile_first=parts[8], tile_count=parts[9], num_decode=nd, num_tiles=nt,
-        max_decode_len=max((s.ctx_len + 1 for s in spans if len(s.tokens) == 1), default=0),
-        q_lens=[len(s.tokens) for s in spans], ctx_lens=[s.ctx_len for s in spans],
-        max_q_len=max((len(s.tokens) for s in spans), default=0),
-        max_seq_len=max((s.ctx_len + len(s.tokens) for s in spans), default=0),
-    )
+    return batch_from_device(packed, dev)

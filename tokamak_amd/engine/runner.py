@@ -16,7 +16,8 @@ import torch
 
 from tokamak_amd.cache.manager import CacheManager
 from tokamak_amd.config.registry import load_model_description
-from tokamak_amd.engine.batch import StepBatch, StepSpan, build_batch
+from tokamak_amd.engine.batch import StepBatch, StepSpan, batch_from_device, pack_batch
+from tokamak_amd.engine.decode_graph import DecodeGraph, pow2_at_least
 from tokamak_amd.engine.model import LayeredModel
 from tokamak_amd.engine.storage import CacheStorage
 from tokamak_amd.weights.loader import load_weights
@@ -45,7 +46,7 @@ class StepEntry:
 class ModelRunner:
     def __init__(self, plan, source, *, dtype="bfloat16", page_size: int = 16,
                  kv_pool_tokens: int, max_requests: int = 64,
-                 device: str | torch.device = "cuda:0") -> None:
+                 device: str | torch.device = "cuda:0", use_graphs: bool = True) -> None:
         self.dtype = resolve_dtype(dtype)
         self.device = torch.device(device)
         if self.device.type != "cuda" or not torch.cuda.is_available():
@@ -63,6 +64,8 @@ class ModelRunner:
                                     dtype=self.dtype, device=self.device)
         self.num_groups = len(groups)
         self._ctx_len: dict[object, int] = {}
+        self.use_graphs = use_graphs
+        self._graphs: dict[tuple, DecodeGraph] = {}
 
     @classmethod
     def from_folder(cls, folder: str | Path, **kwargs) -> ModelRunner:
@@ -91,14 +94,18 @@ class ModelRunner:
             self.end(request)
 
     # -- the step --------------------------------------------------------------
-    def prepare(self, entries: list[StepEntry]) -> StepBatch:
+    def _spans(self, entries: list[StepEntry]) -> list[StepSpan]:
         spans = []
         vocab = self.plan.vocab_size
+        seen = set()
         for e in entries:
             if not e.tokens:
                 raise ValueError(f"request {e.request!r} brings no tokens to this step")
             if min(e.tokens) < 0 or max(e.tokens) >= vocab:
                 raise ValueError(f"request {e.request!r} has a token id outside [0, {vocab})")
+            if e.request in seen:
+                raise ValueError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
             ctx = self._ctx_len.get(e.request)
             if ctx is None:
                 slot = self.manager.admit(e.request)
@@ -117,19 +124,45 @@ class ModelRunner:
                 state_slot=self.manager.slots.slot_of(e.request),
                 tables=[self.manager.block_table(e.request, g) for g in range(self.num_groups)],
                 want=list(e.want)))
-        if len({id(s.request) if not isinstance(s.request, (int, str)) else s.request for s in spans}) != len(spans):
-            raise ValueError("a request appears twice in one step")
-        return build_batch(spans, self.num_groups, self.device)
+        return spans
+
+    def prepare(self, entries: list[StepEntry]) -> StepBatch:
+        """Reserve what the entries need and build the step's descriptor."""
+        packed = pack_batch(self._spans(entries), self.num_groups)
+        host = torch.from_numpy(packed.buf)
+        return batch_from_device(packed, host.pin_memory().to(self.device, non_blocking=True))
+
+    def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor:
+        """All entries bring one token: replay the captured step of this shape."""
+        spans = self._spans(entries)
+        wanted = [i for i, s in enumerate(spans) if s.want]
+        for s in spans:
+            s.want = [0]            # the captured step computes every row's logits
+        widths = [pow2_at_least(max(len(s.tables[g]) for s in spans), 16) for g in range(self.num_groups)]
+        packed = pack_batch(spans, self.num_groups, fixed_widths=widths)
+        packed.max_decode_len = pow2_at_least(packed.max_decode_len, 256)
+        key = (len(spans), tuple(widths), packed.max_decode_len)
+        graph = self._graphs.get(key)
+        if graph is None:
+            graph = self._graphs[key] = DecodeGraph(self.model, self.storage, packed, self.device)
+        logits = graph.run(packed)
+        if len(wanted) == len(spans):
+            return logits
+        return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)] if wanted else logits[:0]
 
     @torch.inference_mode()
     def step(self, entries: list[StepEntry]) -> torch.Tensor:
         """Run the entries as one batch; logits float32 [wanted, vocab], in the
-        order of the entries and of each entry's ``want``."""
+        order of the entries and of each entry's ``want``.  The tensor may be
+        reused by the next step: read it before stepping again."""
         if not entries:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
-        batch = self.prepare(entries)
         with torch.cuda.device(self.device):
-            logits = self.model.forward(batch, self.storage)
+            if (self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+                    and all(list(e.want) in ([], [0]) for e in entries)):
+                logits = self._graph_step(entries)
+            else:
+                logits = self.model.forward(self.prepare(entries), self.storage)
         for e in entries:
             self._ctx_len[e.request] += len(e.tokens)
         return logits

@@ -6,10 +6,45 @@ import torch
 
 from tokamak_amd.kernels import ops
 
+SKINNY_MAX_ROWS = 64
+TARGET_WAVES = 2048   # waves wanted in flight for a weight-streaming product
+
+
+def skinny_fits(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    k = x.shape[1]
+    return (k % 8 == 0 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def skinny_plan(n: int, k: int) -> tuple[int, int]:
+    """(row tiles per block, waves per block) from the weight's shape alone, so a
+    row's result does not depend on how many rows are in the batch."""
+    row_tiles = 2 if n >= 8192 else 1
+    blocks = -(-n // (16 * row_tiles))
+    waves = 1
+    while waves < 16 and blocks * waves < TARGET_WAVES and k // (waves * 2) >= 64:
+        waves *= 2
+    if row_tiles == 2 and waves == 2:
+        waves = 4
+    return row_tiles, waves
+
 
 def gemm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
-    """out[M, N] = x[M, K] @ weight[N, K]^T; out is bfloat16 or float32."""
-    if out.dtype == torch.bfloat16:
+    """out[M, N] = x[M, K] @ weight[N, K]^T; out is bfloat16 or float32.
+
+    Up to 64 rows (decode batches, wanted logits rows): the hand-written
+    weight-streaming MFMA kernel.  More rows with bfloat16 output: the library
+    product torch binds (as the reference's nn.Linear does).  More rows with
+    float32 output (many wanted logits rows): the skinny kernel, 64 rows at a time.
+    """
+    m = x.shape[0]
+    n, k = weight.shape
+    if skinny_fits(x, weight) and (m <= SKINNY_MAX_ROWS or out.dtype == torch.float32):
+        row_tiles, waves = skinny_plan(n, k)
+        for at in range(0, m, SKINNY_MAX_ROWS):
+            ops.gemm_skinny(x[at:at + SKINNY_MAX_ROWS], weight, out[at:at + SKINNY_MAX_ROWS],
+                            row_tiles=row_tiles, waves=waves)
+    elif out.dtype == torch.bfloat16:
         torch.matmul(x, weight.t(), out=out)
     else:
         ops.gemm_tiled(x, weight, out)

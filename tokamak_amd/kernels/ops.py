@@ -70,6 +70,10 @@ _SIGS = {
         "tk_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long,
                           c_long, c_long, c_void_p],
     },
+    "gemm_mfma": {
+        "tk_gemm_skinny": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
+                           c_long, c_int, c_int, c_void_p],
+    },
     "attention_generic": {
         "tk_paged_attention_generic": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -204,6 +208,23 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     _check(_fn("gemm_tiled", "tk_gemm_tiled")(_code(a.dtype), _code(out.dtype), _p(a), _p(w), _p(out),
                                               m, n, k, a.stride(0), w.stride(0), out.stride(0),
                                               _stream()), "gemm_tiled")
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, row_tiles: int, waves: int) -> None:
+    """out[M, N] = a[M, K] @ w[N, K]^T on the matrix cores for M <= 64 (bf16 in,
+    float32 accumulation, bf16 or float32 out).  ``row_tiles`` (1 or 2) tiles of
+    16 weight rows per block; ``waves`` (1..16) waves of a block split K."""
+    for t in (a, w, out):
+        _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "the skinny product takes bfloat16 inputs")
+    _need(w.shape[1] == k and out.shape == (m, n), "gemm shapes disagree")
+    _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+          and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "skinny product needs M <= 64 and 16-byte aligned rows")
+    _need(row_tiles in (1, 2) and 1 <= waves <= 16, "row_tiles in (1, 2), waves in 1..16")
+    _check(_fn("gemm_mfma", "tk_gemm_skinny")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
+                                              w.stride(0), out.stride(0), row_tiles, waves, _stream()), "gemm_skinny")
 
 
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
