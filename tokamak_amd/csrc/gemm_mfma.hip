@@ -1,5 +1,9 @@
 // bf16 matrix products on the matrix cores with float32 accumulation.
 //
+// stream (below, second): the weight-streaming product for M <= 64 that decode uses.
+// skinny (first): an older, simpler form that reads MFMA operands straight from
+// memory; kept as the fallback for shapes the streaming kernel refuses.
+//
 // skinny:  C[M,N] = A[M,K] * W[N,K]^T for few rows M (decode batches, M <= 64).
 // The step is bound by reading W once, so the kernel is laid out around the
 // weight stream: a block owns 16*NT weight rows; its waves split K between them
@@ -36,22 +40,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
   const int s_begin = wave * per;
   const int s_end = min(steps, s_begin + per);
 
+  // Row pointers are clamped into the matrix: rows past N (or M) are computed from a
+  // valid row's data and never stored, so the loads need no predicate.
   const bf16_t* wp[NT];
-  bool wok[NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int row = n0 + t * 16 + r;
-    wok[t] = row < N;
-    wp[t] = W + (size_t)(wok[t] ? row : 0) * ldw + kb * 8;
-  }
+  for (int t = 0; t < NT; ++t) wp[t] = W + (size_t)min(n0 + t * 16 + r, N - 1) * ldw + kb * 8;
   const bf16_t* ap[MT];
-  bool aok[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int row = t * 16 + r;
-    aok[t] = row < M;
-    ap[t] = A + (size_t)(aok[t] ? row : 0) * lda + kb * 8;
-  }
+  for (int t = 0; t < MT; ++t) ap[t] = A + (size_t)min(t * 16 + r, M - 1) * lda + kb * 8;
 
   float4v acc[NT][MT];
 #pragma unroll
@@ -59,18 +55,45 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
     for (int j = 0; j < MT; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
 
+  // whole steps (all 32 k inside K), UNR at a time: every load of a group is issued
+  // before the first product, so a wave keeps UNR*(NT+MT) 16-byte loads in flight
+  constexpr int UNR = (NT * MT >= 4) ? 2 : 4;
+  const int s_whole = min(s_end, K / 32);
+  int s = s_begin;
+  for (; s + UNR <= s_whole; s += UNR) {
+    Frag8 wf[UNR][NT], af[UNR][MT];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) wf[u][t].u = *reinterpret_cast<const uint4*>(wp[t] + (s + u) * 32);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) af[u][t].u = *reinterpret_cast<const uint4*>(ap[t] + (s + u) * 32);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][i].v, af[u][j].v, acc[i][j], 0, 0, 0);
+  }
+  // leftover steps, the last of which may reach past K (K is a multiple of 8, so a
+  // 16-byte piece is whole or absent; an absent piece is read at k = 0 and zeroed)
   const uint4 zero = make_uint4(0, 0, 0, 0);
-#pragma unroll 4
-  for (int s = s_begin; s < s_end; ++s) {
-    const int k = s * 32;
-    const bool kok = k + kb * 8 < K;  // K is a multiple of 8: a 16-byte piece is whole or absent
+  for (; s < s_end; ++s) {
+    const bool kok = s * 32 + kb * 8 < K;
+    const int koff = kok ? s * 32 : -kb * 8;
     Frag8 wf[NT], af[MT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
-      wf[t].u = (wok[t] && kok) ? *reinterpret_cast<const uint4*>(wp[t] + k) : zero;
+    for (int t = 0; t < NT; ++t) {
+      const uint4 v = *reinterpret_cast<const uint4*>(wp[t] + koff);
+      wf[t].u = kok ? v : zero;
+    }
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
-      af[t].u = (aok[t] && kok) ? *reinterpret_cast<const uint4*>(ap[t] + k) : zero;
+    for (int t = 0; t < MT; ++t) {
+      const uint4 v = *reinterpret_cast<const uint4*>(ap[t] + koff);
+      af[t].u = kok ? v : zero;
+    }
 #pragma unroll
     for (int i = 0; i < NT; ++i)
 #pragma unroll
@@ -142,6 +165,12 @@ static int pick_tiles(int nt, int waves, const void* A, const void* W, void* C, 
                       long lda, long ldw, long ldc, hipStream_t stream) {
   const int mt = (M + 15) / 16;
 #define TK_GO(NT_, MT_) return pick_waves<NT_, MT_, TO>(waves, A, W, C, M, N, K, lda, ldw, ldc, stream)
+  if (nt >= 4) {
+    if (mt == 1) TK_GO(4, 1);
+    if (mt == 2) TK_GO(4, 2);
+    if (mt == 3) TK_GO(4, 3);
+    TK_GO(4, 4);
+  }
   if (nt >= 2) {
     if (mt == 1) TK_GO(2, 1);
     if (mt == 2) TK_GO(2, 2);
@@ -156,12 +185,193 @@ static int pick_tiles(int nt, int waves, const void* A, const void* W, void* C, 
 }
 
 // out_dtype: 0 float32, 1 bfloat16.  M <= 64, K a multiple of 8, rows 16-byte aligned.
-// nt: weight-row tiles (of 16) per block, 1 or 2; waves: how many waves split K.
+// nt: weight-row tiles (of 16) per block, 1, 2 or 4; waves: how many waves split K.
 TK_API int tk_gemm_skinny(int out_dtype, const void* A, const void* W, void* C, int M, int N, int K,
                           long lda, long ldw, long ldc, int nt, int waves, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
   if (out_dtype == 0) return pick_tiles<float>(nt, waves, A, W, C, M, N, K, lda, ldw, ldc, stream);
   if (out_dtype == 1) return pick_tiles<bf16_t>(nt, waves, A, W, C, M, N, K, lda, ldw, ldc, stream);
+  return -1;
+}
+
+
+// ---------------------------------------------------------------------------
+// stream:  C[M,N] = A[M,K] * W[N,K]^T, M <= 64, W read exactly once and in long
+// contiguous pieces.
+//
+// A block of 4 waves owns 64 weight rows (16 per wave) and one share of K (split
+// s of KS).  K is walked in chunks of 256:
+//   * every wave loads its 16 rows x 256 k (8 KB) with 16-byte loads in which 32
+//     consecutive lanes cover 512 contiguous bytes of one row, keeps them in
+//     registers while the previous chunk is computed, then parks them in its own
+//     LDS tile (row stride 264 elements: conflict-free 16-byte reads by row);
+//   * the block loads the activations' chunk [16*MT x 256] once into a shared
+//     LDS tile (they are small and sit in L2);
+//   * each wave then reads MFMA fragments back from LDS: lane (r, kb) takes
+//     W[row r][k + kb*8 .. +8] as A operand and X[row r][same k] as B operand of
+//     v_mfma_f32_16x16x32_bf16 and accumulates D[weight row][batch row].
+// With KS > 1 every block writes its partial tile to a workspace and bumps a
+// counter of its row block; the block that arrives last adds all KS partials in
+// split order (so the sum does not depend on arrival order), writes C and
+// resets the counter.  Nothing spins or waits on another block.
+// ---------------------------------------------------------------------------
+constexpr int SBK = 256;        // k per chunk
+constexpr int SLD = SBK + 8;    // LDS row stride in elements
+
+template <int MT, typename TO>
+__global__ __launch_bounds__(256) void gemm_stream_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TO* __restrict__ C, int M, int N,
+    int K, long lda, long ldw, long ldc, int chunks_per_split, int KS, float* __restrict__ partial,
+    int* __restrict__ counters) {
+  __shared__ __attribute__((aligned(16))) bf16_t ws[4][16][SLD];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[16 * MT][SLD];
+  __shared__ int last_flag;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, kb = lane >> 4;
+  const int row_block = blockIdx.x, split = blockIdx.y;
+  const int n_wave = row_block * 64 + wave * 16;
+  const int total_chunks = (K + SBK - 1) / SBK;
+  const int c_begin = split * chunks_per_split;
+  const int c_end = min(total_chunks, c_begin + chunks_per_split);
+
+  // loader roles: W piece i of this lane = row 2i + lane/32, 16-byte column lane%32
+  const int w_col = (lane & 31) * 8, w_row0 = lane >> 5;
+  // X pieces of this thread: piece p = i*256 + tid -> row p/32, column p%32
+  const int x_col = (tid & 31) * 8, x_row0 = tid >> 5;
+
+  uint4 wreg[8];
+  uint4 xreg[2 * MT];
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  // Rows are clamped into the matrices (rows past N or M are computed from a valid
+  // row and never stored); only a piece past K is zeroed, after an unconditional
+  // load from k = 0, so the loads of a chunk are all in flight together.
+  const bf16_t* wrow[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) wrow[i] = W + (size_t)min(n_wave + 2 * i + w_row0, N - 1) * ldw;
+  const bf16_t* xrow[2 * MT];
+#pragma unroll
+  for (int i = 0; i < 2 * MT; ++i) xrow[i] = A + (size_t)min(i * 8 + x_row0, M - 1) * lda;
+  auto fetch = [&](int c) {
+    const int k0 = c * SBK;
+    const bool kw = k0 + w_col < K, kx = k0 + x_col < K;
+    const int wo = kw ? k0 + w_col : 0, xo = kx ? k0 + x_col : 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) wreg[i] = *reinterpret_cast<const uint4*>(wrow[i] + wo);
+#pragma unroll
+    for (int i = 0; i < 2 * MT; ++i) xreg[i] = *reinterpret_cast<const uint4*>(xrow[i] + xo);
+    if (k0 + SBK > K) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) wreg[i] = kw ? wreg[i] : zero;
+#pragma unroll
+      for (int i = 0; i < 2 * MT; ++i) xreg[i] = kx ? xreg[i] : zero;
+    }
+  };
+
+  float4v acc[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  if (c_begin < c_end) fetch(c_begin);
+  for (int c = c_begin; c < c_end; ++c) {
+    __syncthreads();  // the previous chunk's fragments have been read
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      *reinterpret_cast<uint4*>(&ws[wave][2 * i + w_row0][w_col]) = wreg[i];
+#pragma unroll
+    for (int i = 0; i < 2 * MT; ++i)
+      *reinterpret_cast<uint4*>(&xs[i * 8 + x_row0][x_col]) = xreg[i];
+    __syncthreads();
+    if (c + 1 < c_end) fetch(c + 1);  // in flight while this chunk is multiplied
+#pragma unroll
+    for (int s = 0; s < SBK / 32; ++s) {
+      Frag8 wf;
+      wf.u = *reinterpret_cast<const uint4*>(&ws[wave][r][s * 32 + kb * 8]);
+#pragma unroll
+      for (int j = 0; j < MT; ++j) {
+        Frag8 xf;
+        xf.u = *reinterpret_cast<const uint4*>(&xs[j * 16 + r][s * 32 + kb * 8]);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf.v, acc[j], 0, 0, 0);
+      }
+    }
+  }
+
+  if (KS > 1) {
+    // partial tiles are stored in accumulator layout: [split][row block][wave][j][lane][4]
+    const size_t tile = (size_t)4 * MT * 256;
+    float* mine = partial + ((size_t)split * gridDim.x + row_block) * tile + (size_t)(wave * MT) * 256;
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+      *reinterpret_cast<float4*>(mine + j * 256 + lane * 4) =
+          make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) last_flag = (atomicAdd(&counters[row_block], 1) == KS - 1);
+    __syncthreads();
+    if (!last_flag) return;
+    __threadfence();
+#pragma unroll
+    for (int j = 0; j < MT; ++j) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < KS; ++s) {
+      const float* src = partial + ((size_t)s * gridDim.x + row_block) * tile + (size_t)(wave * MT) * 256;
+#pragma unroll
+      for (int j = 0; j < MT; ++j) {
+        const float4 v = *reinterpret_cast<const float4*>(src + j * 256 + lane * 4);
+        acc[j][0] += v.x;
+        acc[j][1] += v.y;
+        acc[j][2] += v.z;
+        acc[j][3] += v.w;
+      }
+    }
+    if (tid == 0) counters[row_block] = 0;  // ready for the next product on this stream
+  }
+
+  // acc[j][e] = C[batch row j*16 + r][weight row n_wave + kb*4 + e]
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int m = j * 16 + r;
+    if (m >= M) continue;
+    const int n = n_wave + kb * 4;
+    TO* cp = C + (size_t)m * ldc + n;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (n + e < N) Elem<TO>::store(cp + e, acc[j][e]);
+  }
+}
+
+template <typename TO>
+static int launch_stream(const void* A, const void* W, void* C, int M, int N, int K, long lda,
+                         long ldw, long ldc, int KS, float* partial, int* counters,
+                         hipStream_t stream) {
+  const int total_chunks = (K + SBK - 1) / SBK;
+  const int cps = (total_chunks + KS - 1) / KS;
+  KS = (total_chunks + cps - 1) / cps;  // no empty splits
+  dim3 grid((N + 63) / 64, KS);
+  const int mt = (M + 15) / 16;
+#define TK_STREAM(MT_)                                                                           \
+  gemm_stream_kernel<MT_, TO><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W,     \
+                                                        (TO*)C, M, N, K, lda, ldw, ldc, cps, KS, \
+                                                        partial, counters)
+  if (mt == 1) TK_STREAM(1);
+  else if (mt == 2) TK_STREAM(2);
+  else if (mt == 3) TK_STREAM(3);
+  else TK_STREAM(4);
+#undef TK_STREAM
+  return launch_status();
+}
+
+// out_dtype: 0 float32, 1 bfloat16.  M <= 64; K a multiple of 8; rows 16-byte aligned.
+// splits: shares of K (>= 1).  With splits > 1, `partial` must hold
+// splits * ceil(N/64) * 4 * ceil(M/16) * 256 floats and `counters` ceil(N/64) ints
+// that are zero before the first call (the kernel leaves them zero).
+TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, int M, int N, int K,
+                          long lda, long ldw, long ldc, int splits, float* partial, int* counters,
+                          hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1) return -1;
+  if (splits > 1 && (!partial || !counters)) return -1;
+  if ((N + 63) / 64 > 0x7fffffff / 2 || splits > 65535) return -1;
+  if (out_dtype == 0) return launch_stream<float>(A, W, C, M, N, K, lda, ldw, ldc, splits, partial, counters, stream);
+  if (out_dtype == 1) return launch_stream<bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, splits, partial, counters, stream);
   return -1;
 }

@@ -7,7 +7,7 @@ import torch
 from tokamak_amd.kernels import ops
 
 SKINNY_MAX_ROWS = 64
-TARGET_WAVES = 2048   # waves wanted in flight for a weight-streaming product
+TARGET_WAVES = 4096   # waves wanted in flight for a weight-streaming product
 
 
 def skinny_fits(x: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -16,16 +16,25 @@ def skinny_fits(x: torch.Tensor, weight: torch.Tensor) -> bool:
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def skinny_plan(n: int, k: int) -> tuple[int, int]:
-    """(row tiles per block, waves per block) from the weight's shape alone, so a
-    row's result does not depend on how many rows are in the batch."""
-    row_tiles = 2 if n >= 8192 else 1
+def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
+    """(tiles of 16 weight rows per block, waves of a block that split K).
+
+    More row tiles per block let the activation fragments be reused; more waves
+    put more loads in flight when the matrix has few rows.  Chosen from
+    measurements on the projection shapes of 0.6B to 32B models.
+    """
+    if m > 32:
+        row_tiles = 4 if n >= 6144 else 2
+    elif m <= 2 or n < 6144:
+        row_tiles = 1
+    else:
+        row_tiles = 4 if n >= 65536 else 2
     blocks = -(-n // (16 * row_tiles))
-    waves = 1
-    while waves < 16 and blocks * waves < TARGET_WAVES and k // (waves * 2) >= 64:
+    waves = 4
+    while waves < 16 and blocks * waves < TARGET_WAVES:
         waves *= 2
-    if row_tiles == 2 and waves == 2:
-        waves = 4
+    while waves > 1 and k // waves < 64:
+        waves //= 2
     return row_tiles, waves
 
 
@@ -40,7 +49,7 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
     m = x.shape[0]
     n, k = weight.shape
     if skinny_fits(x, weight) and (m <= SKINNY_MAX_ROWS or out.dtype == torch.float32):
-        row_tiles, waves = skinny_plan(n, k)
+        row_tiles, waves = skinny_plan(min(m, SKINNY_MAX_ROWS), n, k)
         for at in range(0, m, SKINNY_MAX_ROWS):
             ops.gemm_skinny(x[at:at + SKINNY_MAX_ROWS], weight, out[at:at + SKINNY_MAX_ROWS],
                             row_tiles=row_tiles, waves=waves)

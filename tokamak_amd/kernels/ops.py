@@ -71,6 +71,8 @@ _SIGS = {
                           c_long, c_long, c_void_p],
     },
     "gemm_mfma": {
+        "tk_gemm_stream": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
+                           c_long, c_int, c_void_p, c_void_p, c_void_p],
         "tk_gemm_skinny": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                            c_long, c_int, c_int, c_void_p],
     },
@@ -210,6 +212,32 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
                                               _stream()), "gemm_tiled")
 
 
+def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: int,
+                partial: torch.Tensor | None, counters: torch.Tensor | None) -> None:
+    """out[M, N] = a[M, K] @ w[N, K]^T for M <= 64 with the weight-streaming MFMA
+    kernel.  ``splits`` shares of K; with more than one, ``partial`` (float32) and
+    ``counters`` (int32, all zero) are the workspace the blocks meet in."""
+    for t in (a, w, out):
+        _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "the streaming product takes bfloat16 inputs")
+    _need(w.shape[1] == k and out.shape == (m, n), "gemm shapes disagree")
+    _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+          and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "streaming product needs M <= 64 and 16-byte aligned rows")
+    _need(1 <= splits <= 64, "splits in 1..64")
+    if splits > 1:
+        row_blocks = -(-n // 64)
+        need = splits * row_blocks * 4 * (-(-m // 16)) * 256
+        _need(partial is not None and partial.dtype == torch.float32 and partial.numel() >= need
+              and partial.is_cuda and partial.is_contiguous(), "split-K workspace too small")
+        _need(counters is not None and counters.dtype == torch.int32 and counters.numel() >= row_blocks
+              and counters.is_cuda and counters.is_contiguous(), "split-K counters too small")
+    _check(_fn("gemm_mfma", "tk_gemm_stream")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
+                                              w.stride(0), out.stride(0), splits, _p(partial), _p(counters),
+                                              _stream()), "gemm_stream")
+
+
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, row_tiles: int, waves: int) -> None:
     """out[M, N] = a[M, K] @ w[N, K]^T on the matrix cores for M <= 64 (bf16 in,
     float32 accumulation, bf16 or float32 out).  ``row_tiles`` (1 or 2) tiles of
@@ -222,7 +250,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, row_tile
     _need(w.shape[1] == k and out.shape == (m, n), "gemm shapes disagree")
     _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "skinny product needs M <= 64 and 16-byte aligned rows")
-    _need(row_tiles in (1, 2) and 1 <= waves <= 16, "row_tiles in (1, 2), waves in 1..16")
+    _need(row_tiles in (1, 2, 4) and 1 <= waves <= 16, "row_tiles in (1, 2, 4), waves in 1..16")
     _check(_fn("gemm_mfma", "tk_gemm_skinny")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
                                               w.stride(0), out.stride(0), row_tiles, waves, _stream()), "gemm_skinny")
 
