@@ -1,0 +1,186 @@
+"""Each part of a layer alone against the plain implementation's function for
+it, at sizes of its own; and the sampler against the plain distribution."""
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from kernel_util import make_batch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = {torch.float32: dict(rtol=2e-4, atol=2e-5), torch.bfloat16: dict(rtol=3e-2, atol=2e-2)}
+
+
+def rand(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def fetcher(tensors, dtype):
+    def fetch(name):
+        t = tensors[name]
+        return t.to(DEV, torch.float32 if t.dim() == 1 else dtype).contiguous()
+    return fetch
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_rmsnorm_part(dtype):
+    from tokamak_amd.config import get_part
+
+    norm = get_part("norm", "rmsnorm")(dim=200, eps=3e-6, dtype=dtype, device=DEV)
+    assert list(norm.expected_tensors("n.")) == ["n.weight"]
+    w = 1 + 0.2 * rand(200, seed=1)
+    norm.bind("n.", fetcher({"n.weight": w}, dtype))
+    resid, delta = rand(9, 200, seed=2, scale=2.0), rand(9, 200, seed=3).to(dtype)
+    r = resid.to(DEV)
+    h = norm.forward(r, delta.to(DEV))
+    x = resid + delta.float()
+    torch.testing.assert_close(h.cpu().float(), plain.rmsnorm(x, w, 3e-6), **TOL[dtype])
+    torch.testing.assert_close(r.cpu(), x, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_swiglu_part(dtype):
+    from tokamak_amd.config import get_part
+
+    H, I = 96, 200
+    ff = get_part("feed_forward", "swiglu")(hidden_size=H, intermediate_size=I, dtype=dtype, device=DEV)
+    w = {"m.gate_proj.weight": rand(I, H, seed=1, scale=H ** -0.5).to(dtype).float(),
+         "m.up_proj.weight": rand(I, H, seed=2, scale=H ** -0.5).to(dtype).float(),
+         "m.down_proj.weight": rand(H, I, seed=3, scale=I ** -0.5).to(dtype).float()}
+    assert set(ff.expected_tensors("m.")) == set(w)
+    ff.bind("m.", fetcher(w, dtype))
+    for rows in (1, 7, 70):
+        x = rand(rows, H, seed=4).to(dtype)
+        got = ff.forward(x.to(DEV), None).cpu().float()
+        torch.testing.assert_close(got, plain.swiglu(x.float(), w, "m."), **TOL[dtype])
+    # zero gate weights give zero output (reference tests/unit/test_layers.py:71-79)
+    w0 = dict(w)
+    w0["m.gate_proj.weight"] = torch.zeros(I, H)
+    ff.bind("m.", fetcher(w0, dtype))
+    assert ff.forward(rand(3, H, seed=5).to(dtype).to(DEV), None).abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_rotary_part_tables(dtype):
+    from tokamak_amd.config import get_part
+
+    rot = get_part("position", "rotary_half")(rotary_dim=48, theta=50000.0, dtype=dtype, device=DEV)
+    batch = make_batch([(5, 1000, list(range(70))), (1, 0, [70])])
+    cos, sin = rot.prepare(batch)
+    assert rot.prepare(batch)[0] is cos            # once per step, shared by the layers
+    positions = torch.tensor([1000, 1001, 1002, 1003, 1004, 0])
+    want_cos, want_sin = plain.rope_tables(positions, 48, 50000.0)
+    torch.testing.assert_close(cos.cpu(), want_cos[:, :24], rtol=1e-5, atol=2e-6)
+    torch.testing.assert_close(sin.cpu(), want_sin[:, :24], rtol=1e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("nh, nkv, hd, H, ps", [(6, 2, 32, 80, 8), (8, 2, 128, 96, 16), (5, 5, 48, 64, 16)])
+def test_attention_part_whole_and_in_portions(dtype, nh, nkv, hd, H, ps):
+    """The mixer alone: one request whole, then the same tokens in portions and a
+    final single token, against the plain attention block."""
+    from tokamak_amd.config import PartSpec, get_part
+    from tokamak_amd.engine.storage import SlotStore
+
+    pos = PartSpec.of("rotary_half", rotary_dim=hd, theta=10000.0)
+    mixer = get_part("mixer", "gqa_attention")(
+        hidden_size=H, num_heads=nh, num_kv_heads=nkv, head_dim=hd, qk_norm_eps=1e-6,
+        softmax_scale=hd ** -0.5, position=(pos.kind, pos.params), window=None, dtype=dtype, device=DEV)
+    w = {"a.q_proj.weight": rand(nh * hd, H, seed=1, scale=H ** -0.5), "a.k_proj.weight": rand(nkv * hd, H, seed=2, scale=H ** -0.5),
+         "a.v_proj.weight": rand(nkv * hd, H, seed=3, scale=H ** -0.5), "a.o_proj.weight": rand(H, nh * hd, seed=4, scale=(nh * hd) ** -0.5),
+         "a.q_norm.weight": 1 + 0.2 * rand(hd, seed=5), "a.k_norm.weight": 1 + 0.2 * rand(hd, seed=6)}
+    w = {k: (v.to(dtype).float() if v.dim() == 2 else v) for k, v in w.items()}
+    assert set(mixer.expected_tensors("a.")) == set(w)
+    mixer.bind("a.", fetcher(w, dtype))
+    req = mixer.cache_request()
+    assert req.arrays == ("k", "v") and req.elems_per_token == nkv * hd and req.window is None
+    T = 45
+    x = rand(T, H, seed=7).to(dtype)
+    s = dict(nh=nh, nkv=nkv, hd=hd, eps=1e-6, theta=10000.0)
+    want = plain.attention_block(x.float(), w, "a.", s, torch.arange(T))
+    pages = 8
+    table = [5, 2, 7, 0, 3, 6][: -(-T // ps)] if ps == 16 else [5, 2, 7, 0, 3, 6]
+    for cuts in ([T], [16, 7, 2, 19, 1]):
+        store = SlotStore(group=0, page_size=ps, arrays={
+            "k": torch.full((pages, nkv * hd * ps), float("nan"), dtype=dtype, device=DEV),
+            "v": torch.full((pages, nkv * hd * ps), float("nan"), dtype=dtype, device=DEV)})
+        at, outs = 0, []
+        for n in cuts:
+            batch = make_batch([(n, at, table)])
+            outs.append(mixer.forward(x[at:at + n].to(DEV), batch, store))
+            at += n
+        torch.testing.assert_close(torch.cat(outs).cpu().float(), want, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_embedding_and_head_parts(dtype):
+    from tokamak_amd.config import get_part
+
+    V, H = 331, 120
+    emb = get_part("embedding", "token_embedding")(vocab_size=V, dim=H, dtype=dtype, device=DEV)
+    table = rand(V, H, seed=1).to(dtype).float()
+    emb.bind("e.", fetcher({"e.weight": table}, dtype))
+    ids = torch.tensor([3, 330, 0, 3], dtype=torch.int32, device=DEV)
+    torch.testing.assert_close(emb.forward(ids).cpu(), table[ids.cpu().long()], rtol=0, atol=0)
+    head = get_part("head", "linear_head")(vocab_size=V, dim=H, tied=True, dtype=dtype, device=DEV)
+    assert head.expected_tensors("h.")["h.weight"].ignored
+    head.tie(emb)
+    h = rand(5, H, seed=2).to(dtype)
+    logits = head.forward(h.to(DEV))
+    assert logits.dtype == torch.float32
+    torch.testing.assert_close(logits.cpu(), h.float() @ table.T, rtol=1e-3, atol=1e-3)
+
+
+# -- sampler -------------------------------------------------------------------
+def test_argmax_first_maximum_wins():
+    from tokamak_amd.sampling.sampler import greedy_tokens
+
+    logits = torch.tensor([[0.1, 2.0, -1.0], [3.0, 0.0, 0.5]], device=DEV)   # reference test_sampler.py:12-15
+    assert greedy_tokens(logits).tolist() == [1, 0]
+    big = torch.randn(5, 151936, generator=torch.Generator().manual_seed(0))
+    big[2, 77] = big[2, 150000] = 50.0          # a tie: the lower index wins
+    assert greedy_tokens(big.to(DEV)).tolist() == big.argmax(-1).tolist()
+    assert greedy_tokens(big.to(DEV))[2].item() == 77
+
+
+@pytest.mark.parametrize("V", [5, 331, 151936])
+def test_sampling_distribution_matches_plain(V):
+    from tokamak_amd import SamplingParams
+    from tokamak_amd.sampling.sampler import sample_tokens
+
+    logits = torch.randn(6, V, generator=torch.Generator().manual_seed(V)) * 3
+    params = [SamplingParams(temperature=0.8), SamplingParams(temperature=1.3, top_k=4),
+              SamplingParams(temperature=1.0, top_p=0.7), SamplingParams(temperature=0.5, top_k=50, top_p=0.9),
+              SamplingParams(temperature=0.0), SamplingParams(temperature=2.0, top_k=1)]
+    tokens, probs = sample_tokens(logits.to(DEV), params, [1, 2, 3, 4, 5, 6], [0] * 6, return_probs=True)
+    tokens, probs = tokens.cpu(), probs.cpu()
+    for i, p in enumerate(params):
+        if p.is_greedy:
+            assert tokens[i].item() == logits[i].argmax().item()
+            continue
+        want = plain.sampling_probs(logits[i], p.temperature, p.top_k, p.top_p).float()
+        torch.testing.assert_close(probs[i], want, rtol=2e-3, atol=1e-6)
+        assert (probs[i] > 0).sum() == (want > 0).sum()
+        assert probs[i][tokens[i]] > 0
+    assert tokens[5].item() == logits[5].argmax().item()       # top_k = 1 is greedy at any temperature
+
+
+def test_sampling_vectors_and_seeds():
+    """Vectors of reference tests/unit/test_sampler.py:26-56."""
+    from tokamak_amd import SamplingParams
+    from tokamak_amd.sampling.sampler import sample_tokens
+
+    def draws(logits, params, n=200):
+        rows = logits.repeat(n, 1).to(DEV)
+        return sample_tokens(rows, [params] * n, list(range(n)), [0] * n).cpu().tolist()
+
+    assert set(draws(torch.tensor([[1.0, 2.0, 3.0, 4.0, 5.0]]), SamplingParams(top_k=2))) == {3, 4}
+    assert set(draws(torch.tensor([[0.5, 0.3, 0.2]]).log(), SamplingParams(top_p=0.7))) == {0, 1}
+    assert set(draws(torch.tensor([[0.9, 0.06, 0.04]]).log(), SamplingParams(top_p=0.05), 50)) == {0}
+    logits = torch.randn(1, 1000, generator=torch.Generator().manual_seed(7))
+    p = SamplingParams(temperature=0.8, top_p=0.95)
+    a = sample_tokens(logits.repeat(4, 1).to(DEV), [p] * 4, [42, 42, 43, 42], [0, 0, 0, 1]).cpu().tolist()
+    assert a[0] == a[1]                     # same seed and draw count: same token
+    counts = torch.bincount(torch.tensor(draws(torch.tensor([[0.5, 0.3, 0.2]]).log(), SamplingParams(), 4000)), minlength=3)
+    torch.testing.assert_close(counts.float() / 4000, torch.tensor([0.5, 0.3, 0.2]), rtol=0, atol=0.03)

@@ -50,6 +50,17 @@ class LayeredModel:
         self.final_norm = _build("norm", plan.final_norm, dtype, device)
         self.head = _build("head", plan.head, dtype, device)
 
+    @property
+    def capturable(self) -> bool:
+        """Whether a decode step of this model may be recorded into a HIP graph."""
+        parts = [self.embedding, self.final_norm, self.head]
+        for block in self.blocks:
+            parts += [block.mixer, block.feed_forward, block.mixer_norm, block.feed_forward_norm]
+            position = getattr(block.mixer, "position", None)
+            if position is not None:
+                parts.append(position)
+        return all(getattr(p, "capturable", False) for p in parts)
+
     # -- weights -------------------------------------------------------------
     def _named_parts(self):
         p = self.plan

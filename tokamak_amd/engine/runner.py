@@ -64,7 +64,7 @@ class ModelRunner:
                                     dtype=self.dtype, device=self.device)
         self.num_groups = len(groups)
         self._ctx_len: dict[object, int] = {}
-        self.use_graphs = use_graphs
+        self.use_graphs = use_graphs and self.model.capturable
         self._graphs: dict[tuple, DecodeGraph] = {}
 
     @classmethod

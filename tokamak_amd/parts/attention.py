@@ -23,6 +23,8 @@ class GQAAttention(Mixer):
     ``window``: None for full causal attention, W to see the last W positions.
     """
 
+    capturable = True
+
     def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qk_norm_eps: float | None, softmax_scale: float, position, window: int | None,
                  dtype, device) -> None:

@@ -30,7 +30,15 @@ Fetch = Callable[[str], "torch.Tensor | None"]
 
 
 class Part:
-    """Common base: parameters, expected tensors, binding."""
+    """Common base: parameters, expected tensors, binding.
+
+    ``capturable``: the part's ``forward`` only launches work on the current
+    stream (no host synchronisation, no data-dependent host decisions), so a
+    decode step through it may be recorded into a HIP graph.  A model is captured
+    only if every part of it says so.
+    """
+
+    capturable = False
 
     def __init__(self, *, dtype: torch.dtype, device: torch.device | str) -> None:
         self.dtype = dtype

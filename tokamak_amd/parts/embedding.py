@@ -15,6 +15,8 @@ class TokenEmbedding(Part):
     """Plain row gather into the float32 residual stream, no scaling
     (reference: src/tokamak/model/transformer.py:140)."""
 
+    capturable = True
+
     def __init__(self, *, vocab_size: int, dim: int, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)
         self.vocab_size, self.dim = int(vocab_size), int(dim)
@@ -35,6 +37,8 @@ class TokenEmbedding(Part):
 class LinearHead(Part):
     """logits = h @ W^T in float32; a tied head uses the embedding matrix itself
     (reference: src/tokamak/model/transformer.py:154-156,173-176)."""
+
+    capturable = True
 
     def __init__(self, *, vocab_size: int, dim: int, tied: bool, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)

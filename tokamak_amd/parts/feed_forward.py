@@ -19,6 +19,8 @@ class SwiGLU(FeedForward):
     yields both halves.
     """
 
+    capturable = True
+
     def __init__(self, *, hidden_size: int, intermediate_size: int, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)
         self.hidden_size = int(hidden_size)

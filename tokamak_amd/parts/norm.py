@@ -18,6 +18,8 @@ class RMSNorm(Norm):
     computes the statistics in float32, rounds, then multiplies by the weight).
     """
 
+    capturable = True
+
     def __init__(self, *, dim: int, eps: float, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)
         self.dim = int(dim)

@@ -19,6 +19,8 @@ class RotaryHalf(PositionEncoding):
     is applied by the mixer's fused kernel.
     """
 
+    capturable = True
+
     def __init__(self, *, rotary_dim: int, theta: float, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)
         if rotary_dim % 2:
