@@ -10,14 +10,14 @@ from tokamak_amd.engine.batch import StepSpan, build_batch
 
 def pack_pages(k_cache, v_cache, k_seq, v_seq, table, ps):
     """Write a request's keys/values ([T, nkv, hd]) into its pages.
-    K page: [nkv][hd/8][ps][8]; V page: [nkv][hd][ps]."""
+    K page: [nkv][hd/8][ps][8]; V page: [nkv][hd/16][ps/4][16][4]."""
     T, nkv, hd = k_seq.shape
     for t in range(T):
         page, off = table[t // ps], t % ps
         kp = k_cache[page].view(nkv, hd // 8, ps, 8)
-        vp = v_cache[page].view(nkv, hd, ps)
+        vp = v_cache[page].view(nkv, hd // 16, ps // 4, 16, 4)
         kp[:, :, off, :] = k_seq[t].view(nkv, hd // 8, 8).to(k_cache.dtype)
-        vp[:, :, off] = v_seq[t].to(v_cache.dtype)
+        vp[:, :, off // 4, :, off % 4] = v_seq[t].view(nkv, hd // 16, 16).to(v_cache.dtype)
 
 
 def unpack_pages(k_cache, v_cache, table, T, nkv, hd, ps):
@@ -26,7 +26,7 @@ def unpack_pages(k_cache, v_cache, table, T, nkv, hd, ps):
     for t in range(T):
         page, off = table[t // ps], t % ps
         k[t] = k_cache[page].view(nkv, hd // 8, ps, 8)[:, :, off, :].reshape(nkv, hd).cpu()
-        v[t] = v_cache[page].view(nkv, hd, ps)[:, :, off].cpu()
+        v[t] = v_cache[page].view(nkv, hd // 16, ps // 4, 16, 4)[:, :, off // 4, :, off % 4].reshape(nkv, hd).cpu()
     return k, v
 
 

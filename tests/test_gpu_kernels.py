@@ -154,7 +154,7 @@ def test_unsupported_sizes_are_refused_not_wrong():
     cache = torch.zeros(2, 2 * 12 * 16, device=DEV)
     tables = torch.zeros(1, 4, dtype=torch.int32, device=DEV)
     idx = torch.zeros(1, dtype=torch.int32, device=DEV)
-    with pytest.raises(ops.KernelError, match="multiple of 8"):
+    with pytest.raises(ops.KernelError, match="multiple of 16"):
         ops.paged_attention_generic(q, cache, cache, tables, idx, idx, q.clone(), num_heads=4, num_kv_heads=2,
                                     head_dim=12, page_size=16, scale=1.0)
     with pytest.raises(ops.KernelError, match="GPU"):

@@ -1,4 +1,4 @@
-// Paged causal attention for any head size (multiple of 8, up to 512), any
+// Paged causal attention for any head size (multiple of 16, up to 512), any
 // number of heads and groups, any page size that is a multiple of 8, in float32
 // or bf16 storage with float32 arithmetic throughout.  It serves prompt portions
 // and decode tokens alike: every query token walks its own request's block table
@@ -9,7 +9,7 @@
 // (online softmax), so the result does not depend on how the request was cut
 // into steps or what else is in the batch.
 //
-// Cache pages: K [nkv][hd/8][ps][8], V [nkv][hd][ps] (see elementwise.hip).
+// Cache pages: K [nkv][hd/8][ps][8], V [nkv][hd/16][ps/4][16][4] (see elementwise.hip).
 #include "common.h"
 
 using namespace tk;
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_generic_kernel(
         for (int e = 0; e < 8; ++e) dot = fmaf(q_s[j * 8 + e], Elem<T>::load(kk + e), dot);
       }
       s = dot;
-      vbase = (long)((size_t)page * page_elems + head_off + off);
+      vbase = (long)((size_t)page * page_elems + head_off + (size_t)(off >> 2) * 64 + (off & 3));
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -76,10 +76,11 @@ __global__ __launch_bounds__(kWave) void paged_attention_generic_kernel(
     for (int i = 0; i < kAccPerLane; ++i) {
       const int d = lane + i * kWave;
       if (d < hd) {
+        const size_t v_dim_off = (size_t)(d >> 4) * (ps >> 2) * 64 + (d & 15) * 4;
         float a = acc[i] * alpha;
         for (int t = 0; t < count; ++t) {
           const long b = base_s[t];
-          if (b >= 0) a = fmaf(p_s[t], Elem<T>::load(v_cache + b + (size_t)d * ps), a);
+          if (b >= 0) a = fmaf(p_s[t], Elem<T>::load(v_cache + b + v_dim_off), a);
         }
         acc[i] = a;
       }
@@ -100,7 +101,7 @@ TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_ca
                                       int N, int nh, int nkv, int hd, int ps, int max_pages,
                                       float scale, int window, hipStream_t stream) {
   if (N <= 0) return 0;
-  if (hd > kMaxHd || hd % 8 != 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || nh > 65535) return -1;
+  if (hd > kMaxHd || hd % 16 != 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || ps % 4 != 0 || nh > 65535) return -1;
   dim3 grid(N, nh);
   if (dtype == 0)
     paged_attention_generic_kernel<float><<<grid, kWave, 0, stream>>>(

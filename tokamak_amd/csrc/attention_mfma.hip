@@ -1,12 +1,13 @@
 // Paged causal attention on the matrix cores (bf16 in, float32 softmax and
-// accumulation) for head sizes 64 and 128 and page sizes that are multiples of 16.
+// accumulation) for head sizes 64 and 128 and page sizes 16, 32, 64, ... (powers of two).
 //
 // One 64-lane wave owns a work item: up to 16 "columns" per column set that share
 // one kv head and one request, and a range of that request's keys (a split).
 //   heads mode  (decode):  the columns of set s are query heads s*16 .. s*16+15 of
 //                          the group, all of one token;
-//   tokens mode (prefill): the columns are 16 consecutive tokens of one request,
-//                          set s is query head s of the group.
+//   tokens mode:           the columns are 16 consecutive tokens of one request,
+//                          set s is query head s of the group (kept for reference;
+//                          prompt portions use attention_prefill_kernel below).
 // Keys are taken 16 at a time (one MFMA tile, never across a page edge):
 //   S^T[key][col] = K[key][:] . Q[col][:]      v_mfma_f32_16x16x32_bf16, K rows as A
 //   P^T = exp2(S^T * c - m[col])               float32, one column per lane
@@ -14,7 +15,7 @@
 // The result layout of the first product is exactly the B operand layout of the
 // second, so probabilities never leave registers, and both K and V^T operands
 // are loaded straight from the pages (K page [nkv][hd/8][ps][8], V page
-// [nkv][hd][ps]) in contiguous 16- and 8-byte pieces: no LDS is used.
+// [nkv][hd/16][ps/4][16][4]) in contiguous 16- and 8-byte pieces.
 //
 // With more than one split the wave writes an unnormalised partial (o, m, l) and
 // a second kernel merges the splits of each (token, head).
@@ -114,10 +115,12 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
 #pragma unroll
     for (int c = 0; c < KCH; ++c)
       kreg[c].u = *reinterpret_cast<const uint4*>(kp + (size_t)(c * 4 + kb) * ps * 8);
-    const bf16_t* vp = v_cache + (size_t)page * page_elems + head_off + (size_t)col * ps + off + kb * 4;
+    // V page [hd/16][ps/4][16][4]: lane (dim col, quad kb) of block d reads 8 bytes, the
+    // wave 512 contiguous bytes
+    const bf16_t* vp = v_cache + (size_t)page * page_elems + head_off + (size_t)((off >> 2) + kb) * 64 + col * 4;
 #pragma unroll
     for (int d = 0; d < DBL; ++d)
-      vreg[d].u = *reinterpret_cast<const uint2*>(vp + (size_t)d * 16 * ps);
+      vreg[d].u = *reinterpret_cast<const uint2*>(vp + (size_t)d * (ps >> 2) * 64);
   };
 
   load_tile(k_begin);
@@ -250,6 +253,226 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(
   for (int i = 0; i < HD / 64; ++i) out[orow * HD + lane + i * 64] = float_to_bf16(o[i] * inv);
 }
 
+// ---------------------------------------------------------------------------
+// Prompt portions: one block per (16-token tile, kv head, group of HPB query
+// heads), one wave per query head.  The waves share the keys and values: the
+// block copies 64 keys at a time from the pages into LDS (same piece order as in
+// the pages, so every wave reads its MFMA operands back in contiguous 16- and
+// 8-byte pieces without bank conflicts), the next 64 keys already being in
+// flight into registers while the current ones are multiplied.  Per 64 keys a
+// wave does one softmax update: 16 QK^T products (16x16x32), one maximum, one
+// rescale, then 16 PV products (16x16x32 over two 16-key groups at a time: the
+// k index of that product runs over quads of both groups, which is exactly how
+// the lanes hold the probabilities).
+// ---------------------------------------------------------------------------
+template <int HD, int HPB>
+__global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
+    const int* __restrict__ positions, const int* __restrict__ req_of_token,
+    const int* __restrict__ item_token, const int* __restrict__ item_count,
+    bf16_t* __restrict__ out, int num_items, int nh, int nkv, int ps, float scale_log2) {
+  constexpr int KCH = HD / 32, DBL = HD / 16;
+  constexpr int THREADS = 64 * HPB;
+  constexpr int KPIECES = 4 * (HD / 8) * 16;   // 16-byte pieces of K per stage of 64 keys
+  constexpr int VPIECES = 4 * (HD / 16) * 32;  // and of V
+  constexpr int KPT = KPIECES / THREADS, VPT = VPIECES / THREADS;
+  __shared__ __attribute__((aligned(16))) bf16_t ks[KPIECES * 8];
+  __shared__ __attribute__((aligned(16))) bf16_t vs[VPIECES * 8];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, kb = lane >> 4;
+  const int G = nh / nkv;
+  const int groups_per_kv = G / HPB;
+  const int kvh = blockIdx.x / groups_per_kv;
+  const int head = kvh * G + (blockIdx.x % groups_per_kv) * HPB + wave;
+  const int item = num_items - 1 - blockIdx.y;  // later tiles have more keys: start them first
+
+  const int n0 = item_token[item];
+  const int count = item_count[item];
+  const int pos0 = positions[n0];
+  const int last_pos = pos0 + count - 1;
+  const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
+  const size_t page_elems = (size_t)nkv * HD * ps;
+  const size_t head_off = (size_t)kvh * HD * ps;
+  const int c_pos = pos0 + col;
+  const bool c_valid = col < count;
+
+  bf16x8 qreg[KCH];
+  {
+    const bf16_t* qp = q + ((size_t)(n0 + (c_valid ? col : 0)) * nh + head) * HD + kb * 8;
+#pragma unroll
+    for (int c = 0; c < KCH; ++c) {
+      Frag8 f;
+      f.u = *reinterpret_cast<const uint4*>(qp + c * 32);
+      if (!c_valid) f.u = make_uint4(0, 0, 0, 0);
+      qreg[c] = f.v;
+    }
+  }
+
+  float m_run = -INFINITY, l_run = 0.f;
+  float4v acc[DBL];
+#pragma unroll
+  for (int d = 0; d < DBL; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // loader: piece p of K is (group j, dim chunk i, key) = (p / (16*HD/8), (p/16) % (HD/8), p % 16);
+  // piece p of V is (group j, dim block, 16-byte piece of the 512-byte run)
+  uint4 kpre[KPT], vpre[VPT];
+  const int ps_shift = __ffs(ps) - 1;  // page sizes are powers of two here
+  auto fetch = [&](int s0) {
+    // the (up to four) pages of this stage; a group past the end reads the stage's first page
+    // (valid memory, masked later), so no load is predicated
+    const bf16_t* kbase[4];
+    const bf16_t* vbase[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c0 = (s0 + j * 16 <= last_pos) ? s0 + j * 16 : s0;
+      const size_t base = (size_t)table[c0 >> ps_shift] * page_elems + head_off;
+      const int off = c0 & (ps - 1);
+      kbase[j] = k_cache + base + (size_t)off * 8;
+      vbase[j] = v_cache + base + (size_t)(off >> 2) * 64;
+    }
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int p = i * THREADS + tid;
+      const int j = p / (16 * (HD / 8)), ci = (p / 16) % (HD / 8), key = p % 16;
+      kpre[i] = *reinterpret_cast<const uint4*>(kbase[j] + ((size_t)ci * ps + key) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int p = i * THREADS + tid;
+      const int j = p / (32 * (HD / 16)), db = (p / 32) % (HD / 16), w = p % 32;
+      vpre[i] = *reinterpret_cast<const uint4*>(vbase[j] + (size_t)db * (ps >> 2) * 64 + w * 8);
+    }
+  };
+
+  fetch(0);
+  for (int s0 = 0; s0 <= last_pos; s0 += 64) {
+    __syncthreads();  // every wave has read the previous stage
+#pragma unroll
+    for (int i = 0; i < KPT; ++i)
+      *reinterpret_cast<uint4*>(ks + (size_t)(i * THREADS + tid) * 8) = kpre[i];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+      *reinterpret_cast<uint4*>(vs + (size_t)(i * THREADS + tid) * 8) = vpre[i];
+    __syncthreads();
+    if (s0 + 64 <= last_pos) fetch(s0 + 64);
+
+    // S^T for 4 groups of 16 keys
+    float sv[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float4v sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < KCH; ++c) {
+        Frag8 kf;
+        kf.u = *reinterpret_cast<const uint4*>(ks + ((size_t)(j * (HD / 8) + c * 4 + kb) * 16 + col) * 8);
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[c], sc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sv[j][i] = sc[i] * scale_log2;
+    }
+    if (s0 + 63 > pos0) {  // some key of this stage is hidden from some column, or is past the end
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = s0 + j * 16 + kb * 4 + i;
+          if (key > c_pos || key > last_pos) sv[j][i] = -INFINITY;
+        }
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, sv[j][i]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    const float m_new = fmaxf(m_run, tmax);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);
+    m_run = m_new;
+    float psum = 0.f;
+    Frag8 pb[2];  // pb[h]: groups 2h and 2h+1, four probabilities each
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      float p[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[i] = fast_exp2(sv[2 * h][i] - m_safe);
+        p[4 + i] = fast_exp2(sv[2 * h + 1][i] - m_safe);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) psum += p[i];
+      pb[h].u = make_uint4((uint32_t)float_to_bf16(p[0]) | ((uint32_t)float_to_bf16(p[1]) << 16),
+                           (uint32_t)float_to_bf16(p[2]) | ((uint32_t)float_to_bf16(p[3]) << 16),
+                           (uint32_t)float_to_bf16(p[4]) | ((uint32_t)float_to_bf16(p[5]) << 16),
+                           (uint32_t)float_to_bf16(p[6]) | ((uint32_t)float_to_bf16(p[7]) << 16));
+    }
+    l_run = l_run * alpha + psum;
+    const bool tail = s0 + 63 > last_pos;  // keys past the end may hold anything: zero their values
+#pragma unroll
+    for (int d = 0; d < DBL; ++d) {
+      float4v a = acc[d];
+      a[0] *= alpha;
+      a[1] *= alpha;
+      a[2] *= alpha;
+      a[3] *= alpha;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        // A operand: V^T[dim col][k], k = (group 2h quad kb) then (group 2h+1 quad kb)
+        uint2 lo = *reinterpret_cast<const uint2*>(vs + ((size_t)((2 * h) * DBL + d) * 4 + kb) * 64 + col * 4);
+        uint2 hi = *reinterpret_cast<const uint2*>(vs + ((size_t)((2 * h + 1) * DBL + d) * 4 + kb) * 64 + col * 4);
+        if (tail) {
+          const int k0 = s0 + (2 * h) * 16 + kb * 4, k1 = k0 + 16;
+          if (k0 + 0 > last_pos) lo.x &= 0xffff0000u;
+          if (k0 + 1 > last_pos) lo.x &= 0x0000ffffu;
+          if (k0 + 2 > last_pos) lo.y &= 0xffff0000u;
+          if (k0 + 3 > last_pos) lo.y &= 0x0000ffffu;
+          if (k1 + 0 > last_pos) hi.x &= 0xffff0000u;
+          if (k1 + 1 > last_pos) hi.x &= 0x0000ffffu;
+          if (k1 + 2 > last_pos) hi.y &= 0xffff0000u;
+          if (k1 + 3 > last_pos) hi.y &= 0x0000ffffu;
+        }
+        Frag8 vf;
+        vf.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pb[h].v, a, 0, 0, 0);
+      }
+      acc[d] = a;
+    }
+  }
+
+  float l = l_run;
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  if (c_valid) {
+    const float inv = 1.f / l;
+    bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * HD + kb * 4;
+#pragma unroll
+    for (int d = 0; d < DBL; ++d) {
+      uint2 o;
+      o.x = (uint32_t)float_to_bf16(acc[d][0] * inv) | ((uint32_t)float_to_bf16(acc[d][1] * inv) << 16);
+      o.y = (uint32_t)float_to_bf16(acc[d][2] * inv) | ((uint32_t)float_to_bf16(acc[d][3] * inv) << 16);
+      *reinterpret_cast<uint2*>(op + d * 16) = o;
+    }
+  }
+}
+
+template <int HD, int HPB>
+static int launch_prefill(const void* q, const void* k_cache, const void* v_cache,
+                          const int* block_tables, int max_pages, const int* positions,
+                          const int* req_of_token, const int* item_token, const int* item_count,
+                          int num_items, void* out, int nh, int nkv, int ps, float scale,
+                          hipStream_t stream) {
+  const int G = nh / nkv;
+  dim3 grid(nkv * (G / HPB), num_items);
+  attention_prefill_kernel<HD, HPB><<<grid, 64 * HPB, 0, stream>>>(
+      (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
+      positions, req_of_token, item_token, item_count, (bf16_t*)out, num_items, nh, nkv, ps,
+      scale * 1.4426950408889634f);
+  return launch_status();
+}
+
 template <int HD, int NSETS, bool TOKENS>
 static int launch(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                   int max_pages, const int* positions, const int* req_of_token,
@@ -280,7 +503,7 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
                              int split_keys, int nh, int nkv, int hd, int ps, float scale,
                              hipStream_t stream) {
   if (num_items <= 0) return 0;
-  if (nkv <= 0 || nh % nkv != 0 || ps % 16 != 0 || split_keys % 16 != 0 || nsplit < 1) return -1;
+  if (nkv <= 0 || nh % nkv != 0 || ps < 16 || (ps & (ps - 1)) != 0 || split_keys % 16 != 0 || nsplit < 1) return -1;
   if (num_items > 65535 || nh > 65535) return -1;
   const int G = nh / nkv;
 #define TK_ARGS                                                                                   \
@@ -293,17 +516,21 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
     return -2;
   }
   if (nsplit != 1) return -1;
-  const int nsets = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
+  const int hpb = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
+#define TK_PARGS                                                                                  \
+  q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
+      num_items, out, nh, nkv, ps, scale, stream
   if (hd == 128) {
-    if (nsets == 4) return launch<128, 4, true>(TK_ARGS);
-    if (nsets == 2) return launch<128, 2, true>(TK_ARGS);
-    return launch<128, 1, true>(TK_ARGS);
+    if (hpb == 4) return launch_prefill<128, 4>(TK_PARGS);
+    if (hpb == 2) return launch_prefill<128, 2>(TK_PARGS);
+    return launch_prefill<128, 1>(TK_PARGS);
   }
   if (hd == 64) {
-    if (nsets == 4) return launch<64, 4, true>(TK_ARGS);
-    if (nsets == 2) return launch<64, 2, true>(TK_ARGS);
-    return launch<64, 1, true>(TK_ARGS);
+    if (hpb == 4) return launch_prefill<64, 4>(TK_PARGS);
+    if (hpb == 2) return launch_prefill<64, 2>(TK_PARGS);
+    return launch_prefill<64, 1>(TK_PARGS);
   }
+#undef TK_PARGS
 #undef TK_ARGS
   return -2;
 }

@@ -116,7 +116,11 @@ TK_API int tk_rope_tables(const int* positions, const float* inv_freq, float* co
 //   K page: [nkv][hd/8][ps][8]   (8 consecutive dims of one token are adjacent,
 //                                 then tokens, so lanes that hold consecutive
 //                                 tokens read consecutive 16-byte pieces)
-//   V page: [nkv][hd][ps]        (tokens of one dim adjacent)
+//   V page: [nkv][hd/16][ps/4][16][4]  (4 consecutive tokens of one dim adjacent,
+//                                 then 16 dims, then groups of 4 tokens: the A
+//                                 operand of the PV product, lane (dim, quad),
+//                                 is 8 contiguous bytes and a wave reads 512
+//                                 contiguous bytes)
 // One 64-lane block per (token, head).
 // ---------------------------------------------------------------------------
 constexpr int kMaxHeadDim = 512;
@@ -187,7 +191,8 @@ __global__ void qknorm_rope_store_kernel(
   } else {
     const int kvh = head - nh - nkv_in;
     T* base = v_cache + (size_t)page * page_elems + (size_t)kvh * hd * ps;
-    for (int d = lane; d < hd; d += kWave) Elem<T>::store(base + (size_t)d * ps + off, vec[d]);
+    for (int d = lane; d < hd; d += kWave)
+      Elem<T>::store(base + ((size_t)(d >> 4) * (ps >> 2) + (off >> 2)) * 64 + (d & 15) * 4 + (off & 3), vec[d]);
   }
 }
 
@@ -198,7 +203,7 @@ TK_API int tk_qknorm_rope_store(int dtype, const void* qkv, const float* q_weigh
                                 int N, int nh, int nkv_in, int nkv, int hd, int rot, int ps,
                                 int max_pages, float eps, hipStream_t stream) {
   if (N <= 0) return 0;
-  if (hd > kMaxHeadDim || hd % 8 != 0 || rot > hd || rot % 2 != 0) return -1;
+  if (hd > kMaxHeadDim || hd % 16 != 0 || ps % 4 != 0 || rot > hd || rot % 2 != 0) return -1;
   if (nkv_in != 0 && nkv_in != nkv) return -1;
   dim3 grid(N, nh + 2 * nkv_in);
   if (dtype == 0)

@@ -12,8 +12,8 @@ MAX_DECODE_WAVES = 8192   # above this, splits are made longer
 
 
 def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
-    return (dtype == torch.bfloat16 and head_dim in MFMA_HEAD_DIMS and page_size % 16 == 0
-            and group <= 16 and window is None)
+    return (dtype == torch.bfloat16 and head_dim in MFMA_HEAD_DIMS and page_size >= 16
+            and page_size & (page_size - 1) == 0 and group <= 16 and window is None)
 
 
 def decode_split(num_decode: int, num_kv_heads: int, max_len: int) -> tuple[int, int]:

@@ -168,7 +168,7 @@ def qknorm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor | None,
     width = (num_heads + 2 * nkv_in) * head_dim
     _need(qkv.shape[-1] == width and qkv.shape[0] >= n, f"qkv must be [N, {width}]")
     _need(q_out.dtype == qkv.dtype and q_out.numel() >= n * num_heads * head_dim, "q_out too small")
-    _need(head_dim % 8 == 0 and head_dim <= 512, "head_dim must be a multiple of 8, at most 512")
+    _need(head_dim % 16 == 0 and head_dim <= 512 and page_size % 8 == 0, "head_dim must be a multiple of 16 (at most 512), page_size a multiple of 8")
     _need(rotary_dim % 2 == 0 and rotary_dim <= head_dim, "rotary_dim must be even and <= head_dim")
     _need(cos.numel() >= n * (rotary_dim // 2) and sin.numel() >= n * (rotary_dim // 2), "rotary tables too small")
     for w in (q_weight, k_weight):
@@ -265,7 +265,7 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     n = positions.numel()
     _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "attention tensors must share a dtype")
     _need(q.numel() >= n * num_heads * head_dim and out.numel() >= n * num_heads * head_dim, "q/out too small")
-    _need(head_dim % 8 == 0 and head_dim <= 512, "head_dim must be a multiple of 8, at most 512")
+    _need(head_dim % 16 == 0 and head_dim <= 512 and page_size % 8 == 0, "head_dim must be a multiple of 16 (at most 512), page_size a multiple of 8")
     _need(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
     page_elems = num_kv_heads * head_dim * page_size
     _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
@@ -293,7 +293,8 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     _need(q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
           and out.dtype == torch.bfloat16, "the MFMA attention kernel takes bfloat16")
     _need(q.numel() >= n * num_heads * head_dim and out.numel() >= n * num_heads * head_dim, "q/out too small")
-    _need(num_heads % num_kv_heads == 0 and page_size % 16 == 0 and split_keys % 16 == 0, "bad head counts, page size or split")
+    _need(num_heads % num_kv_heads == 0 and page_size >= 16 and page_size & (page_size - 1) == 0
+          and split_keys % 16 == 0, "bad head counts, page size (a power of two >= 16) or split")
     page_elems = num_kv_heads * head_dim * page_size
     _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
     _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32 and block_tables.dtype == torch.int32

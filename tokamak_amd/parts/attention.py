@@ -31,8 +31,8 @@ class GQAAttention(Mixer):
         super().__init__(dtype=dtype, device=device)
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads ({num_heads}) must be divisible by num_kv_heads ({num_kv_heads})")
-        if head_dim % 8 or head_dim > 512:
-            raise ValueError(f"head_dim must be a multiple of 8 and at most 512, got {head_dim}")
+        if head_dim % 16 or head_dim > 512:
+            raise ValueError(f"head_dim must be a multiple of 16 and at most 512, got {head_dim}")
         self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
         self.head_dim = int(head_dim)
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
