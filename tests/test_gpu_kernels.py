@@ -295,3 +295,66 @@ def test_float32_product_is_true_32_bit_and_row_independent():
     whole = linear(big.to(DEV), wt.to(DEV)).cpu()
     one = linear(big[41:42].to(DEV), wt.to(DEV)).cpu()
     assert torch.equal(whole[41:42], one)
+
+
+@pytest.mark.parametrize("M, N, K", [(1, 64, 64), (8, 6144, 4096), (64, 4096, 4096), (33, 331, 200), (17, 4096, 12288), (64, 1000, 264)])
+def test_streaming_product_and_its_partial_sums(M, N, K):
+    """The LDS-staged weight-streaming kernel, unsplit and split over K: the
+    partial sums add up to the product, whoever adds them."""
+    from tokamak_amd.kernels import ops
+
+    x = rand(M, K, seed=1).to(torch.bfloat16)
+    w = rand(N, K, seed=2, scale=K ** -0.5).to(torch.bfloat16)
+    want = x.double() @ w.double().T
+    for out_dtype, tol in ((torch.float32, dict(rtol=1e-3, atol=1e-3)), (torch.bfloat16, dict(rtol=2e-2, atol=1e-2))):
+        out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+        assert ops.gemm_stream(x.to(DEV), w.to(DEV), out) == 1
+        torch.testing.assert_close(out.cpu().double(), want, **tol)
+    for splits in (2, 3, 8):
+        parts = torch.full((splits, M, N), float("nan"), device=DEV)
+        used = ops.gemm_stream(x.to(DEV), w.to(DEV), parts, splits=splits)
+        assert 1 <= used <= splits
+        torch.testing.assert_close(parts[:used].sum(0).cpu().double(), want, rtol=1e-3, atol=1e-3)
+        if used > 1:
+            assert parts[0].abs().max() > 0 and not torch.allclose(parts[0].cpu().double(), want, rtol=1e-2, atol=1e-2)
+
+
+def test_consumers_add_partial_sums():
+    """The norm kernel and the q/k norm kernel take a split-K product's partial
+    sums and add them in float32."""
+    from tokamak_amd.kernels import ops
+
+    M, H, P, eps = 5, 200, 3, 1e-5
+    resid, w = rand(M, H, seed=1), 1 + 0.1 * rand(H, seed=2)
+    parts = rand(P, M, H, seed=3)
+    total = parts.sum(0)
+    r = resid.to(DEV)
+    out = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
+    ops.add_rmsnorm(r, parts.to(DEV), w.to(DEV), eps, out)
+    torch.testing.assert_close(r.cpu(), resid + total, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(out.cpu().float(), plain.rmsnorm(resid + total, w, eps), **TOL[torch.bfloat16])
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, H, dtype=torch.bfloat16, device=DEV)
+    r2 = resid.to(DEV)
+    ops.add_rmsnorm(r2, parts.to(DEV), w.to(DEV), eps, out2, rows=rows, write_resid=False)
+    torch.testing.assert_close(out2.cpu().float(), plain.rmsnorm((resid + total)[[4, 1]], w, eps), **TOL[torch.bfloat16])
+
+    nh, nkv, hd, ps = 4, 2, 32, 16
+    batch = make_batch([(6, 3, [1, 0])])
+    N = 6
+    qkv_parts = rand(P, N, (nh + 2 * nkv) * hd, seed=4)
+    whole = qkv_parts.sum(0)
+    cos = torch.ones(N, hd // 2, device=DEV)
+    sin = torch.zeros(N, hd // 2, device=DEV)
+    outs = []
+    for inp in (qkv_parts, whole):
+        k_cache = torch.zeros(2, nkv * hd * ps, dtype=torch.bfloat16, device=DEV)
+        v_cache = torch.zeros_like(k_cache)
+        q_out = torch.empty(N, nh * hd, dtype=torch.bfloat16, device=DEV)
+        ops.qknorm_rope_store(inp.to(DEV), torch.ones(hd, device=DEV), torch.ones(hd, device=DEV), cos, sin,
+                              batch.positions, batch.req_of_token, batch.block_tables[0], q_out, k_cache, v_cache,
+                              num_heads=nh, num_kv_heads=nkv, head_dim=hd, rotary_dim=hd, page_size=ps, eps=eps)
+        outs.append((q_out.cpu(), k_cache.cpu(), v_cache.cpu()))
+    for a, b in zip(*outs):
+        torch.testing.assert_close(a.float(), b.float(), rtol=1e-2, atol=1e-2)
+    assert outs[0][2].abs().max() > 0

@@ -26,6 +26,7 @@ using namespace tk;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 union Frag8 {
   uint4 u;
@@ -317,46 +318,53 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
 
   // loader: piece p of K is (group j, dim chunk i, key) = (p / (16*HD/8), (p/16) % (HD/8), p % 16);
   // piece p of V is (group j, dim block, 16-byte piece of the 512-byte run)
-  uint4 kpre[KPT], vpre[VPT];
+  u32x4 kpre[KPT], vpre[VPT];
   const int ps_shift = __ffs(ps) - 1;  // page sizes are powers of two here
-  auto fetch = [&](int s0) {
-    // the (up to four) pages of this stage; a group past the end reads the stage's first page
-    // (valid memory, masked later), so no load is predicated
-    const bf16_t* kbase[4];
-    const bf16_t* vbase[4];
+  // Piece p of a stage belongs to 16-key group j = p / pieces-per-group.  A group past
+  // the request's end reads the stage's first group instead (valid memory, masked
+  // later), so no load is predicated and all of a stage's loads are in flight together.
+  int k_j[KPT], k_in[KPT], v_j[VPT], v_in[VPT];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int c0 = (s0 + j * 16 <= last_pos) ? s0 + j * 16 : s0;
-      const size_t base = (size_t)table[c0 >> ps_shift] * page_elems + head_off;
-      const int off = c0 & (ps - 1);
-      kbase[j] = k_cache + base + (size_t)off * 8;
-      vbase[j] = v_cache + base + (size_t)(off >> 2) * 64;
-    }
+  for (int i = 0; i < KPT; ++i) {
+    const int p = i * THREADS + tid;
+    k_j[i] = p / (16 * (HD / 8));
+    k_in[i] = (((p / 16) % (HD / 8)) * ps + (p % 16)) * 8;  // element offset inside the page's head
+  }
 #pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int p = i * THREADS + tid;
-      const int j = p / (16 * (HD / 8)), ci = (p / 16) % (HD / 8), key = p % 16;
-      kpre[i] = *reinterpret_cast<const uint4*>(kbase[j] + ((size_t)ci * ps + key) * 8);
-    }
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const int p = i * THREADS + tid;
-      const int j = p / (32 * (HD / 16)), db = (p / 32) % (HD / 16), w = p % 32;
-      vpre[i] = *reinterpret_cast<const uint4*>(vbase[j] + (size_t)db * (ps >> 2) * 64 + w * 8);
-    }
-  };
+  for (int i = 0; i < VPT; ++i) {
+    const int p = i * THREADS + tid;
+    v_j[i] = p / (32 * (HD / 16));
+    v_in[i] = ((p / 32) % (HD / 16)) * (ps >> 2) * 64 + (p % 32) * 8;
+  }
+#define TK_FETCH(S0)                                                                              \
+  {                                                                                               \
+    _Pragma("unroll") for (int i = 0; i < KPT; ++i) {                                             \
+      int c0 = (S0) + k_j[i] * 16;                                                                \
+      c0 = (c0 <= last_pos) ? c0 : (S0);                                                          \
+      const size_t base = (size_t)table[c0 >> ps_shift] * page_elems + head_off;                  \
+      kpre[i] = *reinterpret_cast<const u32x4*>(k_cache + base + (size_t)(c0 & (ps - 1)) * 8 +    \
+                                                k_in[i]);                                         \
+    }                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < VPT; ++i) {                                             \
+      int c0 = (S0) + v_j[i] * 16;                                                                \
+      c0 = (c0 <= last_pos) ? c0 : (S0);                                                          \
+      const size_t base = (size_t)table[c0 >> ps_shift] * page_elems + head_off;                  \
+      vpre[i] = *reinterpret_cast<const u32x4*>(v_cache + base +                                  \
+                                                (size_t)((c0 & (ps - 1)) >> 2) * 64 + v_in[i]);   \
+    }                                                                                             \
+  }
 
-  fetch(0);
+  TK_FETCH(0)
   for (int s0 = 0; s0 <= last_pos; s0 += 64) {
     __syncthreads();  // every wave has read the previous stage
 #pragma unroll
     for (int i = 0; i < KPT; ++i)
-      *reinterpret_cast<uint4*>(ks + (size_t)(i * THREADS + tid) * 8) = kpre[i];
+      *reinterpret_cast<u32x4*>(ks + (size_t)(i * THREADS + tid) * 8) = kpre[i];
 #pragma unroll
     for (int i = 0; i < VPT; ++i)
-      *reinterpret_cast<uint4*>(vs + (size_t)(i * THREADS + tid) * 8) = vpre[i];
+      *reinterpret_cast<u32x4*>(vs + (size_t)(i * THREADS + tid) * 8) = vpre[i];
     __syncthreads();
-    if (s0 + 64 <= last_pos) fetch(s0 + 64);
+    if (s0 + 64 <= last_pos) TK_FETCH(s0 + 64)
 
     // S^T for 4 groups of 16 keys
     float sv[4][4];
@@ -425,14 +433,10 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
         uint2 hi = *reinterpret_cast<const uint2*>(vs + ((size_t)((2 * h + 1) * DBL + d) * 4 + kb) * 64 + col * 4);
         if (tail) {
           const int k0 = s0 + (2 * h) * 16 + kb * 4, k1 = k0 + 16;
-          if (k0 + 0 > last_pos) lo.x &= 0xffff0000u;
-          if (k0 + 1 > last_pos) lo.x &= 0x0000ffffu;
-          if (k0 + 2 > last_pos) lo.y &= 0xffff0000u;
-          if (k0 + 3 > last_pos) lo.y &= 0x0000ffffu;
-          if (k1 + 0 > last_pos) hi.x &= 0xffff0000u;
-          if (k1 + 1 > last_pos) hi.x &= 0x0000ffffu;
-          if (k1 + 2 > last_pos) hi.y &= 0xffff0000u;
-          if (k1 + 3 > last_pos) hi.y &= 0x0000ffffu;
+          lo.x &= (k0 + 0 > last_pos ? 0u : 0x0000ffffu) | (k0 + 1 > last_pos ? 0u : 0xffff0000u);
+          lo.y &= (k0 + 2 > last_pos ? 0u : 0x0000ffffu) | (k0 + 3 > last_pos ? 0u : 0xffff0000u);
+          hi.x &= (k1 + 0 > last_pos ? 0u : 0x0000ffffu) | (k1 + 1 > last_pos ? 0u : 0xffff0000u);
+          hi.y &= (k1 + 2 > last_pos ? 0u : 0x0000ffffu) | (k1 + 3 > last_pos ? 0u : 0xffff0000u);
         }
         Frag8 vf;
         vf.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
@@ -457,6 +461,8 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
     }
   }
 }
+
+#undef TK_FETCH
 
 template <int HD, int HPB>
 static int launch_prefill(const void* q, const void* k_cache, const void* v_cache,

@@ -40,20 +40,23 @@ TK_API int tk_embed_gather(int dtype, const void* table, const int* ids, float* 
 // row = rows ? rows[m] : m.  With `rows`, write_resid must be 0 (a row could be
 // named twice).
 // ---------------------------------------------------------------------------
-template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta,
-                                   const int* __restrict__ rows, const float* __restrict__ weight,
-                                   T* __restrict__ out, int H, float eps, int write_resid) {
+// delta may come as `parts` float32 partial sums, part_stride elements apart
+// (a split-K product's output): they are added in order.
+template <typename T, typename TD>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                                   int parts, long part_stride, const int* __restrict__ rows,
+                                   const float* __restrict__ weight, T* __restrict__ out, int H,
+                                   float eps, int write_resid) {
   __shared__ float scratch[16];
   const int m = blockIdx.x;
   const size_t row = rows ? (size_t)rows[m] : (size_t)m;
   float* x = resid + row * H;
-  const T* dl = delta ? delta + row * H : nullptr;
+  const TD* dl = delta ? delta + row * H : nullptr;
   float ss = 0.f;
   for (int d = threadIdx.x; d < H; d += blockDim.x) {
     float v = x[d];
     if (dl) {
-      v += Elem<T>::load(dl + d);
+      for (int p = 0; p < parts; ++p) v += Elem<TD>::load(dl + (size_t)p * part_stride + d);
       if (write_resid) x[d] = v;
     }
     ss += v * v;
@@ -63,22 +66,31 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
   T* o = out + (size_t)m * H;
   for (int d = threadIdx.x; d < H; d += blockDim.x) {
     float v = x[d];
-    if (dl && !write_resid) v += Elem<T>::load(dl + d);
+    if (dl && !write_resid)
+      for (int p = 0; p < parts; ++p) v += Elem<TD>::load(dl + (size_t)p * part_stride + d);
     Elem<T>::store(o + d, v * rstd * weight[d]);
   }
 }
 
-TK_API int tk_add_rmsnorm(int dtype, float* resid, const void* delta, const int* rows,
-                          const float* weight, void* out, int M, int H, float eps, int write_resid,
-                          hipStream_t stream) {
+// delta_f32: delta is float32 (possibly `parts` partial sums) whatever the dtype
+TK_API int tk_add_rmsnorm(int dtype, float* resid, const void* delta, int delta_f32, int parts,
+                          long part_stride, const int* rows, const float* weight, void* out, int M,
+                          int H, float eps, int write_resid, hipStream_t stream) {
   if (M <= 0) return 0;
   if (rows && write_resid) return -1;
+  if (parts < 1 || (parts > 1 && !delta_f32 && dtype != 0)) return -1;
   if (dtype == 0)
-    add_rmsnorm_kernel<float><<<M, 256, 0, stream>>>(resid, (const float*)delta, rows, weight,
-                                                     (float*)out, H, eps, write_resid);
+    add_rmsnorm_kernel<float, float><<<M, 256, 0, stream>>>(resid, (const float*)delta, parts,
+                                                            part_stride, rows, weight, (float*)out,
+                                                            H, eps, write_resid);
+  else if (delta_f32)
+    add_rmsnorm_kernel<bf16_t, float><<<M, 256, 0, stream>>>(resid, (const float*)delta, parts,
+                                                             part_stride, rows, weight,
+                                                             (bf16_t*)out, H, eps, write_resid);
   else
-    add_rmsnorm_kernel<bf16_t><<<M, 256, 0, stream>>>(resid, (const bf16_t*)delta, rows, weight,
-                                                      (bf16_t*)out, H, eps, write_resid);
+    add_rmsnorm_kernel<bf16_t, bf16_t><<<M, 256, 0, stream>>>(resid, (const bf16_t*)delta, parts,
+                                                              part_stride, rows, weight,
+                                                              (bf16_t*)out, H, eps, write_resid);
   return launch_status();
 }
 
@@ -125,9 +137,10 @@ TK_API int tk_rope_tables(const int* positions, const float* inv_freq, float* co
 // ---------------------------------------------------------------------------
 constexpr int kMaxHeadDim = 512;
 
-template <typename T>
+template <typename T, typename TIN>
 __global__ void qknorm_rope_store_kernel(
-    const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+    const TIN* __restrict__ qkv, int parts, long part_stride, const float* __restrict__ q_weight,
+    const float* __restrict__ k_weight,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ block_tables, T* __restrict__ q_out, T* __restrict__ k_cache,
@@ -136,14 +149,15 @@ __global__ void qknorm_rope_store_kernel(
   __shared__ float vec[kMaxHeadDim];
   const int n = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int row_width = (nh + 2 * nkv_in) * hd;
-  const T* src = qkv + (size_t)n * row_width + (size_t)head * hd;
+  const TIN* src = qkv + (size_t)n * row_width + (size_t)head * hd;
   const bool is_q = head < nh;
   const bool is_k = !is_q && head < nh + nkv_in;
   const float* w = is_q ? q_weight : (is_k ? k_weight : nullptr);
 
   float ss = 0.f;
   for (int d = lane; d < hd; d += kWave) {
-    const float v = Elem<T>::load(src + d);
+    float v = 0.f;
+    for (int p = 0; p < parts; ++p) v += Elem<TIN>::load(src + (size_t)p * part_stride + d);
     vec[d] = v;
     ss += v * v;
   }
@@ -196,26 +210,27 @@ __global__ void qknorm_rope_store_kernel(
   }
 }
 
-TK_API int tk_qknorm_rope_store(int dtype, const void* qkv, const float* q_weight,
-                                const float* k_weight, const float* cos_t, const float* sin_t,
-                                const int* positions, const int* req_of_token,
+// in_f32: qkv is float32 (possibly `parts` partial sums, part_stride elements apart)
+TK_API int tk_qknorm_rope_store(int dtype, const void* qkv, int in_f32, int parts, long part_stride,
+                                const float* q_weight, const float* k_weight, const float* cos_t,
+                                const float* sin_t, const int* positions, const int* req_of_token,
                                 const int* block_tables, void* q_out, void* k_cache, void* v_cache,
                                 int N, int nh, int nkv_in, int nkv, int hd, int rot, int ps,
                                 int max_pages, float eps, hipStream_t stream) {
   if (N <= 0) return 0;
   if (hd > kMaxHeadDim || hd % 16 != 0 || ps % 4 != 0 || rot > hd || rot % 2 != 0) return -1;
   if (nkv_in != 0 && nkv_in != nkv) return -1;
+  if (parts < 1 || (parts > 1 && !in_f32 && dtype != 0)) return -1;
   dim3 grid(N, nh + 2 * nkv_in);
-  if (dtype == 0)
-    qknorm_rope_store_kernel<float><<<grid, kWave, 0, stream>>>(
-        (const float*)qkv, q_weight, k_weight, cos_t, sin_t, positions, req_of_token, block_tables,
-        (float*)q_out, (float*)k_cache, (float*)v_cache, nh, nkv_in, nkv, hd, rot, ps, max_pages,
-        eps);
-  else
-    qknorm_rope_store_kernel<bf16_t><<<grid, kWave, 0, stream>>>(
-        (const bf16_t*)qkv, q_weight, k_weight, cos_t, sin_t, positions, req_of_token, block_tables,
-        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv_in, nkv, hd, rot, ps, max_pages,
-        eps);
+#define TK_QK(T_, TIN_)                                                                          \
+  qknorm_rope_store_kernel<T_, TIN_><<<grid, kWave, 0, stream>>>(                                \
+      (const TIN_*)qkv, parts, part_stride, q_weight, k_weight, cos_t, sin_t, positions,         \
+      req_of_token, block_tables, (T_*)q_out, (T_*)k_cache, (T_*)v_cache, nh, nkv_in, nkv, hd,   \
+      rot, ps, max_pages, eps)
+  if (dtype == 0) TK_QK(float, float);
+  else if (in_f32) TK_QK(bf16_t, float);
+  else TK_QK(bf16_t, bf16_t);
+#undef TK_QK
   return launch_status();
 }
 

@@ -19,6 +19,7 @@ using namespace tk;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // arrays of HIP's uint4 struct end up in scratch
 
 union Frag8 {
   uint4 u;
@@ -211,10 +212,9 @@ TK_API int tk_gemm_skinny(int out_dtype, const void* A, const void* W, void* C, 
 //   * each wave then reads MFMA fragments back from LDS: lane (r, kb) takes
 //     W[row r][k + kb*8 .. +8] as A operand and X[row r][same k] as B operand of
 //     v_mfma_f32_16x16x32_bf16 and accumulates D[weight row][batch row].
-// With KS > 1 every block writes its partial tile to a workspace and bumps a
-// counter of its row block; the block that arrives last adds all KS partials in
-// split order (so the sum does not depend on arrival order), writes C and
-// resets the counter.  Nothing spins or waits on another block.
+// With KS > 1 split s writes float32 partial sums to its own copy of C; the kernel
+// that reads C next (residual add + norm, or the q/k norm + rotation kernel) adds
+// the copies in split order.  No block waits for, or signals, another.
 // ---------------------------------------------------------------------------
 constexpr int SBK = 256;        // k per chunk
 constexpr int SLD = SBK + 8;    // LDS row stride in elements
@@ -222,11 +222,9 @@ constexpr int SLD = SBK + 8;    // LDS row stride in elements
 template <int MT, typename TO>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TO* __restrict__ C, int M, int N,
-    int K, long lda, long ldw, long ldc, int chunks_per_split, int KS, float* __restrict__ partial,
-    int* __restrict__ counters) {
+    int K, long lda, long ldw, long ldc, int chunks_per_split, long split_stride) {
   __shared__ __attribute__((aligned(16))) bf16_t ws[4][16][SLD];
   __shared__ __attribute__((aligned(16))) bf16_t xs[16 * MT][SLD];
-  __shared__ int last_flag;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, kb = lane >> 4;
   const int row_block = blockIdx.x, split = blockIdx.y;
@@ -240,9 +238,9 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
   // X pieces of this thread: piece p = i*256 + tid -> row p/32, column p%32
   const int x_col = (tid & 31) * 8, x_row0 = tid >> 5;
 
-  uint4 wreg[8];
-  uint4 xreg[2 * MT];
-  const uint4 zero = make_uint4(0, 0, 0, 0);
+  u32x4 wreg[8];
+  u32x4 xreg[2 * MT];
+  const u32x4 zero = {0u, 0u, 0u, 0u};
   // Rows are clamped into the matrices (rows past N or M are computed from a valid
   // row and never stored); only a piece past K is zeroed, after an unconditional
   // load from k = 0, so the loads of a chunk are all in flight together.
@@ -257,9 +255,9 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
     const bool kw = k0 + w_col < K, kx = k0 + x_col < K;
     const int wo = kw ? k0 + w_col : 0, xo = kx ? k0 + x_col : 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) wreg[i] = *reinterpret_cast<const uint4*>(wrow[i] + wo);
+    for (int i = 0; i < 8; ++i) wreg[i] = *reinterpret_cast<const u32x4*>(wrow[i] + wo);
 #pragma unroll
-    for (int i = 0; i < 2 * MT; ++i) xreg[i] = *reinterpret_cast<const uint4*>(xrow[i] + xo);
+    for (int i = 0; i < 2 * MT; ++i) xreg[i] = *reinterpret_cast<const u32x4*>(xrow[i] + xo);
     if (k0 + SBK > K) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) wreg[i] = kw ? wreg[i] : zero;
@@ -277,10 +275,10 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
     __syncthreads();  // the previous chunk's fragments have been read
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      *reinterpret_cast<uint4*>(&ws[wave][2 * i + w_row0][w_col]) = wreg[i];
+      *reinterpret_cast<u32x4*>(&ws[wave][2 * i + w_row0][w_col]) = wreg[i];
 #pragma unroll
     for (int i = 0; i < 2 * MT; ++i)
-      *reinterpret_cast<uint4*>(&xs[i * 8 + x_row0][x_col]) = xreg[i];
+      *reinterpret_cast<u32x4*>(&xs[i * 8 + x_row0][x_col]) = xreg[i];
     __syncthreads();
     if (c + 1 < c_end) fetch(c + 1);  // in flight while this chunk is multiplied
 #pragma unroll
@@ -296,35 +294,9 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
     }
   }
 
-  if (KS > 1) {
-    // partial tiles are stored in accumulator layout: [split][row block][wave][j][lane][4]
-    const size_t tile = (size_t)4 * MT * 256;
-    float* mine = partial + ((size_t)split * gridDim.x + row_block) * tile + (size_t)(wave * MT) * 256;
-#pragma unroll
-    for (int j = 0; j < MT; ++j)
-      *reinterpret_cast<float4*>(mine + j * 256 + lane * 4) =
-          make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) last_flag = (atomicAdd(&counters[row_block], 1) == KS - 1);
-    __syncthreads();
-    if (!last_flag) return;
-    __threadfence();
-#pragma unroll
-    for (int j = 0; j < MT; ++j) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < KS; ++s) {
-      const float* src = partial + ((size_t)s * gridDim.x + row_block) * tile + (size_t)(wave * MT) * 256;
-#pragma unroll
-      for (int j = 0; j < MT; ++j) {
-        const float4 v = *reinterpret_cast<const float4*>(src + j * 256 + lane * 4);
-        acc[j][0] += v.x;
-        acc[j][1] += v.y;
-        acc[j][2] += v.z;
-        acc[j][3] += v.w;
-      }
-    }
-    if (tid == 0) counters[row_block] = 0;  // ready for the next product on this stream
-  }
+  // With several splits, split s writes its partial sums to C + s * split_stride; whoever
+  // reads C next adds the splits (in split order, so the sum is deterministic).
+  C += (size_t)split * split_stride;
 
   // acc[j][e] = C[batch row j*16 + r][weight row n_wave + kb*4 + e]
 #pragma unroll
@@ -341,17 +313,14 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
 
 template <typename TO>
 static int launch_stream(const void* A, const void* W, void* C, int M, int N, int K, long lda,
-                         long ldw, long ldc, int KS, float* partial, int* counters,
+                         long ldw, long ldc, int chunks_per_split, int KS, long split_stride,
                          hipStream_t stream) {
-  const int total_chunks = (K + SBK - 1) / SBK;
-  const int cps = (total_chunks + KS - 1) / KS;
-  KS = (total_chunks + cps - 1) / cps;  // no empty splits
   dim3 grid((N + 63) / 64, KS);
   const int mt = (M + 15) / 16;
-#define TK_STREAM(MT_)                                                                           \
-  gemm_stream_kernel<MT_, TO><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W,     \
-                                                        (TO*)C, M, N, K, lda, ldw, ldc, cps, KS, \
-                                                        partial, counters)
+#define TK_STREAM(MT_)                                                                        \
+  gemm_stream_kernel<MT_, TO><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W,  \
+                                                        (TO*)C, M, N, K, lda, ldw, ldc,      \
+                                                        chunks_per_split, split_stride)
   if (mt == 1) TK_STREAM(1);
   else if (mt == 2) TK_STREAM(2);
   else if (mt == 3) TK_STREAM(3);
@@ -361,17 +330,20 @@ static int launch_stream(const void* A, const void* W, void* C, int M, int N, in
 }
 
 // out_dtype: 0 float32, 1 bfloat16.  M <= 64; K a multiple of 8; rows 16-byte aligned.
-// splits: shares of K (>= 1).  With splits > 1, `partial` must hold
-// splits * ceil(N/64) * 4 * ceil(M/16) * 256 floats and `counters` ceil(N/64) ints
-// that are zero before the first call (the kernel leaves them zero).
+// splits: shares of K.  With splits > 1 the output must be float32 and C holds
+// `splits` partial results, split_stride elements apart, that the reader adds.
+// Returns the number of splits actually used (<= splits; no split is empty), or < 0.
 TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, int M, int N, int K,
-                          long lda, long ldw, long ldc, int splits, float* partial, int* counters,
+                          long lda, long ldw, long ldc, int splits, long split_stride,
                           hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1) return -1;
-  if (splits > 1 && (!partial || !counters)) return -1;
-  if ((N + 63) / 64 > 0x7fffffff / 2 || splits > 65535) return -1;
-  if (out_dtype == 0) return launch_stream<float>(A, W, C, M, N, K, lda, ldw, ldc, splits, partial, counters, stream);
-  if (out_dtype == 1) return launch_stream<bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, splits, partial, counters, stream);
-  return -1;
+  if (M > 64 || K <= 0 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535) return -1;
+  if (splits > 1 && out_dtype != 0) return -1;
+  const int total_chunks = (K + SBK - 1) / SBK;
+  const int cps = (total_chunks + splits - 1) / splits;
+  const int ks = (total_chunks + cps - 1) / cps;
+  int status = -1;
+  if (out_dtype == 0) status = launch_stream<float>(A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
+  if (out_dtype == 1) status = launch_stream<bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
+  return status == 0 ? ks : (status > 0 ? -status : status);
 }

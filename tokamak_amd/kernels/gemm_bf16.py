@@ -7,7 +7,9 @@ import torch
 from tokamak_amd.kernels import ops
 
 SKINNY_MAX_ROWS = 64
-TARGET_WAVES = 4096   # waves wanted in flight for a weight-streaming product
+TARGET_WAVES = 4096     # waves wanted in flight for the direct-operand kernel
+STREAM_MIN_ROWS_OUT = 1024    # weight rows from which the LDS-staged kernel (64 rows a block) is used
+STREAM_TARGET_BLOCKS = 512
 
 
 def skinny_fits(x: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -17,12 +19,10 @@ def skinny_fits(x: torch.Tensor, weight: torch.Tensor) -> bool:
 
 
 def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
-    """(tiles of 16 weight rows per block, waves of a block that split K).
-
-    More row tiles per block let the activation fragments be reused; more waves
-    put more loads in flight when the matrix has few rows.  Chosen from
-    measurements on the projection shapes of 0.6B to 32B models.
-    """
+    """(tiles of 16 weight rows per block, waves of a block that split K) for the
+    direct-operand kernel.  More row tiles per block let the activation fragments
+    be reused; more waves put more loads in flight when the matrix has few rows.
+    Chosen from measurements on the projection shapes of 0.6B to 32B models."""
     if m > 32:
         row_tiles = 4 if n >= 6144 else 2
     elif m <= 2 or n < 6144:
@@ -38,22 +38,46 @@ def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
     return row_tiles, waves
 
 
-def gemm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
-    """out[M, N] = x[M, K] @ weight[N, K]^T; out is bfloat16 or float32.
+def stream_splits(n: int, k: int) -> int:
+    """Shares of K for the LDS-staged kernel so that enough blocks exist."""
+    blocks = -(-n // 64)
+    chunks = -(-k // 256)
+    return max(1, min(chunks // 2, -(-STREAM_TARGET_BLOCKS // blocks), 64))
 
-    Up to 64 rows (decode batches, wanted logits rows): the hand-written
-    weight-streaming MFMA kernel.  More rows with bfloat16 output: the library
-    product torch binds (as the reference's nn.Linear does).  More rows with
-    float32 output (many wanted logits rows): the skinny kernel, 64 rows at a time.
+
+def gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype, allow_partials: bool = False) -> torch.Tensor:
+    """x[M, K] @ weight[N, K]^T -> [M, N] in ``out_dtype``; or, if the caller can
+    add them (``allow_partials``), float32 partial sums [P, M, N] of a split-K product.
+
+    Up to 64 rows (decode batches, wanted logits rows): hand-written
+    weight-streaming MFMA kernels: the LDS-staged one, split over K into partial
+    sums when the matrix has few rows and the caller adds them; the
+    direct-operand one for very small matrices.  More than 64 rows
+    with bfloat16 output: the library product torch binds (as the reference's
+    nn.Linear does); with float32 output: 64 rows at a time.
     """
     m = x.shape[0]
     n, k = weight.shape
-    if skinny_fits(x, weight) and (m <= SKINNY_MAX_ROWS or out.dtype == torch.float32):
-        row_tiles, waves = skinny_plan(min(m, SKINNY_MAX_ROWS), n, k)
+    dev = x.device
+    if skinny_fits(x, weight) and (m <= SKINNY_MAX_ROWS or out_dtype == torch.float32):
+        if m <= SKINNY_MAX_ROWS and allow_partials:
+            splits = stream_splits(n, k)
+            if splits > 1:
+                out = torch.empty((splits, m, n), dtype=torch.float32, device=dev)
+                used = ops.gemm_stream(x, weight, out, splits=splits)
+                return out[:used]
+        out = torch.empty((m, n), dtype=out_dtype, device=dev)
         for at in range(0, m, SKINNY_MAX_ROWS):
-            ops.gemm_skinny(x[at:at + SKINNY_MAX_ROWS], weight, out[at:at + SKINNY_MAX_ROWS],
-                            row_tiles=row_tiles, waves=waves)
-    elif out.dtype == torch.bfloat16:
+            xs, os_ = x[at:at + SKINNY_MAX_ROWS], out[at:at + SKINNY_MAX_ROWS]
+            if n >= STREAM_MIN_ROWS_OUT:
+                ops.gemm_stream(xs, weight, os_)
+            else:
+                row_tiles, waves = skinny_plan(xs.shape[0], n, k)
+                ops.gemm_skinny(xs, weight, os_, row_tiles=row_tiles, waves=waves)
+        return out
+    out = torch.empty((m, n), dtype=out_dtype, device=dev)
+    if out_dtype == torch.bfloat16:
         torch.matmul(x, weight.t(), out=out)
     else:
         ops.gemm_tiled(x, weight, out)
+    return out

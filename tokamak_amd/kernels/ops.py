@@ -58,10 +58,10 @@ def _check(status: int, name: str) -> None:
 _SIGS = {
     "elementwise": {
         "tk_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
-        "tk_add_rmsnorm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                           c_float, c_int, c_void_p],
+        "tk_add_rmsnorm": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p,
+                           c_void_p, c_int, c_int, c_float, c_int, c_void_p],
         "tk_rope_tables": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
-        "tk_qknorm_rope_store": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        "tk_qknorm_rope_store": [c_int, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
         "tk_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -72,7 +72,7 @@ _SIGS = {
     },
     "gemm_mfma": {
         "tk_gemm_stream": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
-                           c_long, c_int, c_void_p, c_void_p, c_void_p],
+                           c_long, c_int, c_long, c_void_p],
         "tk_gemm_skinny": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                            c_long, c_int, c_int, c_void_p],
     },
@@ -121,10 +121,26 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, resid: torch.Tensor) ->
                                                  n, h, v, _stream()), "embed_gather")
 
 
+def _partials(t: torch.Tensor | None, rows: int, width: int, dtype: torch.dtype, what: str):
+    """(is_f32, parts, part_stride) of an input that is either [rows, width] in
+    ``dtype`` or float32 partial sums [parts, rows, width] (a split-K product)."""
+    if t is None:
+        return 0, 1, 0
+    if t.dim() == 3:
+        _need(t.dtype == torch.float32 and t.shape[1] >= rows and t.shape[2] == width, f"{what}: partial sums must be float32 [parts, rows, {width}]")
+        return 1, t.shape[0], t.stride(0)
+    _need(t.dim() == 2 and t.shape[1] == width and t.shape[0] >= rows, f"{what} must be [rows, {width}]")
+    if t.dtype == torch.float32:
+        return 1, 1, 0
+    _need(t.dtype == dtype, f"{what} must be float32 or the compute dtype")
+    return 0, 1, 0
+
+
 def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float,
                 out: torch.Tensor, rows: torch.Tensor | None = None,
                 write_resid: bool = True) -> None:
-    """x = resid[row] (+ delta[row]); optionally stored back; out = rmsnorm(x) * weight."""
+    """x = resid[row] (+ delta[row]); optionally stored back; out = rmsnorm(x) * weight.
+    ``delta``: [M, H] in the compute dtype or float32, or float32 partial sums [P, M, H]."""
     _gpu(resid, delta, weight, out, rows)
     h = resid.shape[-1]
     m = out.shape[0] if rows is None else rows.numel()
@@ -136,10 +152,9 @@ def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.T
         _need(rows.dtype == torch.int32 and not (write_resid and delta is not None),
               "row-indexed rmsnorm cannot write the residual")
         write_resid = False
-    if delta is not None:
-        _need(delta.dtype == out.dtype and delta.shape == resid.shape, "delta must match the residual's shape")
-    _check(_fn("elementwise", "tk_add_rmsnorm")(_code(out.dtype), _p(resid), _p(delta), _p(rows),
-                                                _p(weight), _p(out), m, h, float(eps),
+    is_f32, parts, stride = _partials(delta, resid.shape[0], h, out.dtype, "delta")
+    _check(_fn("elementwise", "tk_add_rmsnorm")(_code(out.dtype), _p(resid), _p(delta), is_f32, parts, stride,
+                                                _p(rows), _p(weight), _p(out), m, h, float(eps),
                                                 int(bool(write_resid)), _stream()), "add_rmsnorm")
 
 
@@ -166,8 +181,8 @@ def qknorm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor | None,
     n = positions.numel()
     nkv_in = num_kv_heads if store else 0
     width = (num_heads + 2 * nkv_in) * head_dim
-    _need(qkv.shape[-1] == width and qkv.shape[0] >= n, f"qkv must be [N, {width}]")
-    _need(q_out.dtype == qkv.dtype and q_out.numel() >= n * num_heads * head_dim, "q_out too small")
+    in_f32, parts, stride = _partials(qkv, n, width, q_out.dtype, "qkv")
+    _need(q_out.numel() >= n * num_heads * head_dim, "q_out too small")
     _need(head_dim % 16 == 0 and head_dim <= 512 and page_size % 8 == 0, "head_dim must be a multiple of 16 (at most 512), page_size a multiple of 8")
     _need(rotary_dim % 2 == 0 and rotary_dim <= head_dim, "rotary_dim must be even and <= head_dim")
     _need(cos.numel() >= n * (rotary_dim // 2) and sin.numel() >= n * (rotary_dim // 2), "rotary tables too small")
@@ -179,11 +194,11 @@ def qknorm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor | None,
     max_pages = block_tables.shape[1]
     if store:
         page_elems = num_kv_heads * head_dim * page_size
-        _need(k_cache is not None and v_cache is not None and k_cache.dtype == qkv.dtype
-              and v_cache.dtype == qkv.dtype, "cache dtype must match activations")
+        _need(k_cache is not None and v_cache is not None and k_cache.dtype == q_out.dtype
+              and v_cache.dtype == q_out.dtype, "cache dtype must match activations")
         _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
     _check(_fn("elementwise", "tk_qknorm_rope_store")(
-        _code(qkv.dtype), _p(qkv), _p(q_weight), _p(k_weight), _p(cos), _p(sin), _p(positions),
+        _code(q_out.dtype), _p(qkv), in_f32, parts, stride, _p(q_weight), _p(k_weight), _p(cos), _p(sin), _p(positions),
         _p(req_of_token), _p(block_tables), _p(q_out), _p(k_cache), _p(v_cache), n, num_heads,
         nkv_in, num_kv_heads, head_dim, rotary_dim, page_size, max_pages, float(eps), _stream()),
         "qknorm_rope_store")
@@ -212,30 +227,32 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
                                               _stream()), "gemm_tiled")
 
 
-def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: int,
-                partial: torch.Tensor | None, counters: torch.Tensor | None) -> None:
-    """out[M, N] = a[M, K] @ w[N, K]^T for M <= 64 with the weight-streaming MFMA
-    kernel.  ``splits`` shares of K; with more than one, ``partial`` (float32) and
-    ``counters`` (int32, all zero) are the workspace the blocks meet in."""
-    for t in (a, w, out):
+def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: int = 1) -> int:
+    """out = a[M, K] @ w[N, K]^T for M <= 64 with the LDS-staged weight-streaming
+    MFMA kernel.  ``splits == 1``: out is [M, N], bfloat16 or float32.  More:
+    out is float32 [splits, M, N] and receives partial sums; returns how many of
+    them were written (the reader adds out[:returned])."""
+    for t in (a, w):
         _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
     m, k = a.shape
     n = w.shape[0]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "the streaming product takes bfloat16 inputs")
-    _need(w.shape[1] == k and out.shape == (m, n), "gemm shapes disagree")
+    _need(w.shape[1] == k, "gemm shapes disagree")
     _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "streaming product needs M <= 64 and 16-byte aligned rows")
-    _need(1 <= splits <= 64, "splits in 1..64")
-    if splits > 1:
-        row_blocks = -(-n // 64)
-        need = splits * row_blocks * 4 * (-(-m // 16)) * 256
-        _need(partial is not None and partial.dtype == torch.float32 and partial.numel() >= need
-              and partial.is_cuda and partial.is_contiguous(), "split-K workspace too small")
-        _need(counters is not None and counters.dtype == torch.int32 and counters.numel() >= row_blocks
-              and counters.is_cuda and counters.is_contiguous(), "split-K counters too small")
-    _check(_fn("gemm_mfma", "tk_gemm_stream")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
-                                              w.stride(0), out.stride(0), splits, _p(partial), _p(counters),
-                                              _stream()), "gemm_stream")
+    _need(out.is_cuda and out.stride(-1) == 1, "output must be a GPU tensor with unit inner stride")
+    if splits == 1:
+        _need(out.shape == (m, n), "output must be [M, N]")
+        ldc, stride = out.stride(0), 0
+    else:
+        _need(1 < splits <= 64 and out.dtype == torch.float32 and out.shape == (splits, m, n) and out.is_contiguous(),
+              "with splits the output is contiguous float32 [splits, M, N]")
+        ldc, stride = n, m * n
+    used = _fn("gemm_mfma", "tk_gemm_stream")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
+                                              w.stride(0), ldc, splits, stride, _stream())
+    if used < 1:
+        raise KernelError(f"gemm_stream failed with status {used}")
+    return used
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, row_tiles: int, waves: int) -> None:

@@ -73,7 +73,7 @@ class GQAAttention(Mixer):
         nh, nkv, hd = self.num_heads, self.num_kv_heads, self.head_dim
         n = h.shape[0]
         weight = self.qkv if writes_cache else self.qkv[: nh * hd]
-        qkv = linear(h, weight)
+        qkv = linear(h, weight, allow_partials=True)
         cos, sin = self.position.prepare(batch)
         tables = batch.block_tables[store.group]
         q = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
@@ -86,7 +86,7 @@ class GQAAttention(Mixer):
         paged_attention(q, store.arrays["k"], store.arrays["v"], tables, batch, attended,
                         num_heads=nh, num_kv_heads=nkv, head_dim=hd, page_size=store.page_size,
                         scale=self.softmax_scale, window=self.window)
-        return linear(attended, self.o)
+        return linear(attended, self.o, allow_partials=True)
 
 
 register_part("mixer", "gqa_attention", GQAAttention)

@@ -7,7 +7,9 @@ in: sizes and constants arrive as parameters, checkpoint names arrive as a
 prefix, and everything about the running batch arrives in the ``StepBatch``.
 
 * ``Norm.forward(resid, delta, ...)``: adds ``delta`` into the float32 residual
-  stream and returns the normed activations in the compute dtype.
+  stream and returns the normed activations in the compute dtype.  ``delta`` is
+  a sub-layer's output: [N, H] in the compute dtype or float32, or float32
+  partial sums [P, N, H] of a split-K product, which the norm adds.
 * ``Mixer.forward(h, batch, store, writes_cache)``: token mixing.  It may own
   paged cache (``cache_request``) and/or fixed-size per-request state
   (``state_shape``); it sees its own storage only.

@@ -44,7 +44,7 @@ class SwiGLU(FeedForward):
         gate_up = linear(h, self.gate_up)
         act = torch.empty((h.shape[0], self.intermediate_size), dtype=h.dtype, device=h.device)
         ops.silu_mul(gate_up, act)
-        return linear(act, self.down)
+        return linear(act, self.down, allow_partials=True)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)
