@@ -42,6 +42,92 @@ TK_API int tk_embed_gather(int dtype, const void* table, const int* ids, float* 
 // ---------------------------------------------------------------------------
 // delta may come as `parts` float32 partial sums, part_stride elements apart
 // (a split-K product's output): they are added in order.
+template <typename TD> struct Load4;
+template <> struct Load4<float> {
+  static __device__ __forceinline__ float4 at(const float* p) { return *reinterpret_cast<const float4*>(p); }
+};
+template <> struct Load4<bf16_t> {
+  static __device__ __forceinline__ float4 at(const bf16_t* p) {
+    const uint2 u = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                       __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+  }
+};
+template <typename T> struct Store4;
+template <> struct Store4<float> {
+  static __device__ __forceinline__ void at(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+};
+template <> struct Store4<bf16_t> {
+  static __device__ __forceinline__ void at(bf16_t* p, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)float_to_bf16(v.x) | ((uint32_t)float_to_bf16(v.y) << 16);
+    u.y = (uint32_t)float_to_bf16(v.z) | ((uint32_t)float_to_bf16(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+  }
+};
+
+// Vector form: H a multiple of 4 and at most 4 * kNormGroups * blockDim.  A thread
+// keeps its elements of the row in registers, and all loads of the partial sums
+// are issued before the first add, so a row costs about one memory round trip.
+constexpr int kNormGroups = 4;
+
+template <typename T, typename TD>
+__global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
+    float* __restrict__ resid, const TD* __restrict__ delta, int parts, long part_stride,
+    const int* __restrict__ rows, const float* __restrict__ weight, T* __restrict__ out, int H,
+    float eps, int write_resid) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  const size_t row = rows ? (size_t)rows[m] : (size_t)m;
+  float* x = resid + row * H;
+  const TD* dl = delta ? delta + row * H : nullptr;
+  float4 xv[kNormGroups];
+  float ss = 0.f;
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    const int d = (g * blockDim.x + threadIdx.x) * 4;
+    xv[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (d < H) {
+      float4 v = *reinterpret_cast<const float4*>(x + d);
+      if (dl) {
+        int p = 0;
+        for (; p + 4 <= parts; p += 4) {
+          const float4 a = Load4<TD>::at(dl + (size_t)p * part_stride + d);
+          const float4 b = Load4<TD>::at(dl + (size_t)(p + 1) * part_stride + d);
+          const float4 c = Load4<TD>::at(dl + (size_t)(p + 2) * part_stride + d);
+          const float4 e = Load4<TD>::at(dl + (size_t)(p + 3) * part_stride + d);
+          v.x = (((v.x + a.x) + b.x) + c.x) + e.x;
+          v.y = (((v.y + a.y) + b.y) + c.y) + e.y;
+          v.z = (((v.z + a.z) + b.z) + c.z) + e.z;
+          v.w = (((v.w + a.w) + b.w) + c.w) + e.w;
+        }
+        for (; p < parts; ++p) {
+          const float4 a = Load4<TD>::at(dl + (size_t)p * part_stride + d);
+          v.x += a.x;
+          v.y += a.y;
+          v.z += a.z;
+          v.w += a.w;
+        }
+        if (write_resid) *reinterpret_cast<float4*>(x + d) = v;
+      }
+      xv[g] = v;
+      ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float rstd = rsqrtf(ss / (float)H + eps);
+  T* o = out + (size_t)m * H;
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    const int d = (g * blockDim.x + threadIdx.x) * 4;
+    if (d < H) {
+      const float4 w = *reinterpret_cast<const float4*>(weight + d);
+      Store4<T>::at(o + d, make_float4(xv[g].x * rstd * w.x, xv[g].y * rstd * w.y,
+                                       xv[g].z * rstd * w.z, xv[g].w * rstd * w.w));
+    }
+  }
+}
+
 template <typename T, typename TD>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
                                    int parts, long part_stride, const int* __restrict__ rows,
@@ -79,18 +165,26 @@ TK_API int tk_add_rmsnorm(int dtype, float* resid, const void* delta, int delta_
   if (M <= 0) return 0;
   if (rows && write_resid) return -1;
   if (parts < 1 || (parts > 1 && !delta_f32 && dtype != 0)) return -1;
-  if (dtype == 0)
-    add_rmsnorm_kernel<float, float><<<M, 256, 0, stream>>>(resid, (const float*)delta, parts,
-                                                            part_stride, rows, weight, (float*)out,
-                                                            H, eps, write_resid);
-  else if (delta_f32)
-    add_rmsnorm_kernel<bf16_t, float><<<M, 256, 0, stream>>>(resid, (const float*)delta, parts,
-                                                             part_stride, rows, weight,
-                                                             (bf16_t*)out, H, eps, write_resid);
-  else
-    add_rmsnorm_kernel<bf16_t, bf16_t><<<M, 256, 0, stream>>>(resid, (const bf16_t*)delta, parts,
-                                                              part_stride, rows, weight,
-                                                              (bf16_t*)out, H, eps, write_resid);
+  // vector form when the row fits a block's registers and everything is 16-byte aligned
+  int threads = 64;
+  while (threads < 1024 && threads * 4 < H) threads *= 2;
+  const bool vec = H % 4 == 0 && H <= threads * 4 * kNormGroups && part_stride % 4 == 0 &&
+                   ((uintptr_t)resid % 16 == 0) && ((uintptr_t)delta % 16 == 0) &&
+                   ((uintptr_t)weight % 16 == 0) && ((uintptr_t)out % 16 == 0);
+#define TK_NORM(KERNEL, T_, TD_)                                                                 \
+  KERNEL<T_, TD_><<<M, threads, 0, stream>>>(resid, (const TD_*)delta, parts, part_stride, rows, \
+                                             weight, (T_*)out, H, eps, write_resid)
+  if (vec) {
+    if (dtype == 0) TK_NORM(add_rmsnorm_vec_kernel, float, float);
+    else if (delta_f32) TK_NORM(add_rmsnorm_vec_kernel, bf16_t, float);
+    else TK_NORM(add_rmsnorm_vec_kernel, bf16_t, bf16_t);
+  } else {
+    threads = 256;
+    if (dtype == 0) TK_NORM(add_rmsnorm_kernel, float, float);
+    else if (delta_f32) TK_NORM(add_rmsnorm_kernel, bf16_t, float);
+    else TK_NORM(add_rmsnorm_kernel, bf16_t, bf16_t);
+  }
+#undef TK_NORM
   return launch_status();
 }
 
