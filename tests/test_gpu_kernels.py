@@ -358,3 +358,16 @@ def test_consumers_add_partial_sums():
     for a, b in zip(*outs):
         torch.testing.assert_close(a.float(), b.float(), rtol=1e-2, atol=1e-2)
     assert outs[0][2].abs().max() > 0
+
+
+@pytest.mark.parametrize("M, I, K", [(1, 64, 64), (8, 12288, 4096), (64, 200, 96), (33, 3072, 1024), (17, 136, 120)])
+def test_fused_gate_up_silu_product(M, I, K):
+    from tokamak_amd.kernels import ops
+
+    x = rand(M, K, seed=1).to(torch.bfloat16)
+    w = rand(2 * I, K, seed=2, scale=2 * K ** -0.5).to(torch.bfloat16)
+    out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_stream_swiglu(x.to(DEV), w.to(DEV), out)
+    g = x.double() @ w[:I].double().T
+    u = x.double() @ w[I:].double().T
+    torch.testing.assert_close(out.cpu().double(), g / (1 + torch.exp(-g)) * u, rtol=2e-2, atol=1e-2)

@@ -148,7 +148,10 @@ def test_toy_model_is_invariant_under_cutting(dtype):
     for rid, toks in (("a", a), ("b", b), ("c", c)):
         whole[rid] = runner.step([StepEntry(rid, toks, list(range(len(toks))))]).cpu()
         runner.end(rid)
-    tol = dict(rtol=1e-4, atol=2e-5) if dtype == "float32" else dict(rtol=5e-2, atol=5e-2)
+    # the suite's criterion (replay_util.TOL): float32 5e-5; bfloat16 2e-3 + 2% of the logits' scale
+    scale = max(float(w.abs().max()) for w in whole.values())
+    tol = dict(rtol=0, atol=5e-5) if dtype == "float32" else dict(rtol=0, atol=2e-3 + 2e-2 * scale)
+    print(f"toy model {dtype}: logit scale {scale:.2f}, tolerance {tol['atol']:.4f}")
     # portions down to two tokens, then single tokens
     got, at = [], 0
     for n in (16, 7, 2, 30, 2, 1, 1, 11):

@@ -219,7 +219,10 @@ TK_API int tk_gemm_skinny(int out_dtype, const void* A, const void* W, void* C, 
 constexpr int SBK = 256;        // k per chunk
 constexpr int SLD = SBK + 8;    // LDS row stride in elements
 
-template <int MT, typename TO>
+// GATED: W is [2N, K], gate rows then up rows; the block owns 32 output columns, waves
+// 0,1 their gate rows and waves 2,3 the matching up rows, and the result is
+// silu(gate) * up [M, N] (the SwiGLU feed-forward's first half in one kernel).
+template <int MT, typename TO, bool GATED>
 __global__ __launch_bounds__(256) void gemm_stream_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TO* __restrict__ C, int M, int N,
     int K, long lda, long ldw, long ldc, int chunks_per_split, long split_stride) {
@@ -228,7 +231,10 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, kb = lane >> 4;
   const int row_block = blockIdx.x, split = blockIdx.y;
-  const int n_wave = row_block * 64 + wave * 16;
+  // n_wave: first output column of this wave; w_first/w_limit: its weight rows
+  const int n_wave = GATED ? row_block * 32 + (wave & 1) * 16 : row_block * 64 + wave * 16;
+  const int w_first = (GATED && wave >= 2) ? N + n_wave : n_wave;
+  const int w_limit = (GATED && wave >= 2) ? 2 * N : N;
   const int total_chunks = (K + SBK - 1) / SBK;
   const int c_begin = split * chunks_per_split;
   const int c_end = min(total_chunks, c_begin + chunks_per_split);
@@ -246,7 +252,7 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
   // load from k = 0, so the loads of a chunk are all in flight together.
   const bf16_t* wrow[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) wrow[i] = W + (size_t)min(n_wave + 2 * i + w_row0, N - 1) * ldw;
+  for (int i = 0; i < 8; ++i) wrow[i] = W + (size_t)min(w_first + 2 * i + w_row0, w_limit - 1) * ldw;
   const bf16_t* xrow[2 * MT];
 #pragma unroll
   for (int i = 0; i < 2 * MT; ++i) xrow[i] = A + (size_t)min(i * 8 + x_row0, M - 1) * lda;
@@ -298,7 +304,28 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
   // reads C next adds the splits (in split order, so the sum is deterministic).
   C += (size_t)split * split_stride;
 
-  // acc[j][e] = C[batch row j*16 + r][weight row n_wave + kb*4 + e]
+  if (GATED) {
+    float* up = reinterpret_cast<float*>(&xs[0][0]);  // [2 up waves][MT][64 lanes][4]
+    __syncthreads();                                   // the last chunk's fragments have been read
+    if (wave >= 2) {
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+        *reinterpret_cast<float4*>(up + ((size_t)((wave - 2) * MT + j) * 64 + lane) * 4) =
+            make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+    }
+    __syncthreads();
+    if (wave >= 2) return;
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      const float4 u = *reinterpret_cast<const float4*>(up + ((size_t)(wave * MT + j) * 64 + lane) * 4);
+      acc[j][0] = acc[j][0] / (1.f + __expf(-acc[j][0])) * u.x;
+      acc[j][1] = acc[j][1] / (1.f + __expf(-acc[j][1])) * u.y;
+      acc[j][2] = acc[j][2] / (1.f + __expf(-acc[j][2])) * u.z;
+      acc[j][3] = acc[j][3] / (1.f + __expf(-acc[j][3])) * u.w;
+    }
+  }
+
+  // acc[j][e] = C[batch row j*16 + r][column n_wave + kb*4 + e]
 #pragma unroll
   for (int j = 0; j < MT; ++j) {
     const int m = j * 16 + r;
@@ -311,16 +338,16 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
   }
 }
 
-template <typename TO>
+template <typename TO, bool GATED>
 static int launch_stream(const void* A, const void* W, void* C, int M, int N, int K, long lda,
                          long ldw, long ldc, int chunks_per_split, int KS, long split_stride,
                          hipStream_t stream) {
-  dim3 grid((N + 63) / 64, KS);
+  dim3 grid(GATED ? (N + 31) / 32 : (N + 63) / 64, KS);
   const int mt = (M + 15) / 16;
-#define TK_STREAM(MT_)                                                                        \
-  gemm_stream_kernel<MT_, TO><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W,  \
-                                                        (TO*)C, M, N, K, lda, ldw, ldc,      \
-                                                        chunks_per_split, split_stride)
+#define TK_STREAM(MT_)                                                                          \
+  gemm_stream_kernel<MT_, TO, GATED><<<grid, 256, 0, stream>>>(                                 \
+      (const bf16_t*)A, (const bf16_t*)W, (TO*)C, M, N, K, lda, ldw, ldc, chunks_per_split,     \
+      split_stride)
   if (mt == 1) TK_STREAM(1);
   else if (mt == 2) TK_STREAM(2);
   else if (mt == 3) TK_STREAM(3);
@@ -343,7 +370,16 @@ TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, 
   const int cps = (total_chunks + splits - 1) / splits;
   const int ks = (total_chunks + cps - 1) / cps;
   int status = -1;
-  if (out_dtype == 0) status = launch_stream<float>(A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
-  if (out_dtype == 1) status = launch_stream<bf16_t>(A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
+  if (out_dtype == 0) status = launch_stream<float, false>(A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
+  if (out_dtype == 1) status = launch_stream<bf16_t, false>(A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
   return status == 0 ? ks : (status > 0 ? -status : status);
+}
+
+// C[M, N] = silu(A W_gate^T) * (A W_up^T) with W = [W_gate; W_up] of 2N rows; bfloat16 out.
+TK_API int tk_gemm_stream_swiglu(const void* A, const void* W, void* C, int M, int N, int K, long lda,
+                                 long ldw, long ldc, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
+  const int total_chunks = (K + SBK - 1) / SBK;
+  return launch_stream<bf16_t, true>(A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0, stream);
 }

@@ -30,3 +30,24 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype | None 
     from tokamak_amd.kernels import gemm_bf16
 
     return gemm_bf16.gemm(x, weight, out_dtype, allow_partials)
+
+
+def gated_linear(x: torch.Tensor, gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(x @ gate^T) * (x @ up^T) for ``gate_up`` = [gate; up] ([2I, K]) -> [M, I].
+
+    bfloat16 with up to 64 rows: one fused weight-streaming kernel.  Otherwise
+    the product, then the SiLU-gate kernel.
+    """
+    m = x.shape[0]
+    inter = gate_up.shape[0] // 2
+    out = torch.empty((m, inter), dtype=x.dtype, device=x.device)
+    if m == 0:
+        return out
+    if x.dtype == torch.bfloat16 and m <= 64:
+        from tokamak_amd.kernels import gemm_bf16
+
+        if gemm_bf16.skinny_fits(x, gate_up):
+            ops.gemm_stream_swiglu(x, gate_up, out)
+            return out
+    ops.silu_mul(linear(x, gate_up), out)
+    return out

@@ -73,6 +73,8 @@ _SIGS = {
     "gemm_mfma": {
         "tk_gemm_stream": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                            c_long, c_int, c_long, c_void_p],
+        "tk_gemm_stream_swiglu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long,
+                                  c_void_p],
         "tk_gemm_skinny": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                            c_long, c_int, c_int, c_void_p],
     },
@@ -253,6 +255,20 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
     if used < 1:
         raise KernelError(f"gemm_stream failed with status {used}")
     return used
+
+
+def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out[M, I] = silu(a @ w[:I]^T) * (a @ w[I:]^T) for M <= 64: the gate and up
+    projections and the SiLU product in one weight-streaming kernel (bfloat16)."""
+    for t in (a, w, out):
+        _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
+    m, k = a.shape
+    _need(w.shape[0] % 2 == 0 and w.shape[1] == k and out.shape == (m, w.shape[0] // 2), "gated product shapes disagree")
+    _need(a.dtype == w.dtype == out.dtype == torch.bfloat16, "the gated product is bfloat16")
+    _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+          and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gated product needs M <= 64 and 16-byte aligned rows")
+    _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
+                                                     w.stride(0), out.stride(0), _stream()), "gemm_stream_swiglu")
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, row_tiles: int, waves: int) -> None:

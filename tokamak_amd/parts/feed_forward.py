@@ -5,8 +5,7 @@ from __future__ import annotations
 import torch
 
 from tokamak_amd.config.registry import register_part
-from tokamak_amd.kernels import ops
-from tokamak_amd.kernels.linear import linear
+from tokamak_amd.kernels.linear import gated_linear, linear
 from tokamak_amd.parts.base import FeedForward, Fetch
 from tokamak_amd.weights.spec import TensorSpec
 
@@ -41,10 +40,7 @@ class SwiGLU(FeedForward):
         self.down = fetch(prefix + "down_proj.weight")
 
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
-        gate_up = linear(h, self.gate_up)
-        act = torch.empty((h.shape[0], self.intermediate_size), dtype=h.dtype, device=h.device)
-        ops.silu_mul(gate_up, act)
-        return linear(act, self.down, allow_partials=True)
+        return linear(gated_linear(h, self.gate_up), self.down, allow_partials=True)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)
