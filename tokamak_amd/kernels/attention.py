@@ -7,8 +7,8 @@ import torch
 from tokamak_amd.kernels import ops
 
 MFMA_HEAD_DIMS = (64, 128)
-SPLIT_KEYS = 256          # keys per split of a decode token's context
-MAX_DECODE_WAVES = 8192   # above this, splits are made longer
+SPLIT_KEYS = 256          # fewest keys a split of a decode token's context holds
+TARGET_DECODE_WAVES = 4096  # waves wanted in flight; beyond that splits only cost a merge
 
 
 def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
@@ -17,10 +17,13 @@ def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
 
 
 def decode_split(num_decode: int, num_kv_heads: int, max_len: int) -> tuple[int, int]:
-    """(keys per split, number of splits) for the decode tokens of a step."""
-    split = SPLIT_KEYS
-    while num_decode * num_kv_heads * -(-max_len // split) > MAX_DECODE_WAVES and split < 16384:
-        split *= 2
+    """(keys per split, number of splits) for the decode tokens of a step: as few
+    splits as fill the GPU (one wave per request, kv head and split), never
+    shorter than SPLIT_KEYS."""
+    most = max(1, -(-max_len // SPLIT_KEYS))
+    nsplit = min(most, max(1, -(-TARGET_DECODE_WAVES // (num_decode * num_kv_heads))))
+    split = -(-max_len // nsplit)
+    split = -(-split // 16) * 16
     return split, max(1, -(-max_len // split))
 
 
