@@ -177,8 +177,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
       }
       l_run[s] = l_run[s] * alpha + psum;
       Frag4 pb;
-      pb.v = short4v{(short)float_to_bf16(p[0]), (short)float_to_bf16(p[1]),
-                     (short)float_to_bf16(p[2]), (short)float_to_bf16(p[3])};
+      pb.u = make_uint2(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]));
 #pragma unroll
       for (int d = 0; d < DBL; ++d) {
         float4v a = acc[s][d];
@@ -205,10 +204,9 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
       bf16_t* op = out + row * HD + kb * 4;
 #pragma unroll
       for (int d = 0; d < DBL; ++d) {
-        Frag4 o;
-        o.v = short4v{(short)float_to_bf16(acc[s][d][0] * inv), (short)float_to_bf16(acc[s][d][1] * inv),
-                      (short)float_to_bf16(acc[s][d][2] * inv), (short)float_to_bf16(acc[s][d][3] * inv)};
-        *reinterpret_cast<uint2*>(op + d * 16) = o.u;
+        *reinterpret_cast<uint2*>(op + d * 16) =
+            make_uint2(pack_bf16x2(acc[s][d][0] * inv, acc[s][d][1] * inv),
+                       pack_bf16x2(acc[s][d][2] * inv, acc[s][d][3] * inv));
       }
     } else {
       float* po = part_o + (prow * nsplit + split) * HD + kb * 4;
@@ -378,7 +376,7 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
         sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[c], sc, 0, 0, 0);
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sv[j][i] = sc[i] * scale_log2;
+      for (int i = 0; i < 4; ++i) sv[j][i] = sc[i];
     }
     if (s0 + 63 > pos0) {  // some key of this stage is hidden from some column, or is past the end
 #pragma unroll
@@ -396,7 +394,8 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
       for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, sv[j][i]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-    const float m_new = fmaxf(m_run, tmax);
+    // the running maximum is kept in units of log2: m = max(score) * scale * log2(e)
+    const float m_new = fmaxf(m_run, tmax * scale_log2);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
     const float alpha = fast_exp2(m_run - m_safe);
     m_run = m_new;
@@ -407,25 +406,27 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
       float p[8];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        p[i] = fast_exp2(sv[2 * h][i] - m_safe);
-        p[4 + i] = fast_exp2(sv[2 * h + 1][i] - m_safe);
+        p[i] = fast_exp2(fmaf(sv[2 * h][i], scale_log2, -m_safe));
+        p[4 + i] = fast_exp2(fmaf(sv[2 * h + 1][i], scale_log2, -m_safe));
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) psum += p[i];
-      pb[h].u = make_uint4((uint32_t)float_to_bf16(p[0]) | ((uint32_t)float_to_bf16(p[1]) << 16),
-                           (uint32_t)float_to_bf16(p[2]) | ((uint32_t)float_to_bf16(p[3]) << 16),
-                           (uint32_t)float_to_bf16(p[4]) | ((uint32_t)float_to_bf16(p[5]) << 16),
-                           (uint32_t)float_to_bf16(p[6]) | ((uint32_t)float_to_bf16(p[7]) << 16));
+      pb[h].u = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
+                           pack_bf16x2(p[6], p[7]));
     }
     l_run = l_run * alpha + psum;
+    // the accumulators need rescaling only when some column's maximum moved
+    const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
     const bool tail = s0 + 63 > last_pos;  // keys past the end may hold anything: zero their values
 #pragma unroll
     for (int d = 0; d < DBL; ++d) {
       float4v a = acc[d];
-      a[0] *= alpha;
-      a[1] *= alpha;
-      a[2] *= alpha;
-      a[3] *= alpha;
+      if (rescale) {
+        a[0] *= alpha;
+        a[1] *= alpha;
+        a[2] *= alpha;
+        a[3] *= alpha;
+      }
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         // A operand: V^T[dim col][k], k = (group 2h quad kb) then (group 2h+1 quad kb)
@@ -455,8 +456,8 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
 #pragma unroll
     for (int d = 0; d < DBL; ++d) {
       uint2 o;
-      o.x = (uint32_t)float_to_bf16(acc[d][0] * inv) | ((uint32_t)float_to_bf16(acc[d][1] * inv) << 16);
-      o.y = (uint32_t)float_to_bf16(acc[d][2] * inv) | ((uint32_t)float_to_bf16(acc[d][3] * inv) << 16);
+      o.x = pack_bf16x2(acc[d][0] * inv, acc[d][1] * inv);
+      o.y = pack_bf16x2(acc[d][2] * inv, acc[d][3] * inv);
       *reinterpret_cast<uint2*>(op + d * 16) = o;
     }
   }

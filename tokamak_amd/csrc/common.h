@@ -13,12 +13,19 @@ __device__ __forceinline__ float bf16_to_float(bf16_t v) {
   return __uint_as_float(static_cast<uint32_t>(v) << 16);
 }
 
-// round-to-nearest-even; NaN stays NaN
+// round-to-nearest-even; NaN stays NaN.  gfx950 converts in hardware
+// (v_cvt_pk_bf16_f32), which the compiler emits for these casts.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const f32x2_t f = {lo, hi};
+  const bf16x2_t v = __builtin_convertvector(f, bf16x2_t);
+  return *reinterpret_cast<const uint32_t*>(&v);
+}
+
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<bf16_t>(u >> 16);
+  return static_cast<bf16_t>(pack_bf16x2(f, 0.f) & 0xffffu);
 }
 
 template <typename T> struct Elem;

@@ -60,8 +60,8 @@ template <> struct Store4<float> {
 template <> struct Store4<bf16_t> {
   static __device__ __forceinline__ void at(bf16_t* p, float4 v) {
     uint2 u;
-    u.x = (uint32_t)float_to_bf16(v.x) | ((uint32_t)float_to_bf16(v.y) << 16);
-    u.y = (uint32_t)float_to_bf16(v.z) | ((uint32_t)float_to_bf16(v.w) << 16);
+    u.x = pack_bf16x2(v.x, v.y);
+    u.y = pack_bf16x2(v.z, v.w);
     *reinterpret_cast<uint2*>(p) = u;
   }
 };
@@ -227,9 +227,18 @@ TK_API int tk_rope_tables(const int* positions, const float* inv_freq, float* co
 //                                 operand of the PV product, lane (dim, quad),
 //                                 is 8 contiguous bytes and a wave reads 512
 //                                 contiguous bytes)
-// One 64-lane block per (token, head).
+// One wave per (token, head), four waves a block, each with an LDS row of its own.
 // ---------------------------------------------------------------------------
 constexpr int kMaxHeadDim = 512;
+constexpr int kPairsPerBlock = 4;  // (token, head) pairs per block, one per wave
+
+// Orders one wave's LDS accesses (a wave's LDS instructions execute in order; this
+// keeps the compiler from moving them across the point).
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
 template <typename T, typename TIN>
 __global__ void qknorm_rope_store_kernel(
@@ -239,10 +248,15 @@ __global__ void qknorm_rope_store_kernel(
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ block_tables, T* __restrict__ q_out, T* __restrict__ k_cache,
     T* __restrict__ v_cache, int nh, int nkv_in, int nkv, int hd, int rot, int ps, int max_pages,
-    float eps) {
-  __shared__ float vec[kMaxHeadDim];
-  const int n = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int row_width = (nh + 2 * nkv_in) * hd;
+    float eps, int num_pairs) {
+  __shared__ float vecs[kPairsPerBlock][kMaxHeadDim];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int heads = nh + 2 * nkv_in;
+  const int pair = blockIdx.x * kPairsPerBlock + wave;
+  if (pair >= num_pairs) return;  // nothing below synchronises across waves
+  const int n = pair / heads, head = pair - n * heads;
+  float* vec = vecs[wave];
+  const int row_width = heads * hd;
   const TIN* src = qkv + (size_t)n * row_width + (size_t)head * hd;
   const bool is_q = head < nh;
   const bool is_k = !is_q && head < nh + nkv_in;
@@ -259,10 +273,10 @@ __global__ void qknorm_rope_store_kernel(
     if (w) {
       ss = wave_sum(ss);
       const float rstd = rsqrtf(ss / (float)hd + eps);
-      __syncthreads();
+      wave_lds_sync();
       for (int d = lane; d < hd; d += kWave) vec[d] = vec[d] * rstd * w[d];
     }
-    __syncthreads();
+    wave_lds_sync();
     // out[j] = x[j] cos_j - x[j+half] sin_j ; out[j+half] = x[j+half] cos_j + x[j] sin_j
     const int half = rot / 2;
     float lo[kMaxHeadDim / 2 / kWave], hi[kMaxHeadDim / 2 / kWave];
@@ -273,14 +287,14 @@ __global__ void qknorm_rope_store_kernel(
       lo[cnt] = a * c - b * s;
       hi[cnt] = b * c + a * s;
     }
-    __syncthreads();
+    wave_lds_sync();
     cnt = 0;
     for (int j = lane; j < half; j += kWave, ++cnt) {
       vec[j] = lo[cnt];
       vec[j + half] = hi[cnt];
     }
   }
-  __syncthreads();
+  wave_lds_sync();
 
   if (is_q) {
     T* dst = q_out + ((size_t)n * nh + head) * hd;
@@ -315,12 +329,14 @@ TK_API int tk_qknorm_rope_store(int dtype, const void* qkv, int in_f32, int part
   if (hd > kMaxHeadDim || hd % 16 != 0 || ps % 4 != 0 || rot > hd || rot % 2 != 0) return -1;
   if (nkv_in != 0 && nkv_in != nkv) return -1;
   if (parts < 1 || (parts > 1 && !in_f32 && dtype != 0)) return -1;
-  dim3 grid(N, nh + 2 * nkv_in);
+  const long pairs = (long)N * (nh + 2 * nkv_in);
+  if (pairs > 0x7fffffffL) return -1;
+  const unsigned grid = (unsigned)((pairs + kPairsPerBlock - 1) / kPairsPerBlock);
 #define TK_QK(T_, TIN_)                                                                          \
-  qknorm_rope_store_kernel<T_, TIN_><<<grid, kWave, 0, stream>>>(                                \
+  qknorm_rope_store_kernel<T_, TIN_><<<grid, kWave * kPairsPerBlock, 0, stream>>>(               \
       (const TIN_*)qkv, parts, part_stride, q_weight, k_weight, cos_t, sin_t, positions,         \
       req_of_token, block_tables, (T_*)q_out, (T_*)k_cache, (T_*)v_cache, nh, nkv_in, nkv, hd,   \
-      rot, ps, max_pages, eps)
+      rot, ps, max_pages, eps, (int)pairs)
   if (dtype == 0) TK_QK(float, float);
   else if (in_f32) TK_QK(bf16_t, float);
   else TK_QK(bf16_t, bf16_t);
@@ -342,9 +358,36 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   Elem<T>::store(out + idx, g / (1.f + expf(-g)) * u);
 }
 
+// 8 elements a thread (16-byte loads): I a multiple of 8, pointers 16-byte aligned
+__global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
+                                       int I, size_t total8) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total8) return;
+  const int per_row = I / 8;
+  const size_t n = idx / per_row;
+  const int i = (int)(idx - n * per_row) * 8;
+  const uint4 g = *reinterpret_cast<const uint4*>(gu + n * 2 * I + i);
+  const uint4 u = *reinterpret_cast<const uint4*>(gu + n * 2 * I + I + i);
+  const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+  uint32_t ow[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
+    const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
+    ow[k] = pack_bf16x2(g0 / (1.f + expf(-g0)) * u0, g1 / (1.f + expf(-g1)) * u1);
+  }
+  *reinterpret_cast<uint4*>(out + n * I + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 TK_API int tk_silu_mul(int dtype, const void* gu, void* out, int N, int I, hipStream_t stream) {
   if (N <= 0 || I <= 0) return 0;
   const size_t total = (size_t)N * I;
+  if (dtype == 1 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const size_t total8 = total / 8;
+    silu_mul_bf16x8_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>(
+        (const bf16_t*)gu, (bf16_t*)out, I, total8);
+    return launch_status();
+  }
   const unsigned blocks = (unsigned)((total + 255) / 256);
   if (dtype == 0)
     silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
