@@ -166,8 +166,9 @@ TK_API int tk_add_rmsnorm(int dtype, float* resid, const void* delta, int delta_
   if (rows && write_resid) return -1;
   if (parts < 1 || (parts > 1 && !delta_f32 && dtype != 0)) return -1;
   // vector form when the row fits a block's registers and everything is 16-byte aligned
+  // one element group per thread when rows are few (short latency chain), four when many
   int threads = 64;
-  while (threads < 1024 && threads * 4 < H) threads *= 2;
+  while (threads < 1024 && threads * 4 * (M >= 512 ? kNormGroups : 1) < H) threads *= 2;
   const bool vec = H % 4 == 0 && H <= threads * 4 * kNormGroups && part_stride % 4 == 0 &&
                    ((uintptr_t)resid % 16 == 0) && ((uintptr_t)delta % 16 == 0) &&
                    ((uintptr_t)weight % 16 == 0) && ((uintptr_t)out % 16 == 0);
@@ -318,6 +319,89 @@ __global__ void qknorm_rope_store_kernel(
   }
 }
 
+// Fast form for head sizes 64 and 128 rotated over their full width (rot == HD):
+// a lane owns 8 consecutive dims of one head (one 16-byte piece), so a wave covers
+// 64*8/HD heads; the rotation partner (dim +- HD/2) sits HD/16 lanes away, the sum
+// of squares is over HD/8 neighbouring lanes, and nothing goes through LDS.
+template <typename T, typename TIN, int HD>
+__global__ __launch_bounds__(256) void qknorm_rope_store_vec_kernel(
+    const TIN* __restrict__ qkv, int parts, long part_stride, const float* __restrict__ q_weight,
+    const float* __restrict__ k_weight, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, const int* __restrict__ positions,
+    const int* __restrict__ req_of_token, const int* __restrict__ block_tables,
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int nkv_in,
+    int nkv, int ps, int max_pages, float eps, long num_pairs) {
+  constexpr int LPH = HD / 8;  // lanes per head
+  const long slot = ((long)blockIdx.x * blockDim.x + threadIdx.x) / LPH;  // (token, head) pair
+  if (slot >= num_pairs) return;  // whole LPH-lane groups leave together
+  const int sub = threadIdx.x % LPH, d0 = sub * 8;
+  const int heads = nh + 2 * nkv_in;
+  const int n = (int)(slot / heads), head = (int)(slot - (long)n * heads);
+  const bool is_q = head < nh, is_k = !is_q && head < nh + nkv_in;
+  const TIN* src = qkv + (size_t)n * heads * HD + (size_t)head * HD + d0;
+  float x[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = 0.f;
+  for (int p = 0; p < parts; ++p) {
+    const float4 a = Load4<TIN>::at(src + (size_t)p * part_stride);
+    const float4 b = Load4<TIN>::at(src + (size_t)p * part_stride + 4);
+    x[0] += a.x; x[1] += a.y; x[2] += a.z; x[3] += a.w;
+    x[4] += b.x; x[5] += b.y; x[6] += b.z; x[7] += b.w;
+  }
+  if (is_q || is_k) {
+    const float* w = is_q ? q_weight : k_weight;
+    const int j0 = d0 % (HD / 2);  // index into the cos/sin row
+    const float4 c0 = *reinterpret_cast<const float4*>(cos_t + (size_t)n * (HD / 2) + j0);
+    const float4 c1 = *reinterpret_cast<const float4*>(cos_t + (size_t)n * (HD / 2) + j0 + 4);
+    const float4 s0 = *reinterpret_cast<const float4*>(sin_t + (size_t)n * (HD / 2) + j0);
+    const float4 s1 = *reinterpret_cast<const float4*>(sin_t + (size_t)n * (HD / 2) + j0 + 4);
+    const float cs[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+    const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+    if (w) {
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+#pragma unroll
+      for (int m = LPH / 2; m >= 1; m >>= 1) ss += __shfl_xor(ss, m, kWave);
+      const float rstd = rsqrtf(ss / (float)HD + eps);
+      const float4 w0 = *reinterpret_cast<const float4*>(w + d0);
+      const float4 w1 = *reinterpret_cast<const float4*>(w + d0 + 4);
+      const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = x[e] * rstd * wv[e];
+    }
+    // first half: x cos - partner sin; second half: x cos + partner sin
+    const float sign = (d0 < HD / 2) ? -1.f : 1.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float partner = __shfl_xor(x[e], LPH / 2, kWave);
+      x[e] = x[e] * cs[e] + sign * partner * sn[e];
+    }
+  }
+  if (is_q) {
+    Store4<T>::at(q_out + ((size_t)n * nh + head) * HD + d0, make_float4(x[0], x[1], x[2], x[3]));
+    Store4<T>::at(q_out + ((size_t)n * nh + head) * HD + d0 + 4, make_float4(x[4], x[5], x[6], x[7]));
+    return;
+  }
+  const int pos = positions[n];
+  const int page = block_tables[(size_t)req_of_token[n] * max_pages + pos / ps];
+  const int off = pos % ps;
+  const size_t page_elems = (size_t)nkv * HD * ps;
+  if (is_k) {
+    T* base = k_cache + (size_t)page * page_elems + (size_t)(head - nh) * HD * ps;
+    T* dst = base + ((size_t)sub * ps + off) * 8;  // dims d0 .. d0+7 of this token: one 8-element piece
+    Store4<T>::at(dst, make_float4(x[0], x[1], x[2], x[3]));
+    Store4<T>::at(dst + 4, make_float4(x[4], x[5], x[6], x[7]));
+  } else {
+    T* base = v_cache + (size_t)page * page_elems + (size_t)(head - nh - nkv_in) * HD * ps;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int d = d0 + e;
+      Elem<T>::store(base + ((size_t)(d >> 4) * (ps >> 2) + (off >> 2)) * 64 + (d & 15) * 4 + (off & 3), x[e]);
+    }
+  }
+}
+
 // in_f32: qkv is float32 (possibly `parts` partial sums, part_stride elements apart)
 TK_API int tk_qknorm_rope_store(int dtype, const void* qkv, int in_f32, int parts, long part_stride,
                                 const float* q_weight, const float* k_weight, const float* cos_t,
@@ -331,6 +415,29 @@ TK_API int tk_qknorm_rope_store(int dtype, const void* qkv, int in_f32, int part
   if (parts < 1 || (parts > 1 && !in_f32 && dtype != 0)) return -1;
   const long pairs = (long)N * (nh + 2 * nkv_in);
   if (pairs > 0x7fffffffL) return -1;
+  if ((hd == 128 || hd == 64) && rot == hd && part_stride % 4 == 0 && (uintptr_t)qkv % 16 == 0 &&
+      (uintptr_t)q_out % 16 == 0 && (uintptr_t)k_cache % 16 == 0 && (uintptr_t)cos_t % 16 == 0 &&
+      (uintptr_t)sin_t % 16 == 0 && (!q_weight || (uintptr_t)q_weight % 16 == 0) &&
+      (!k_weight || (uintptr_t)k_weight % 16 == 0) && (q_weight != nullptr) == (k_weight != nullptr)) {
+    const long lanes = pairs * (hd / 8);
+    const unsigned vgrid = (unsigned)((lanes + 255) / 256);
+#define TK_QKV(T_, TIN_, HD_)                                                                     \
+  qknorm_rope_store_vec_kernel<T_, TIN_, HD_><<<vgrid, 256, 0, stream>>>(                         \
+      (const TIN_*)qkv, parts, part_stride, q_weight, k_weight, cos_t, sin_t, positions,          \
+      req_of_token, block_tables, (T_*)q_out, (T_*)k_cache, (T_*)v_cache, nh, nkv_in, nkv, ps,    \
+      max_pages, eps, pairs)
+    if (hd == 128) {
+      if (dtype == 0) TK_QKV(float, float, 128);
+      else if (in_f32) TK_QKV(bf16_t, float, 128);
+      else TK_QKV(bf16_t, bf16_t, 128);
+    } else {
+      if (dtype == 0) TK_QKV(float, float, 64);
+      else if (in_f32) TK_QKV(bf16_t, float, 64);
+      else TK_QKV(bf16_t, bf16_t, 64);
+    }
+#undef TK_QKV
+    return launch_status();
+  }
   const unsigned grid = (unsigned)((pairs + kPairsPerBlock - 1) / kPairsPerBlock);
 #define TK_QK(T_, TIN_)                                                                          \
   qknorm_rope_store_kernel<T_, TIN_><<<grid, kWave * kPairsPerBlock, 0, stream>>>(               \
