@@ -1,13 +1,9 @@
 // Paged causal attention on the matrix cores (bf16 in, float32 softmax and
 // accumulation) for head sizes 64 and 128 and page sizes 16, 32, 64, ... (powers of two).
 //
-// One 64-lane wave owns a work item: up to 16 "columns" per column set that share
-// one kv head and one request, and a range of that request's keys (a split).
-//   heads mode  (decode):  the columns of set s are query heads s*16 .. s*16+15 of
-//                          the group, all of one token;
-//   tokens mode:           the columns are 16 consecutive tokens of one request,
-//                          set s is query head s of the group (kept for reference;
-//                          prompt portions use attention_prefill_kernel below).
+// Decode tokens (attention_decode_kernel): one 64-lane wave owns one token, one kv
+// head and a range of that request's keys (a split); its 16 "columns" are the
+// query heads of the group.
 // Keys are taken 16 at a time (one MFMA tile, never across a page edge):
 //   S^T[key][col] = K[key][:] . Q[col][:]      v_mfma_f32_16x16x32_bf16, K rows as A
 //   P^T = exp2(S^T * c - m[col])               float32, one column per lane
@@ -39,8 +35,8 @@ union Frag4 {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-template <int HD, int NSETS, bool TOKENS>
-__global__ __launch_bounds__(64) void attention_mfma_kernel(
+template <int HD, int NSETS>
+__global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
@@ -52,12 +48,10 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
   const int lane = threadIdx.x, col = lane & 15, kb = lane >> 4;
   const int split = blockIdx.x, item = blockIdx.z;
   const int G = nh / nkv;
-  const int sets_per_group = TOKENS ? G / NSETS : 1;
-  const int kvh = blockIdx.y / sets_per_group;
-  const int set0 = (blockIdx.y % sets_per_group) * NSETS;  // first head of the group (tokens mode)
+  const int kvh = blockIdx.y;
 
   const int n0 = item_token[item];
-  const int count = TOKENS ? item_count[item] : 1;
+  const int count = 1;
   const int pos0 = positions[n0];
   const int last_pos = pos0 + count - 1;
   const int k_begin = split * split_keys;
@@ -70,18 +64,12 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
   // which (token, head) this lane's column is, per set
   int c_token[NSETS], c_head[NSETS];
   bool c_valid[NSETS];
-  const int c_pos = TOKENS ? pos0 + col : pos0;
+  const int c_pos = pos0;
 #pragma unroll
   for (int s = 0; s < NSETS; ++s) {
-    if (TOKENS) {
-      c_token[s] = n0 + col;
-      c_head[s] = kvh * G + set0 + s;
-      c_valid[s] = col < count;
-    } else {
-      c_token[s] = n0;
-      c_head[s] = kvh * G + s * 16 + col;
-      c_valid[s] = s * 16 + col < G;
-    }
+    c_token[s] = n0;
+    c_head[s] = kvh * G + s * 16 + col;
+    c_valid[s] = s * 16 + col < G;
   }
 
   // Q as B operand: lane (col, kb) holds Q[col][c*32 + kb*8 .. +8]
@@ -234,20 +222,29 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(
   const size_t row = (size_t)blockIdx.x * nh + head;  // partial row (by item)
   const size_t orow = (size_t)n * nh + head;          // output row (by token)
   const int used = min(nsplit, positions[n] / split_keys + 1);
+  const float* ml = part_ml + row * nsplit * 2;
+  // lane s holds split s's (m, l): one load each, then the maximum over the wave
   float mx = -INFINITY;
-  for (int s = 0; s < used; ++s) mx = fmaxf(mx, part_ml[(row * nsplit + s) * 2]);
+  for (int s = lane; s < used; s += kWave) mx = fmaxf(mx, ml[s * 2]);
+  mx = wave_max(mx);
   float denom = 0.f;
   float o[HD / 64];
 #pragma unroll
   for (int i = 0; i < HD / 64; ++i) o[i] = 0.f;
-  for (int s = 0; s < used; ++s) {
-    const float w = fast_exp2(part_ml[(row * nsplit + s) * 2] - mx);
-    denom += w * part_ml[(row * nsplit + s) * 2 + 1];
-    const float* po = part_o + (row * nsplit + s) * HD;
+  for (int s0 = 0; s0 < used; s0 += kWave) {
+    const int mine = s0 + lane;
+    const float w_mine = mine < used ? fast_exp2(ml[mine * 2] - mx) : 0.f;
+    denom += mine < used ? w_mine * ml[mine * 2 + 1] : 0.f;
+    const int count = min(kWave, used - s0);
+    const float* po = part_o + (row * nsplit + s0) * HD;
+#pragma unroll 4
+    for (int t = 0; t < count; ++t) {
+      const float w = __shfl(w_mine, t, kWave);
 #pragma unroll
-    for (int i = 0; i < HD / 64; ++i) o[i] += w * po[lane + i * 64];
+      for (int i = 0; i < HD / 64; ++i) o[i] = fmaf(w, po[(size_t)t * HD + lane + i * 64], o[i]);
+    }
   }
-  const float inv = 1.f / denom;
+  const float inv = 1.f / wave_sum(denom);
 #pragma unroll
   for (int i = 0; i < HD / 64; ++i) out[orow * HD + lane + i * 64] = float_to_bf16(o[i] * inv);
 }
@@ -480,15 +477,15 @@ static int launch_prefill(const void* q, const void* k_cache, const void* v_cach
   return launch_status();
 }
 
-template <int HD, int NSETS, bool TOKENS>
+template <int HD, int NSETS>
 static int launch(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                   int max_pages, const int* positions, const int* req_of_token,
                   const int* item_token, const int* item_count, int num_items, void* out,
                   float* part_o, float* part_ml, int nsplit, int split_keys, int nh, int nkv, int ps,
                   float scale, hipStream_t stream) {
   const int G = nh / nkv;
-  dim3 grid(nsplit, TOKENS ? nkv * (G / NSETS) : nkv, num_items);
-  attention_mfma_kernel<HD, NSETS, TOKENS><<<grid, 64, 0, stream>>>(
+  dim3 grid(nsplit, nkv, num_items);
+  attention_decode_kernel<HD, NSETS><<<grid, 64, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
       positions, req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit,
       split_keys, nh, nkv, ps, scale * 1.4426950408889634f);
@@ -518,8 +515,8 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
       num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream
   if (mode == 0) {
     if (G > 16) return -2;
-    if (hd == 128) return launch<128, 1, false>(TK_ARGS);
-    if (hd == 64) return launch<64, 1, false>(TK_ARGS);
+    if (hd == 128) return launch<128, 1>(TK_ARGS);
+    if (hd == 64) return launch<64, 1>(TK_ARGS);
     return -2;
   }
   if (nsplit != 1) return -1;

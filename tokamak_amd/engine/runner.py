@@ -23,6 +23,8 @@ from tokamak_amd.engine.storage import CacheStorage
 from tokamak_amd.weights.loader import load_weights
 from tokamak_amd.weights.sources import SafetensorsSource
 
+MAX_GRAPHS = 256   # captured decode shapes kept; the one used longest ago goes first
+
 DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32,
           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
 
@@ -142,9 +144,12 @@ class ModelRunner:
         packed = pack_batch(spans, self.num_groups, fixed_widths=widths)
         packed.max_decode_len = pow2_at_least(packed.max_decode_len, 256)
         key = (len(spans), tuple(widths), packed.max_decode_len)
-        graph = self._graphs.get(key)
+        graph = self._graphs.pop(key, None)
         if graph is None:
-            graph = self._graphs[key] = DecodeGraph(self.model, self.storage, packed, self.device)
+            if len(self._graphs) >= MAX_GRAPHS:      # drop the shape used longest ago
+                self._graphs.pop(next(iter(self._graphs)))
+            graph = DecodeGraph(self.model, self.storage, packed, self.device)
+        self._graphs[key] = graph                    # most recently used last
         logits = graph.run(packed)
         if len(wanted) == len(spans):
             return logits
