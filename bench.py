@@ -133,6 +133,52 @@ def time_decode(runner, cfg, batch, context, steps, warmup):
     return elapsed / steps, mean_ctx
 
 
+def run_continuous(args) -> int:
+    """Optional extra workload: continuous batching through ``LLM.generate`` (scheduler,
+    portions of prompts beside decode tokens, captured decode steps).  Prompt lengths
+    uniform in [32, 1024], outputs uniform in [16, 256], greedy, seeded."""
+    import random
+    import tempfile
+
+    import torch
+
+    from tokamak_amd import LLM, SamplingParams
+    from tokamak_amd.models.qwen3 import PRESETS
+    from tokamak_amd.weights import write_random_model
+
+    cfg = dataclasses.replace(PRESETS[args.model], max_position_embeddings=4096)
+    rng = random.Random(0)
+    prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(32, 1024))] for _ in range(args.requests)]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=rng.randint(16, 256), ignore_eos=True)
+              for _ in range(args.requests)]
+    with tempfile.TemporaryDirectory(prefix="tokamak_bench_") as tmp:
+        folder = write_random_model(tmp, cfg, 0)
+        llm = LLM(folder, dtype=args.dtype, max_seq_len=4096, kv_pool_tokens=args.max_batch * 1300,
+                  max_batch_size=args.max_batch, max_num_batched_tokens=2048, prefill_chunk=2048)
+        runs = []
+        for _ in range(2):  # the first run also records the decode graphs
+            steps0 = llm.num_steps
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            outs = llm.generate(prompt_token_ids=prompts, sampling_params=params)
+            torch.cuda.synchronize()
+            runs.append((time.perf_counter() - t0, llm.num_steps - steps0))
+    elapsed, steps = runs[-1]
+    out_tokens = sum(len(o.output_token_ids) for o in outs)
+    print(json.dumps({
+        "metric": f"output tok/s, continuous batching of {args.requests} requests ({args.model}-shaped, random weights)",
+        "value": round(out_tokens / elapsed, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+        "ms_per_step": round(elapsed / steps * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (seeded lengths and token ids, random weights)",
+        "config": {"model": f"{args.model}-shaped", "requests": args.requests, "max_batch": args.max_batch,
+                   "prompt_tokens": sum(map(len, prompts)), "output_tokens": out_tokens,
+                   "first_run_s": round(runs[0][0], 3), "preemptions": llm.num_preemptions,
+                   "parallelism": "single GPU"},
+    }))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -143,10 +189,17 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous"],
+                    help="decode: the headline measurement; continuous: LLM.generate over many requests")
+    ap.add_argument("--model", default="qwen3-0.6b", help="preset shape of the continuous workload")
+    ap.add_argument("--requests", type=int, default=256)
+    ap.add_argument("--max-batch", type=int, default=64)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2
+    if args.workload == "continuous":
+        return run_continuous(args)
 
     import torch
 
