@@ -313,7 +313,7 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
 
   // loader: piece p of K is (group j, dim chunk i, key) = (p / (16*HD/8), (p/16) % (HD/8), p % 16);
   // piece p of V is (group j, dim block, 16-byte piece of the 512-byte run)
-  u32x4 kpre[KPT], vpre[VPT];
+  u32x4 kpre[2][KPT], vpre[2][VPT];
   const int ps_shift = __ffs(ps) - 1;  // page sizes are powers of two here
   // Piece p of a stage belongs to 16-key group j = p / pieces-per-group.  A group past
   // the request's end reads the stage's first group instead (valid memory, masked
@@ -331,35 +331,50 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
     v_j[i] = p / (32 * (HD / 16));
     v_in[i] = ((p / 32) % (HD / 16)) * (ps >> 2) * 64 + (p % 32) * 8;
   }
-#define TK_FETCH(S0)                                                                              \
+  // The four pages of a stage are looked up with wave-uniform indices (scalar loads);
+  // each piece then selects its group's page.  BUF names the register set.
+#define TK_FETCH(S0, BUF)                                                                         \
   {                                                                                               \
+    size_t pbase[4];                                                                              \
+    int poff[4];                                                                                  \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                               \
+      const int c0 = ((S0) + j * 16 <= last_pos) ? (S0) + j * 16 : (S0);                          \
+      pbase[j] = (size_t)table[c0 >> ps_shift] * page_elems + head_off;                           \
+      poff[j] = c0 & (ps - 1);                                                                    \
+    }                                                                                             \
     _Pragma("unroll") for (int i = 0; i < KPT; ++i) {                                             \
-      int c0 = (S0) + k_j[i] * 16;                                                                \
-      c0 = (c0 <= last_pos) ? c0 : (S0);                                                          \
-      const size_t base = (size_t)table[c0 >> ps_shift] * page_elems + head_off;                  \
-      kpre[i] = *reinterpret_cast<const u32x4*>(k_cache + base + (size_t)(c0 & (ps - 1)) * 8 +    \
-                                                k_in[i]);                                         \
+      const int j = k_j[i];                                                                       \
+      const size_t base = j == 0 ? pbase[0] : j == 1 ? pbase[1] : j == 2 ? pbase[2] : pbase[3];   \
+      const int off = j == 0 ? poff[0] : j == 1 ? poff[1] : j == 2 ? poff[2] : poff[3];           \
+      kpre[BUF][i] = *reinterpret_cast<const u32x4*>(k_cache + base + (size_t)off * 8 + k_in[i]); \
     }                                                                                             \
     _Pragma("unroll") for (int i = 0; i < VPT; ++i) {                                             \
-      int c0 = (S0) + v_j[i] * 16;                                                                \
-      c0 = (c0 <= last_pos) ? c0 : (S0);                                                          \
-      const size_t base = (size_t)table[c0 >> ps_shift] * page_elems + head_off;                  \
-      vpre[i] = *reinterpret_cast<const u32x4*>(v_cache + base +                                  \
-                                                (size_t)((c0 & (ps - 1)) >> 2) * 64 + v_in[i]);   \
+      const int j = v_j[i];                                                                       \
+      const size_t base = j == 0 ? pbase[0] : j == 1 ? pbase[1] : j == 2 ? pbase[2] : pbase[3];   \
+      const int off = j == 0 ? poff[0] : j == 1 ? poff[1] : j == 2 ? poff[2] : poff[3];           \
+      vpre[BUF][i] = *reinterpret_cast<const u32x4*>(v_cache + base + (size_t)(off >> 2) * 64 +   \
+                                                     v_in[i]);                                    \
     }                                                                                             \
   }
 
-  TK_FETCH(0)
-  for (int s0 = 0; s0 <= last_pos; s0 += 64) {
+  // Two register sets: while stage s is multiplied, the loads of stages s+1 and s+2 are
+  // in flight, so a stage does not wait a whole memory round trip.
+  TK_FETCH(0, 0)
+  if (64 <= last_pos) TK_FETCH(64, 1)
+  for (int sp = 0; sp <= last_pos; sp += 128) {
+#pragma unroll
+   for (int buf = 0; buf < 2; ++buf) {
+    const int s0 = sp + buf * 64;
+    if (s0 > last_pos) break;
     __syncthreads();  // every wave has read the previous stage
 #pragma unroll
     for (int i = 0; i < KPT; ++i)
-      *reinterpret_cast<u32x4*>(ks + (size_t)(i * THREADS + tid) * 8) = kpre[i];
+      *reinterpret_cast<u32x4*>(ks + (size_t)(i * THREADS + tid) * 8) = kpre[buf][i];
 #pragma unroll
     for (int i = 0; i < VPT; ++i)
-      *reinterpret_cast<u32x4*>(vs + (size_t)(i * THREADS + tid) * 8) = vpre[i];
+      *reinterpret_cast<u32x4*>(vs + (size_t)(i * THREADS + tid) * 8) = vpre[buf][i];
     __syncthreads();
-    if (s0 + 64 <= last_pos) TK_FETCH(s0 + 64)
+    if (s0 + 128 <= last_pos) TK_FETCH(s0 + 128, buf)
 
     // S^T for 4 groups of 16 keys
     float sv[4][4];
@@ -442,6 +457,7 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
       }
       acc[d] = a;
     }
+   }
   }
 
   float l = l_run;
