@@ -179,6 +179,28 @@ def run_continuous(args) -> int:
     return 0
 
 
+def run_phase(args, runner, cfg, full) -> int:
+    """One part alone, so that a profile of the run holds that part's kernels only
+    (the decode part still has to fill the requests' caches first)."""
+    key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    if args.phase == "prefill":
+        seconds = time_prefill(runner, cfg, repeats=max(args.steps, 1))
+        value, steps, what = PREFILL_TOKENS / seconds, max(args.steps, 1), f"prefill tok/s at {PREFILL_TOKENS} tokens"
+    else:
+        seconds, _ = time_decode(runner, cfg, args.batch, args.context, args.steps, args.warmup)
+        value, steps, what = args.batch / seconds, args.steps, f"decode tok/s at batch {args.batch}"
+    print(json.dumps({
+        "metric": f"{what} (Qwen3-8B-shaped, random weights)", "value": round(value, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": round(seconds * 1e3, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": key,
+        "data": "synthetic (uniform random token ids, seeded random weights)",
+        "config": {"model": "qwen3-8b-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers,
+                   "global_batch": args.batch, "seq_len": args.context, "phase": args.phase,
+                   "parallelism": "single GPU"},
+    }))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -189,6 +211,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
+                    help="run only one part (for profiles); the other part's figures are null")
     ap.add_argument("--workload", default="decode", choices=["decode", "continuous"],
                     help="decode: the headline measurement; continuous: LLM.generate over many requests")
     ap.add_argument("--model", default="qwen3-0.6b", help="preset shape of the continuous workload")
@@ -208,10 +232,12 @@ def main() -> int:
     full = PRESETS["qwen3-8b"]
     cfg = dataclasses.replace(full, num_layers=args.layers or full.num_layers)
     elem = 2 if args.dtype == "bfloat16" else 4
-    max_batch = 64 if not args.no_points else args.batch
+    max_batch = 64 if not (args.no_points or args.phase != "all") else args.batch
     pool = max(max_batch, args.batch) * (args.context + 16)
     runner = make_runner(cfg, args.dtype, pool, max(max_batch, args.batch))
 
+    if args.phase != "all":
+        return run_phase(args, runner, cfg, full)
     prefill_s = time_prefill(runner, cfg)
     step_s, mean_ctx = time_decode(runner, cfg, args.batch, args.context, args.steps, args.warmup)
     points = {}

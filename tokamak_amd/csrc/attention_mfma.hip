@@ -250,38 +250,48 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Prompt portions: one block per (16-token tile, kv head, group of HPB query
-// heads), one wave per query head.  The waves share the keys and values: the
-// block copies 64 keys at a time from the pages into LDS (same piece order as in
-// the pages, so every wave reads its MFMA operands back in contiguous 16- and
-// 8-byte pieces without bank conflicts), the next 64 keys already being in
-// flight into registers while the current ones are multiplied.  Per 64 keys a
-// wave does one softmax update: 16 QK^T products (16x16x32), one maximum, one
-// rescale, then 16 PV products (16x16x32 over two 16-key groups at a time: the
-// k index of that product runs over quads of both groups, which is exactly how
-// the lanes hold the probabilities).
+// Prompt portions: one block of four waves per (16-token tile, kv head, group of
+// HPB query heads); wave w < HPB owns query head w of the group, and all four
+// waves load.  The waves share the keys and values: the block copies 64 keys at a
+// time from the pages into LDS, the following stages already being in flight into
+// registers while the current one is multiplied.  K keeps the page's piece order
+// ([dim/8][key][8]); V is regrouped on the way in so that the eight values a lane
+// needs for one PV product (four keys of an even 16-key group, four of the odd one
+// after it, one dim) lie in one 16-byte piece (pieces xor-swizzled against bank
+// conflicts of the 8-byte writes).  Per 64 keys a wave does one softmax
+// update: 16 QK^T products (16x16x32), one maximum, one rescale, then 16 PV
+// products (16x16x32, the k index running over quads of two 16-key groups, which
+// is exactly how the lanes hold the probabilities).
+// Every page lookup is wave-uniform (a piece's 16-key group depends on the wave
+// only), so a load's address is a scalar base plus a per-lane constant.
 // ---------------------------------------------------------------------------
+constexpr int kPrefillThreads = 256;
+
 template <int HD, int HPB>
-__global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
+__global__ __launch_bounds__(kPrefillThreads) __attribute__((amdgpu_waves_per_eu(2)))
+void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ item_token, const int* __restrict__ item_count,
     bf16_t* __restrict__ out, int num_items, int nh, int nkv, int ps, float scale_log2) {
   constexpr int KCH = HD / 32, DBL = HD / 16;
-  constexpr int THREADS = 64 * HPB;
-  constexpr int KPIECES = 4 * (HD / 8) * 16;   // 16-byte pieces of K per stage of 64 keys
-  constexpr int VPIECES = 4 * (HD / 16) * 32;  // and of V
-  constexpr int KPT = KPIECES / THREADS, VPT = VPIECES / THREADS;
-  __shared__ __attribute__((aligned(16))) bf16_t ks[KPIECES * 8];
-  __shared__ __attribute__((aligned(16))) bf16_t vs[VPIECES * 8];
+  constexpr int THREADS = kPrefillThreads;
+  constexpr int GROUP_PIECES = 2 * HD;         // 16-byte pieces of K (and of V) per 16-key group
+  constexpr int PIECES = 4 * GROUP_PIECES;     // per stage of 64 keys
+  constexpr int PPT = PIECES / THREADS;        // pieces of K, and of V, per thread and stage
+  constexpr int NBUF = 1;                      // register sets of prefetch
+  static_assert(GROUP_PIECES % 64 == 0, "a wave's pieces of one load lie in one 16-key group");
+  __shared__ __attribute__((aligned(16))) bf16_t ks[PIECES * 8];
+  __shared__ __attribute__((aligned(16))) bf16_t vs[PIECES * 8];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, kb = lane >> 4;
   const int G = nh / nkv;
   const int groups_per_kv = G / HPB;
   const int kvh = blockIdx.x / groups_per_kv;
-  const int head = kvh * G + (blockIdx.x % groups_per_kv) * HPB + wave;
+  const bool computes = wave < HPB;
+  const int head = kvh * G + (blockIdx.x % groups_per_kv) * HPB + (computes ? wave : 0);
   const int item = num_items - 1 - blockIdx.y;  // later tiles have more keys: start them first
 
   const int n0 = item_token[item];
@@ -311,70 +321,86 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
 #pragma unroll
   for (int d = 0; d < DBL; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  // loader: piece p of K is (group j, dim chunk i, key) = (p / (16*HD/8), (p/16) % (HD/8), p % 16);
-  // piece p of V is (group j, dim block, 16-byte piece of the 512-byte run)
-  u32x4 kpre[2][KPT], vpre[2][VPT];
+  // Piece p = i * THREADS + tid of a stage.  K: (group j, dim chunk c8, key) =
+  // (p / GROUP_PIECES, (p / 16) % (HD/8), p % 16).  V: (group j, dim block d, quad, dim
+  // pair) = (p / GROUP_PIECES, (p / 32) % DBL, (p % 32) / 8, p % 8): two dims x four keys.
+  u32x4 kpre[NBUF][PPT], vpre[NBUF][PPT];
   const int ps_shift = __ffs(ps) - 1;  // page sizes are powers of two here
-  // Piece p of a stage belongs to 16-key group j = p / pieces-per-group.  A group past
-  // the request's end reads the stage's first group instead (valid memory, masked
-  // later), so no load is predicated and all of a stage's loads are in flight together.
-  int k_j[KPT], k_in[KPT], v_j[VPT], v_in[VPT];
+  int grp[PPT];                        // wave-uniform
+  unsigned k_in[PPT], v_in[PPT];       // byte offset inside the page's head, for key 0 of a group
+  int v_quad[PPT];
+  unsigned v_lds[PPT][2];              // element offsets in vs of the piece's two dims
 #pragma unroll
-  for (int i = 0; i < KPT; ++i) {
+  for (int i = 0; i < PPT; ++i) {
     const int p = i * THREADS + tid;
-    k_j[i] = p / (16 * (HD / 8));
-    k_in[i] = (((p / 16) % (HD / 8)) * ps + (p % 16)) * 8;  // element offset inside the page's head
-  }
+    grp[i] = __builtin_amdgcn_readfirstlane(p / GROUP_PIECES);
+    k_in[i] = (unsigned)((((p / 16) % (HD / 8)) * ps + (p % 16)) * 8) * 2u;
+    const int d = (p / 32) % DBL, quad = (p % 32) / 8, dp = p % 8;
+    v_in[i] = (unsigned)(d * (ps >> 2) * 64 + (p % 32) * 8) * 2u;
+    v_quad[i] = quad;
+    // vs: [pair of groups h][d][quad][slot = dim col ^ quad][group parity][4 keys]; the
+    // xor spreads a wave's 8-byte writes over all banks and keeps the reads contiguous
 #pragma unroll
-  for (int i = 0; i < VPT; ++i) {
-    const int p = i * THREADS + tid;
-    v_j[i] = p / (32 * (HD / 16));
-    v_in[i] = ((p / 32) % (HD / 16)) * (ps >> 2) * 64 + (p % 32) * 8;
+    for (int half = 0; half < 2; ++half)
+      v_lds[i][half] = (unsigned)((((((p / GROUP_PIECES) >> 1) * DBL + d) * 4 + quad) * 16 +
+                                   ((2 * dp + half) ^ quad)) * 2 + ((p / GROUP_PIECES) & 1)) * 4u;
   }
-  // The four pages of a stage are looked up with wave-uniform indices (scalar loads);
-  // each piece then selects its group's page.  BUF names the register set.
-#define TK_FETCH(S0, BUF)                                                                         \
-  {                                                                                               \
-    size_t pbase[4];                                                                              \
-    int poff[4];                                                                                  \
-    _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                               \
-      const int c0 = ((S0) + j * 16 <= last_pos) ? (S0) + j * 16 : (S0);                          \
-      pbase[j] = (size_t)table[c0 >> ps_shift] * page_elems + head_off;                           \
-      poff[j] = c0 & (ps - 1);                                                                    \
-    }                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < KPT; ++i) {                                             \
-      const int j = k_j[i];                                                                       \
-      const size_t base = j == 0 ? pbase[0] : j == 1 ? pbase[1] : j == 2 ? pbase[2] : pbase[3];   \
-      const int off = j == 0 ? poff[0] : j == 1 ? poff[1] : j == 2 ? poff[2] : poff[3];           \
-      kpre[BUF][i] = *reinterpret_cast<const u32x4*>(k_cache + base + (size_t)off * 8 + k_in[i]); \
-    }                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < VPT; ++i) {                                             \
-      const int j = v_j[i];                                                                       \
-      const size_t base = j == 0 ? pbase[0] : j == 1 ? pbase[1] : j == 2 ? pbase[2] : pbase[3];   \
-      const int off = j == 0 ? poff[0] : j == 1 ? poff[1] : j == 2 ? poff[2] : poff[3];           \
-      vpre[BUF][i] = *reinterpret_cast<const u32x4*>(v_cache + base + (size_t)(off >> 2) * 64 +   \
-                                                     v_in[i]);                                    \
-    }                                                                                             \
+  // A group past the request's end reads the stage's first group instead (valid
+  // memory, masked later), so no load is predicated and all of a stage's loads are
+  // in flight together.  The page numbers of a stage are looked up one fetch ahead
+  // (scalar loads), so their latency is never waited for.
+  int page_next[PPT];  // of the 16-key group of this wave's piece i
+#define TK_PAGES(S0)                                                             \
+  if ((S0) <= last_pos) {                                                        \
+    _Pragma("unroll") for (int i = 0; i < PPT; ++i) {                            \
+      const int c0 = ((S0) + grp[i] * 16 <= last_pos) ? (S0) + grp[i] * 16 : (S0); \
+      page_next[i] = table[c0 >> ps_shift];                                      \
+    }                                                                            \
+  }
+#define TK_FETCH(S0, BUF)                                                                        \
+  {                                                                                              \
+    _Pragma("unroll") for (int i = 0; i < PPT; ++i) {                                            \
+      const int c0 = ((S0) + grp[i] * 16 <= last_pos) ? (S0) + grp[i] * 16 : (S0);               \
+      const size_t pg = (size_t)__builtin_amdgcn_readfirstlane(page_next[i]) * page_elems + head_off; \
+      const int off = c0 & (ps - 1);                                                             \
+      const char* kp = reinterpret_cast<const char*>(k_cache + pg + (size_t)off * 8);            \
+      const char* vp = reinterpret_cast<const char*>(v_cache + pg + (size_t)(off >> 2) * 64);    \
+      kpre[BUF][i] = *reinterpret_cast<const u32x4*>(kp + k_in[i]);                              \
+      vpre[BUF][i] = *reinterpret_cast<const u32x4*>(vp + v_in[i]);                              \
+    }                                                                                            \
+    TK_PAGES((S0) + 64)                                                                          \
   }
 
-  // Two register sets: while stage s is multiplied, the loads of stages s+1 and s+2 are
-  // in flight, so a stage does not wait a whole memory round trip.
-  TK_FETCH(0, 0)
-  if (64 <= last_pos) TK_FETCH(64, 1)
-  for (int sp = 0; sp <= last_pos; sp += 128) {
+  TK_PAGES(0)
 #pragma unroll
-   for (int buf = 0; buf < 2; ++buf) {
+  for (int b = 0; b < NBUF; ++b)
+    if (b == 0 || b * 64 <= last_pos) TK_FETCH(b * 64, b)
+  for (int sp = 0; sp <= last_pos; sp += 64 * NBUF) {
+#pragma unroll
+   for (int buf = 0; buf < NBUF; ++buf) {
     const int s0 = sp + buf * 64;
     if (s0 > last_pos) break;
     __syncthreads();  // every wave has read the previous stage
+    if (s0 + 63 > last_pos) {
+      // keys past the request's end may hold anything (their probability is zero, but
+      // 0 * NaN is NaN): zero their values on the way into LDS
 #pragma unroll
-    for (int i = 0; i < KPT; ++i)
+      for (int i = 0; i < PPT; ++i) {
+        const int k0 = s0 + grp[i] * 16 + v_quad[i] * 4;
+        const unsigned m01 = (k0 + 0 > last_pos ? 0u : 0x0000ffffu) | (k0 + 1 > last_pos ? 0u : 0xffff0000u);
+        const unsigned m23 = (k0 + 2 > last_pos ? 0u : 0x0000ffffu) | (k0 + 3 > last_pos ? 0u : 0xffff0000u);
+        vpre[buf][i] &= u32x4{m01, m23, m01, m23};
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
       *reinterpret_cast<u32x4*>(ks + (size_t)(i * THREADS + tid) * 8) = kpre[buf][i];
-#pragma unroll
-    for (int i = 0; i < VPT; ++i)
-      *reinterpret_cast<u32x4*>(vs + (size_t)(i * THREADS + tid) * 8) = vpre[buf][i];
+      *reinterpret_cast<uint2*>(vs + v_lds[i][0]) = make_uint2(vpre[buf][i][0], vpre[buf][i][1]);
+      *reinterpret_cast<uint2*>(vs + v_lds[i][1]) = make_uint2(vpre[buf][i][2], vpre[buf][i][3]);
+    }
     __syncthreads();
-    if (s0 + 128 <= last_pos) TK_FETCH(s0 + 128, buf)
+    if (s0 + 64 * NBUF <= last_pos) TK_FETCH(s0 + 64 * NBUF, buf)
+    if (!computes) continue;
 
     // S^T for 4 groups of 16 keys
     float sv[4][4];
@@ -428,31 +454,18 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
     }
     l_run = l_run * alpha + psum;
     // the accumulators need rescaling only when some column's maximum moved
-    const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
-    const bool tail = s0 + 63 > last_pos;  // keys past the end may hold anything: zero their values
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+      for (int d = 0; d < DBL; ++d) acc[d] *= alpha;
+    }
 #pragma unroll
     for (int d = 0; d < DBL; ++d) {
       float4v a = acc[d];
-      if (rescale) {
-        a[0] *= alpha;
-        a[1] *= alpha;
-        a[2] *= alpha;
-        a[3] *= alpha;
-      }
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         // A operand: V^T[dim col][k], k = (group 2h quad kb) then (group 2h+1 quad kb)
-        uint2 lo = *reinterpret_cast<const uint2*>(vs + ((size_t)((2 * h) * DBL + d) * 4 + kb) * 64 + col * 4);
-        uint2 hi = *reinterpret_cast<const uint2*>(vs + ((size_t)((2 * h + 1) * DBL + d) * 4 + kb) * 64 + col * 4);
-        if (tail) {
-          const int k0 = s0 + (2 * h) * 16 + kb * 4, k1 = k0 + 16;
-          lo.x &= (k0 + 0 > last_pos ? 0u : 0x0000ffffu) | (k0 + 1 > last_pos ? 0u : 0xffff0000u);
-          lo.y &= (k0 + 2 > last_pos ? 0u : 0x0000ffffu) | (k0 + 3 > last_pos ? 0u : 0xffff0000u);
-          hi.x &= (k1 + 0 > last_pos ? 0u : 0x0000ffffu) | (k1 + 1 > last_pos ? 0u : 0xffff0000u);
-          hi.y &= (k1 + 2 > last_pos ? 0u : 0x0000ffffu) | (k1 + 3 > last_pos ? 0u : 0xffff0000u);
-        }
         Frag8 vf;
-        vf.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        vf.u = *reinterpret_cast<const uint4*>(vs + ((size_t)((h * DBL + d) * 4 + kb) * 16 + (col ^ kb)) * 8);
         a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pb[h].v, a, 0, 0, 0);
       }
       acc[d] = a;
@@ -463,7 +476,7 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
   float l = l_run;
   l += __shfl_xor(l, 16, kWave);
   l += __shfl_xor(l, 32, kWave);
-  if (c_valid) {
+  if (c_valid && computes) {
     const float inv = 1.f / l;
     bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * HD + kb * 4;
 #pragma unroll
@@ -477,6 +490,7 @@ __global__ __launch_bounds__(64 * HPB) void attention_prefill_kernel(
 }
 
 #undef TK_FETCH
+#undef TK_PAGES
 
 template <int HD, int HPB>
 static int launch_prefill(const void* q, const void* k_cache, const void* v_cache,
@@ -486,7 +500,7 @@ static int launch_prefill(const void* q, const void* k_cache, const void* v_cach
                           hipStream_t stream) {
   const int G = nh / nkv;
   dim3 grid(nkv * (G / HPB), num_items);
-  attention_prefill_kernel<HD, HPB><<<grid, 64 * HPB, 0, stream>>>(
+  attention_prefill_kernel<HD, HPB><<<grid, kPrefillThreads, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
       positions, req_of_token, item_token, item_count, (bf16_t*)out, num_items, nh, nkv, ps,
       scale * 1.4426950408889634f);
