@@ -1,7 +1,9 @@
 """Layers of Qwen3-8B's shape (width 4096, 32 query and 8 kv heads of 128, feed-forward
-12288; two layers and a vocabulary of 8192 to keep it small): float32 and bfloat16
-logits against the plain implementation, whole, in portions and token by token, and
-mixed with a second request."""
+12288; two layers and a vocabulary of 8192 to keep it small), of Qwen3-32B's (width 5120,
+64 query heads in groups of 8, feed-forward 25600; one layer) and of Qwen3-0.6B's (width
+1024, 16 query heads in groups of 2, tied embeddings): float32 and bfloat16 logits
+against the plain implementation, whole, in portions and token by token, and mixed
+with a second request."""
 
 import dataclasses
 
@@ -15,12 +17,14 @@ from tokamak_amd.models import qwen3
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def model():
+@pytest.fixture(scope="module", params=[("qwen3-8b", 2), ("qwen3-32b", 1), ("qwen3-0.6b", 2)],
+                ids=["8b", "32b", "0.6b"])
+def model(request):
     from tokamak_amd.weights.random_init import expected_tensors_of
     from tokamak_amd.weights.sources import RandomSource
 
-    cfg = dataclasses.replace(qwen3.PRESETS["qwen3-8b"], num_layers=2, vocab_size=8192, max_position_embeddings=4096)
+    preset, layers = request.param
+    cfg = dataclasses.replace(qwen3.PRESETS[preset], num_layers=layers, vocab_size=8192, max_position_embeddings=4096)
     plan = qwen3.plan(cfg)
     expected = {n: s for n, s in expected_tensors_of(plan).items() if not s.ignored}
     source = RandomSource(expected, seed=3, matrix_std=0.02, vector_jitter=0.1, dtype=torch.bfloat16)
@@ -37,7 +41,7 @@ def model():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_8b_shaped_layers_match_plain_under_every_cutting(model, dtype):
+def test_full_width_layers_match_plain_under_every_cutting(model, dtype):
     from tokamak_amd.engine.runner import ModelRunner, StepEntry
 
     cfg, plan, source, w = model
