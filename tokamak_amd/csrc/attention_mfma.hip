@@ -24,12 +24,16 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
 union Frag8 {
   uint4 u;
+  u32x4 w;
   bf16x8 v;
 };
 union Frag4 {
   uint2 u;
+  u32x2 w;
   short4v v;
 };
 
@@ -103,13 +107,13 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16_t* kp = k_cache + (size_t)page * page_elems + head_off + (size_t)(off + col) * 8;
 #pragma unroll
     for (int c = 0; c < KCH; ++c)
-      kreg[c].u = *reinterpret_cast<const uint4*>(kp + (size_t)(c * 4 + kb) * ps * 8);
+      kreg[c].w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp + (size_t)(c * 4 + kb) * ps * 8));
     // V page [hd/16][ps/4][16][4]: lane (dim col, quad kb) of block d reads 8 bytes, the
     // wave 512 contiguous bytes
     const bf16_t* vp = v_cache + (size_t)page * page_elems + head_off + (size_t)((off >> 2) + kb) * 64 + col * 4;
 #pragma unroll
     for (int d = 0; d < DBL; ++d)
-      vreg[d].u = *reinterpret_cast<const uint2*>(vp + (size_t)d * (ps >> 2) * 64);
+      vreg[d].w = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(vp + (size_t)d * (ps >> 2) * 64));
   };
 
   load_tile(k_begin);

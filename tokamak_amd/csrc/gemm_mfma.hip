@@ -261,7 +261,8 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
     const bool kw = k0 + w_col < K, kx = k0 + x_col < K;
     const int wo = kw ? k0 + w_col : 0, xo = kx ? k0 + x_col : 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) wreg[i] = *reinterpret_cast<const u32x4*>(wrow[i] + wo);
+    for (int i = 0; i < 8; ++i)  // weights are read once: streaming loads leave the caches to the activations
+      wreg[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[i] + wo));
 #pragma unroll
     for (int i = 0; i < 2 * MT; ++i) xreg[i] = *reinterpret_cast<const u32x4*>(xrow[i] + xo);
     if (k0 + SBK > K) {
