@@ -39,13 +39,35 @@ class LLM:
         max_batch_size: most sequences running at once.
         max_num_batched_tokens: token budget of one step (new).
         prefill_chunk: longest prompt portion in one step (new; default the budget).
+        device: ``"auto"`` or a cuda device; there is no CPU path.
+        kv_backend, scheduling, attention_backend, attention_policy, draft_model: the
+            reference's further options; this engine has one choice for each
+            (``"paged"``, ``"continuous"``, ``"auto"``, ``"full"``, ``None``) and
+            refuses any other with a clear error.
     """
 
-    def __init__(self, model: str | Path, *, dtype: str | torch.dtype = "bfloat16",
+    _ONLY = {"kv_backend": ("paged",), "scheduling": ("continuous",),
+             "attention_backend": ("auto", "hip"), "attention_policy": ("full",), "draft_model": (None,)}
+
+    def __init__(self, model: str | Path, *, dtype: str | torch.dtype = "auto",
                  max_seq_len: int | None = None, block_size: int = 16,
                  kv_pool_tokens: int | None = None, max_batch_size: int = 16,
                  max_num_batched_tokens: int = 2048, prefill_chunk: int | None = None,
-                 device: str | torch.device = "cuda:0") -> None:
+                 device: str | torch.device = "auto", kv_backend: str = "paged",
+                 scheduling: str = "continuous", attention_backend: str = "auto",
+                 attention_policy: str = "full", draft_model=None) -> None:
+        given = {"kv_backend": kv_backend, "scheduling": scheduling, "attention_backend": attention_backend,
+                 "attention_policy": attention_policy, "draft_model": draft_model}
+        for name, value in given.items():
+            if value not in self._ONLY[name]:
+                raise ValueError(f"{name}={value!r} is not supported by this engine; "
+                                 f"supported: {', '.join(map(repr, self._ONLY[name]))}")
+        if dtype == "auto":
+            dtype = "bfloat16"
+        if device == "auto":
+            device = "cuda:0"
+        if torch.device(device).type != "cuda":
+            raise ValueError(f"device={device!r}: this engine runs on the GPU only")
         if block_size < 1:
             raise ValueError(f"block_size must be >= 1, got {block_size}")
         if max_batch_size < 1:
