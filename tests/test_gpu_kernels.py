@@ -319,6 +319,30 @@ def test_streaming_product_and_its_partial_sums(M, N, K):
             assert parts[0].abs().max() > 0 and not torch.allclose(parts[0].cpu().double(), want, rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("M, N, K", [(65, 64, 64), (300, 1000, 512), (2048, 331, 200), (129, 4096, 1024), (130, 4096, 1024)])
+def test_library_product_with_kept_plans_and_measured_algorithms(M, N, K):
+    """The hipBLASLt path for more than 64 rows: right for sizes that are no power of
+    two, the same on every call (the plan and the algorithm are kept), and two shapes
+    of one class (129 and 130 rows) share the algorithm that was measured for the first."""
+    from tokamak_amd.kernels import ops
+
+    x = rand(M, K, seed=1).to(torch.bfloat16)
+    w = rand(N, K, seed=2, scale=K ** -0.5).to(torch.bfloat16)
+    want = x.double() @ w.double().T
+    outs = []
+    for _ in range(3):
+        out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        assert ops.gemm_library(x.to(DEV), w.to(DEV), out)
+        outs.append(out.cpu())
+        torch.testing.assert_close(outs[-1].double(), want, rtol=2e-2, atol=1e-2)
+    assert torch.equal(outs[1], outs[2])
+    # a view with a row stride (the fused qkv output is sliced like this)
+    wide = torch.full((M, N + 64), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert ops.gemm_library(x.to(DEV), w.to(DEV), wide[:, :N])
+    torch.testing.assert_close(wide[:, :N].cpu().double(), want, rtol=2e-2, atol=1e-2)
+    assert torch.isnan(wide[:, N:]).all()
+
+
 def test_consumers_add_partial_sums():
     """The norm kernel and the q/k norm kernel take a split-K product's partial
     sums and add them in float32."""

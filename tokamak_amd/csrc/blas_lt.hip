@@ -1,0 +1,152 @@
+// Library matrix product for prompt portions of more than 64 tokens:
+//   out[M, N] = x[M, K] . w[N, K]^T     bf16 in, float32 accumulation, bf16 out
+// through hipBLASLt, as the reference uses nn.Linear (src/tokamak/model/layers.py:103,
+// src/tokamak/model/transformer.py:67-69,85).  Host code only.
+//
+// Two things a generic call path does not do:
+//  * the plan of a shape (descriptors, algorithm, workspace need) is made once and
+//    kept, so a call costs a map lookup and one launch;
+//  * the algorithm is chosen by measurement: the first time a shape class (N, K, M
+//    rounded up to 128) is seen, the library's candidates for it are each run a few
+//    times on the caller's operands and the fastest is kept for the class.  The
+//    library's own first choice is often not the fastest (by up to 2x for some of
+//    this model's shapes).  The numbers an algorithm computes do not depend on the
+//    others that were tried.
+#include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
+
+#include <cstdint>
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <vector>
+
+#define TK_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+struct Plan {
+  hipblasLtMatmulDesc_t desc = nullptr;
+  hipblasLtMatrixLayout_t lw = nullptr, lx = nullptr, lo = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+};
+
+using ShapeKey = std::tuple<int, int, int, long, long, long>;  // M, N, K, ldx, ldw, ldo
+using ClassKey = std::tuple<int, int, int>;                    // ceil(M / 128), N, K
+
+std::mutex g_lock;
+hipblasLtHandle_t g_handle = nullptr;
+std::map<ShapeKey, Plan> g_plans;
+std::map<ClassKey, hipblasLtMatmulAlgo_t> g_class_algo;
+long g_tuned = 0;
+
+constexpr int kMaxCandidates = 32;
+constexpr int kClassRows = 128;
+
+int make_descriptors(Plan& p, int M, int N, int K, long ldx, long ldw, long ldo) {
+  // column-major view: out^T [N, M] = (w^T)^T [N, K] . x^T [K, M]
+  if (hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) != HIPBLAS_STATUS_SUCCESS) return -10;
+  hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+  hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta));
+  hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb));
+  if (hipblasLtMatrixLayoutCreate(&p.lw, HIP_R_16BF, K, N, ldw) != HIPBLAS_STATUS_SUCCESS) return -11;
+  if (hipblasLtMatrixLayoutCreate(&p.lx, HIP_R_16BF, K, M, ldx) != HIPBLAS_STATUS_SUCCESS) return -11;
+  if (hipblasLtMatrixLayoutCreate(&p.lo, HIP_R_16BF, N, M, ldo) != HIPBLAS_STATUS_SUCCESS) return -11;
+  return 0;
+}
+
+bool usable(const Plan& p, hipblasLtMatmulAlgo_t& algo, size_t ws_bytes) {
+  const float alpha = 1.f, beta = 0.f;
+  size_t need = 0;
+  return hipblaslt_ext::matmulIsAlgoSupported(g_handle, p.desc, &alpha, p.lw, p.lx, &beta, p.lo, p.lo,
+                                              algo, need) == HIPBLAS_STATUS_SUCCESS &&
+         need <= ws_bytes;
+}
+
+hipblasStatus_t run(const Plan& p, hipblasLtMatmulAlgo_t& algo, const void* x, const void* w, void* out,
+                    void* ws, size_t ws_bytes, hipStream_t stream) {
+  const float alpha = 1.f, beta = 0.f;
+  return hipblasLtMatmul(g_handle, p.desc, &alpha, w, p.lw, x, p.lx, &beta, out, p.lo, out, p.lo, &algo,
+                         ws, ws_bytes, stream);
+}
+
+}  // namespace
+
+// tune: how many of the library's candidates to time for a new shape class (<= 1: take
+// its first choice).  Returns 0, or a negative code: -1 bad arguments, -2 no algorithm,
+// -3 the product failed, -10/-11 descriptor creation.
+TK_API int tk_lt_gemm(const void* x, const void* w, void* out, int M, int N, int K, long ldx, long ldw,
+                      long ldo, void* workspace, size_t ws_bytes, int tune, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || ldx < K || ldw < K || ldo < N) return -1;
+  std::lock_guard<std::mutex> guard(g_lock);
+  if (g_handle == nullptr && hipblasLtCreate(&g_handle) != HIPBLAS_STATUS_SUCCESS) return -10;
+
+  const ShapeKey key{M, N, K, ldx, ldw, ldo};
+  auto it = g_plans.find(key);
+  if (it == g_plans.end()) {
+    Plan p;
+    if (const int err = make_descriptors(p, M, N, K, ldx, ldw, ldo)) return err;
+    const ClassKey cls{(M + kClassRows - 1) / kClassRows, N, K};
+    auto known = g_class_algo.find(cls);
+    bool have = false;
+    if (known != g_class_algo.end()) {
+      p.algo = known->second;
+      have = usable(p, p.algo, ws_bytes);
+    }
+    if (!have) {
+      hipblasLtMatmulPreference_t pref;
+      if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return -10;
+      uint64_t cap = ws_bytes;
+      hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &cap, sizeof(cap));
+      const int want = tune > 1 ? (tune < kMaxCandidates ? tune : kMaxCandidates) : 1;
+      std::vector<hipblasLtMatmulHeuristicResult_t> found(want);
+      int got = 0;
+      const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.lw, p.lx, p.lo, p.lo, pref,
+                                                                 want, found.data(), &got);
+      hipblasLtMatmulPreferenceDestroy(pref);
+      if (st != HIPBLAS_STATUS_SUCCESS || got <= 0) return -2;
+      int best = -1;
+      if (got > 1) {
+        hipEvent_t e0, e1;
+        hipEventCreate(&e0);
+        hipEventCreate(&e1);
+        float best_ms = 0.f;
+        for (int i = 0; i < got; ++i) {
+          if (found[i].state != HIPBLAS_STATUS_SUCCESS || found[i].workspaceSize > ws_bytes) continue;
+          if (run(p, found[i].algo, x, w, out, workspace, ws_bytes, stream) != HIPBLAS_STATUS_SUCCESS) continue;
+          hipEventRecord(e0, stream);
+          bool ok = true;
+          for (int r = 0; r < 3 && ok; ++r)
+            ok = run(p, found[i].algo, x, w, out, workspace, ws_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
+          hipEventRecord(e1, stream);
+          if (hipEventSynchronize(e1) != hipSuccess || !ok) continue;
+          float ms = 0.f;
+          hipEventElapsedTime(&ms, e0, e1);
+          if (best < 0 || ms < best_ms) {
+            best = i;
+            best_ms = ms;
+          }
+        }
+        hipEventDestroy(e0);
+        hipEventDestroy(e1);
+        ++g_tuned;
+      } else if (found[0].state == HIPBLAS_STATUS_SUCCESS && found[0].workspaceSize <= ws_bytes) {
+        best = 0;
+      }
+      if (best < 0) return -2;
+      p.algo = found[best].algo;
+      if (got > 1) g_class_algo[cls] = p.algo;
+    }
+    it = g_plans.emplace(key, p).first;
+  }
+  Plan& p = it->second;
+  return run(p, p.algo, x, w, out, workspace, ws_bytes, stream) == HIPBLAS_STATUS_SUCCESS ? 0 : -3;
+}
+
+// How many shape classes have been tuned by measurement so far (for tests and logs).
+TK_API long tk_lt_tuned_classes() {
+  std::lock_guard<std::mutex> guard(g_lock);
+  return g_tuned;
+}

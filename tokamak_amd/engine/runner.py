@@ -20,6 +20,7 @@ from tokamak_amd.engine.batch import StepBatch, StepSpan, batch_from_device, pac
 from tokamak_amd.engine.decode_graph import DecodeGraph, pow2_at_least
 from tokamak_amd.engine.model import LayeredModel
 from tokamak_amd.engine.storage import CacheStorage
+from tokamak_amd.kernels import ops
 from tokamak_amd.weights.loader import load_weights
 from tokamak_amd.weights.sources import SafetensorsSource
 
@@ -167,7 +168,8 @@ class ModelRunner:
                     and all(list(e.want) in ([], [0]) for e in entries)):
                 logits = self._graph_step(entries)
             else:
-                logits = self.model.forward(self.prepare(entries), self.storage)
+                with ops.pinned_stream():
+                    logits = self.model.forward(self.prepare(entries), self.storage)
         for e in entries:
             self._ctx_len[e.request] += len(e.tokens)
         return logits

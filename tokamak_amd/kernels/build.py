@@ -29,7 +29,9 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
 ]
 LIBRARIES = ("elementwise", "gemm_tiled", "attention_generic", "sampling", "gemm_mfma",
-             "attention_mfma")
+             "attention_mfma", "blas_lt")
+# libraries a source links against (blas_lt is host code around hipBLASLt)
+LINK_FLAGS = {"blas_lt": ["-lhipblaslt"]}
 
 _loaded: dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -48,7 +50,7 @@ def sources_of(name: str) -> list[Path]:
 
 def _digest(name: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join([*HIPCC_FLAGS, *LINK_FLAGS.get(name, [])]).encode())
     for path in sources_of(name):
         h.update(path.name.encode())
         h.update(path.read_bytes())
@@ -86,7 +88,8 @@ def compile_library(name: str, *, quiet: bool = False) -> Path:
     out_dir = CSRC if os.access(CSRC, os.W_OK) else _fallback_dir()
     lib = out_dir / f"libtk_{name}.so"
     tmp = out_dir / f".libtk_{name}.{os.getpid()}.so"
-    cmd = [hipcc, *HIPCC_FLAGS, f"-I{CSRC}", str(CSRC / f"{name}.hip"), "-o", str(tmp)]
+    cmd = [hipcc, *HIPCC_FLAGS, f"-I{CSRC}", str(CSRC / f"{name}.hip"), "-o", str(tmp),
+           *LINK_FLAGS.get(name, [])]
     if not quiet:
         print(f"[tokamak_amd] compiling {name}.hip for {ARCH} ...", file=sys.stderr, flush=True)
     start = time.time()

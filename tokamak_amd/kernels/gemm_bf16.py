@@ -53,8 +53,8 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype, allow_pa
     weight-streaming MFMA kernels: the LDS-staged one, split over K into partial
     sums when the matrix has few rows and the caller adds them; the
     direct-operand one for very small matrices.  More than 64 rows
-    with bfloat16 output: the library product torch binds (as the reference's
-    nn.Linear does); with float32 output: 64 rows at a time.
+    with bfloat16 output: the library product (hipBLASLt, as the reference's
+    nn.Linear ends in a library; csrc/blas_lt.hip); with float32 output: 64 rows at a time.
     """
     m = x.shape[0]
     n, k = weight.shape
@@ -77,7 +77,10 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype, allow_pa
         return out
     out = torch.empty((m, n), dtype=out_dtype, device=dev)
     if out_dtype == torch.bfloat16:
-        torch.matmul(x, weight.t(), out=out)
+        # hipBLASLt with kept plans and measured algorithms; shapes it has nothing for
+        # (rows that are not 16-byte aligned, say) go through torch's binding of it
+        if not (skinny_fits(x, weight) and ops.gemm_library(x, weight, out)):
+            torch.matmul(x, weight.t(), out=out)
     else:
         ops.gemm_tiled(x, weight, out)
     return out

@@ -9,7 +9,7 @@ compiled library the call raises.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_float, c_int, c_long, c_void_p
+from ctypes import c_float, c_int, c_long, c_size_t, c_void_p
 
 import torch
 
@@ -33,8 +33,28 @@ def _p(t: torch.Tensor | None) -> c_void_p:
     return c_void_p(0 if t is None else t.data_ptr())
 
 
+_pinned_stream: c_void_p | None = None
+
+
 def _stream() -> c_void_p:
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+    return _pinned_stream if _pinned_stream is not None else c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class pinned_stream:
+    """Within the block every kernel of this module is launched on the stream that is
+    current at entry, without asking torch for it launch by launch (that lookup costs
+    more than the launch).  The caller must not switch streams inside the block."""
+
+    def __enter__(self):
+        global _pinned_stream
+        self._before = _pinned_stream
+        _pinned_stream = c_void_p(torch.cuda.current_stream().cuda_stream)
+        return self
+
+    def __exit__(self, *exc):
+        global _pinned_stream
+        _pinned_stream = self._before
+        return False
 
 
 def _need(cond: bool, msg: str) -> None:
@@ -77,6 +97,10 @@ _SIGS = {
                                   c_void_p],
         "tk_gemm_skinny": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                            c_long, c_int, c_int, c_void_p],
+    },
+    "blas_lt": {
+        "tk_lt_gemm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p,
+                       c_size_t, c_int, c_void_p],
     },
     "attention_generic": {
         "tk_paged_attention_generic": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -269,6 +293,35 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> N
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gated product needs M <= 64 and 16-byte aligned rows")
     _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
                                                      w.stride(0), out.stride(0), _stream()), "gemm_stream_swiglu")
+
+
+LT_WORKSPACE_BYTES = 128 << 20
+LT_TUNE_CANDIDATES = 16
+_lt_workspace: dict[torch.device, torch.Tensor] = {}
+
+
+def gemm_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+    """out[M, N] = a[M, K] @ w[N, K]^T through hipBLASLt (bf16 in and out, float32
+    accumulation), for prompt portions too long for the weight-streaming kernels.
+    The plan of each shape is kept, and the algorithm of a shape class is chosen by
+    timing the library's candidates once (csrc/blas_lt.hip).  Synchronises the first
+    time a shape class is seen, so it must not be recorded into a graph.  Returns
+    False if the library has no algorithm for the shape (nothing was computed)."""
+    for t in (a, w, out):
+        _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
+        _need(t.dtype == torch.bfloat16 and t.data_ptr() % 16 == 0, "the library product is bfloat16 with 16-byte aligned operands")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and out.shape == (m, n), "gemm shapes disagree")
+    ws = _lt_workspace.get(a.device)
+    if ws is None:
+        ws = _lt_workspace[a.device] = torch.empty(LT_WORKSPACE_BYTES, dtype=torch.uint8, device=a.device)
+    status = _fn("blas_lt", "tk_lt_gemm")(_p(a), _p(w), _p(out), m, n, k, a.stride(0), w.stride(0), out.stride(0),
+                                          _p(ws), ws.numel(), LT_TUNE_CANDIDATES, _stream())
+    if status == -2:
+        return False
+    _check(status, "gemm_library")
+    return True
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, row_tiles: int, waves: int) -> None:
