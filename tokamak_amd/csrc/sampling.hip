@@ -14,30 +14,53 @@
 using namespace tk;
 
 // ---------------------------------------------------------------------------
-// argmax: first maximum wins (lowest index), NaN never wins
+// argmax: first maximum wins (lowest index), NaN never wins.  A row is cut into
+// kArgmaxSegments pieces, one block each, so that a few rows still fill the chip;
+// a second small kernel picks among the pieces' winners.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ logits,
-                                                      int* __restrict__ out, int V, long ld) {
-  __shared__ float best_v[16];
-  __shared__ int best_i[16];
-  const float* row = logits + (size_t)blockIdx.x * ld;
+constexpr int kArgmaxSegments = 32;
+constexpr int kArgmaxThreads = 256;
+
+__device__ __forceinline__ void argmax_take(float& bv, int& bi, float v, int i) {
+  if (v > bv || (v == bv && i < bi)) {
+    bv = v;
+    bi = i;
+  }
+}
+
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_segments_kernel(
+    const float* __restrict__ logits, float* __restrict__ part_v, int* __restrict__ part_i, int V,
+    long ld) {
+  __shared__ float best_v[kArgmaxThreads / kWave];
+  __shared__ int best_i[kArgmaxThreads / kWave];
+  const int seg = blockIdx.x, r = blockIdx.y;
+  const float* row = logits + (size_t)r * ld;
+  // segment bounds in whole float4s when the row allows it
+  const int per = ((V + kArgmaxSegments - 1) / kArgmaxSegments + 3) & ~3;
+  const int begin = seg * per, end = min(V, begin + per);
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    const float v = row[i];
-    if (v > bv || (v == bv && i < bi)) {
-      bv = v;
-      bi = i;
+  const bool vec = ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
+  if (vec) {
+    for (int i = begin + threadIdx.x * 4; i < end; i += kArgmaxThreads * 4) {
+      if (i + 4 <= end) {
+        const float4 v = *reinterpret_cast<const float4*>(row + i);
+        argmax_take(bv, bi, v.x, i);
+        argmax_take(bv, bi, v.y, i + 1);
+        argmax_take(bv, bi, v.z, i + 2);
+        argmax_take(bv, bi, v.w, i + 3);
+      } else {
+        for (int j = i; j < end; ++j) argmax_take(bv, bi, row[j], j);
+      }
     }
+  } else {
+    for (int i = begin + threadIdx.x; i < end; i += kArgmaxThreads) argmax_take(bv, bi, row[i], i);
   }
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) {
     const float ov = __shfl_xor(bv, m, kWave);
     const int oi = __shfl_xor(bi, m, kWave);
-    if (ov > bv || (ov == bv && oi < bi)) {
-      bv = ov;
-      bi = oi;
-    }
+    argmax_take(bv, bi, ov, oi);
   }
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   if (lane == 0) {
@@ -46,20 +69,36 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int nw = (blockDim.x + kWave - 1) / kWave;
-    for (int w = 1; w < nw; ++w)
-      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
-        bv = best_v[w];
-        bi = best_i[w];
-      }
-    out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
+    for (int w = 1; w < kArgmaxThreads / kWave; ++w) argmax_take(bv, bi, best_v[w], best_i[w]);
+    part_v[r * kArgmaxSegments + seg] = bv;
+    part_i[r * kArgmaxSegments + seg] = bi;
   }
 }
 
-TK_API int tk_argmax(const float* logits, int* out, int M, int V, long ld, hipStream_t stream) {
+__global__ __launch_bounds__(kWave) void argmax_pick_kernel(const float* __restrict__ part_v,
+                                                            const int* __restrict__ part_i,
+                                                            int* __restrict__ out) {
+  const int r = blockIdx.x, lane = threadIdx.x;
+  float bv = lane < kArgmaxSegments ? part_v[r * kArgmaxSegments + lane] : -INFINITY;
+  int bi = lane < kArgmaxSegments ? part_i[r * kArgmaxSegments + lane] : 0x7fffffff;
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    const float ov = __shfl_xor(bv, m, kWave);
+    const int oi = __shfl_xor(bi, m, kWave);
+    argmax_take(bv, bi, ov, oi);
+  }
+  if (lane == 0) out[r] = (bi == 0x7fffffff) ? 0 : bi;
+}
+
+// part_v, part_i: scratch of M * tk_argmax_segments() floats and ints.
+TK_API int tk_argmax_segments() { return kArgmaxSegments; }
+
+TK_API int tk_argmax(const float* logits, int* out, float* part_v, int* part_i, int M, int V, long ld,
+                     hipStream_t stream) {
   if (M <= 0) return 0;
-  if (V <= 0) return -1;
-  argmax_kernel<<<M, 1024, 0, stream>>>(logits, out, V, ld);
+  if (V <= 0 || M > 65535) return -1;
+  argmax_segments_kernel<<<dim3(kArgmaxSegments, M), kArgmaxThreads, 0, stream>>>(logits, part_v, part_i, V, ld);
+  argmax_pick_kernel<<<M, kWave, 0, stream>>>(part_v, part_i, out);
   return launch_status();
 }
 
@@ -210,15 +249,14 @@ __global__ __launch_bounds__(1024) void sample_kernel(
   }
 }
 
-// Rows whose segment search falls through (rounding at a segment edge) keep the
-// value written by the argmax pre-pass that the host runs into `out` first.
+// `out` must already hold each row's argmax (tk_argmax): greedy rows keep it, and so
+// does a row whose segment search falls through (rounding at a segment edge).
 TK_API int tk_sample(const float* logits, long ld, int M, int V, const float* temperature,
                      const int* top_k, const float* top_p, const unsigned long long* seeds,
                      const unsigned long long* counters, int* out, float* probs_out,
                      hipStream_t stream) {
   if (M <= 0) return 0;
   if (V <= 0) return -1;
-  argmax_kernel<<<M, 1024, 0, stream>>>(logits, out, V, ld);
   sample_kernel<<<M, 1024, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, seeds, counters,
                                         out, probs_out);
   return launch_status();

@@ -113,7 +113,8 @@ _SIGS = {
                               c_int, c_int, c_int, c_int, c_float, c_void_p],
     },
     "sampling": {
-        "tk_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+        "tk_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+        "tk_argmax_segments": [],
         "tk_sample": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p],
     },
@@ -411,7 +412,12 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     _gpu(out)
     m, v = logits.shape
     _need(out.dtype == torch.int32 and out.numel() >= m, "argmax output is int32 [M]")
-    _check(_fn("sampling", "tk_argmax")(_p(logits), _p(out), m, v, logits.stride(0), _stream()), "argmax")
+    _need(m <= 65535, "at most 65535 rows")
+    segments = _fn("sampling", "tk_argmax_segments")()
+    part_v = torch.empty(m * segments, dtype=torch.float32, device=logits.device)
+    part_i = torch.empty(m * segments, dtype=torch.int32, device=logits.device)
+    _check(_fn("sampling", "tk_argmax")(_p(logits), _p(out), _p(part_v), _p(part_i), m, v, logits.stride(0),
+                                        _stream()), "argmax")
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
@@ -429,6 +435,7 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
         _need(t.numel() >= m, "one sampling parameter per row is required")
     _need(out.dtype == torch.int32, "sample output is int32")
     _need(probs_out is None or (probs_out.dtype == torch.float32 and probs_out.shape == (m, v)), "probs_out is float32 [M, V]")
+    argmax(logits, out)  # greedy rows are done with this; the others overwrite it
     _check(_fn("sampling", "tk_sample")(_p(logits), logits.stride(0), m, v, _p(temperature), _p(top_k),
                                         _p(top_p), _p(seeds), _p(counters), _p(out), _p(probs_out),
                                         _stream()), "sample")
