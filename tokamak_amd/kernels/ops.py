@@ -297,7 +297,7 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> N
 
 
 LT_WORKSPACE_BYTES = 128 << 20
-LT_TUNE_CANDIDATES = 16
+LT_TUNE_CANDIDATES = 16     # of the library's candidates, timed once per shape class
 _lt_workspace: dict[torch.device, torch.Tensor] = {}
 
 
