@@ -26,6 +26,7 @@ sys.path.insert(0, str(Path(__file__).resolve().parent))
 HBM_PEAK = 8.0e12
 MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 PREFILL_TOKENS = 2048
+SHAPE_NAMES = {"qwen3-0.6b": "Qwen3-0.6B", "qwen3-8b": "Qwen3-8B", "qwen3-32b": "Qwen3-32B"}
 
 
 def make_runner(cfg, dtype, pool_tokens, max_requests, seed=0):
@@ -190,11 +191,11 @@ def run_phase(args, runner, cfg, full) -> int:
         seconds, _ = time_decode(runner, cfg, args.batch, args.context, args.steps, args.warmup)
         value, steps, what = args.batch / seconds, args.steps, f"decode tok/s at batch {args.batch}"
     print(json.dumps({
-        "metric": f"{what} (Qwen3-8B-shaped, random weights)", "value": round(value, 1), "unit": "tokens/s",
+        "metric": f"{what} ({SHAPE_NAMES[args.shape]}-shaped, random weights)", "value": round(value, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": round(seconds * 1e3, 3),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": key,
         "data": "synthetic (uniform random token ids, seeded random weights)",
-        "config": {"model": "qwen3-8b-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers,
+        "config": {"model": f"{args.shape}-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers,
                    "global_batch": args.batch, "seq_len": args.context, "phase": args.phase,
                    "parallelism": "single GPU"},
     }))
@@ -216,6 +217,8 @@ def main() -> int:
     ap.add_argument("--workload", default="decode", choices=["decode", "continuous"],
                     help="decode: the headline measurement; continuous: LLM.generate over many requests")
     ap.add_argument("--model", default="qwen3-0.6b", help="preset shape of the continuous workload")
+    ap.add_argument("--shape", default="qwen3-8b", choices=["qwen3-0.6b", "qwen3-8b", "qwen3-32b"],
+                    help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
     ap.add_argument("--requests", type=int, default=256)
     ap.add_argument("--max-batch", type=int, default=64)
     args = ap.parse_args()
@@ -229,7 +232,7 @@ def main() -> int:
 
     from tokamak_amd.models.qwen3 import PRESETS
 
-    full = PRESETS["qwen3-8b"]
+    full = PRESETS[args.shape]
     cfg = dataclasses.replace(full, num_layers=args.layers or full.num_layers)
     elem = 2 if args.dtype == "bfloat16" else 4
     max_batch = 64 if not (args.no_points or args.phase != "all") else args.batch
@@ -250,7 +253,7 @@ def main() -> int:
     achieved = step_bytes / step_s
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
     result = {
-        "metric": "decode tok/s at batch 8 (Qwen3-8B-shaped, random weights); prefill tok/s at 2,048 tokens",
+        "metric": f"decode tok/s at batch {args.batch} ({SHAPE_NAMES[args.shape]}-shaped, random weights); prefill tok/s at 2,048 tokens",
         "value": round(args.batch / step_s, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -263,7 +266,7 @@ def main() -> int:
         "dtype": key,
         "data": "synthetic (uniform random token ids, seeded random weights N(0, 0.02), norm weights 1)",
         "config": {
-            "model": "qwen3-8b-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers,
+            "model": f"{args.shape}-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers,
             "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_kv_heads,
             "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size,
             "vocab_size": cfg.vocab_size, "global_batch": args.batch, "seq_len": args.context,
