@@ -84,13 +84,13 @@ def fill(runner, request, tokens, chunk=2048):
     return logits
 
 
-def time_prefill(runner, cfg, repeats=3):
+def time_prefill(runner, cfg, repeats=5):
     import torch
 
     from tokamak_amd.engine.runner import StepEntry
 
     times = []
-    for i in range(repeats + 1):
+    for i in range(repeats + 2):  # the first two are untimed (kernel choice of the library products, clocks)
         ids = random_prompt(cfg.vocab_size, PREFILL_TOKENS, 1000 + i)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -98,7 +98,7 @@ def time_prefill(runner, cfg, repeats=3):
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         runner.end("prefill")
-    return statistics.median(times[1:])
+    return statistics.median(times[2:])
 
 
 def time_decode(runner, cfg, batch, context, steps, warmup):
