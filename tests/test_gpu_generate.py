@@ -122,6 +122,40 @@ def test_preemption_is_invisible(folders):
     assert tight.runner.manager.num_free_pages() == 3
 
 
+@pytest.mark.parametrize("which", ["A", "D"])
+def test_random_workloads_do_not_depend_on_pool_budget_or_portions(tmp_path, which):
+    """Random prompts and sampling parameters: a run with a tight page pool (so requests
+    are preempted and recomputed), few running sequences, a small token budget and short
+    prompt portions produces the tokens and finish reasons of a roomy run (float32)."""
+    import random
+
+    from tiny import TINIES, make_folder
+    from tokamak_amd import LLM, SamplingParams
+
+    folder = make_folder(tmp_path, which)
+    cfg = TINIES[which]["config"]
+    page, longest = TINIES[which]["page_size"], min(cfg.max_position_embeddings, 256)
+    roomy = LLM(folder, dtype="float32", max_seq_len=longest, block_size=page, kv_pool_tokens=16 * longest,
+                max_batch_size=16)
+    preemptions = 0
+    for seed in range(5):
+        rng = random.Random(seed)
+        count = rng.randint(2, 8)
+        prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(1, longest // 2))] for _ in range(count)]
+        params = [SamplingParams(temperature=rng.choice([0.0, 0.0, 0.8, 1.2]), top_k=rng.choice([0, 5, 40]),
+                                 top_p=rng.choice([1.0, 0.9]), max_new_tokens=rng.randint(1, longest // 3),
+                                 seed=rng.randrange(1 << 30), ignore_eos=rng.random() < 0.7) for _ in range(count)]
+        want = roomy.generate(prompt_token_ids=prompts, sampling_params=params)
+        tight = LLM(folder, dtype="float32", max_seq_len=longest, block_size=page,
+                    kv_pool_tokens=longest + rng.randint(0, longest), max_batch_size=rng.randint(1, 6),
+                    max_num_batched_tokens=rng.choice([8, 16, 64, 2048]), prefill_chunk=rng.choice([None, 2, 7, 16, 100]))
+        got = tight.generate(prompt_token_ids=prompts, sampling_params=params)
+        tight.runner.manager.check()
+        preemptions += tight.num_preemptions
+        assert [(o.output_token_ids, o.finish_reason) for o in got] == [(o.output_token_ids, o.finish_reason) for o in want]
+    assert preemptions > 0
+
+
 def test_command_line(folders, capsys):
     from tokamak_amd import cli
 
