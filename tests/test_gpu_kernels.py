@@ -109,6 +109,25 @@ def test_long_context_over_shuffled_pages(dtype, hd):
         torch.testing.assert_close(g, w, **TOL[dtype])
 
 
+@pytest.mark.parametrize("nh, nkv, hd, ps", [(8, 2, 128, 16), (6, 3, 64, 32), (3, 1, 128, 16)])
+def test_short_portions_over_long_contexts_split_their_keys(nh, nkv, hd, ps):
+    """Few tiles over thousands of keys: the dispatcher cuts the keys of the tiles into
+    pieces (checked) that are merged afterwards; portions of other requests in the same
+    step are short, start at zero or end inside a piece, and a decode token rides along."""
+    from tokamak_amd.kernels.attention import tile_split
+
+    requests = [(5000, 37), (0, 20), (700, 3), (2047, 2), (1300, 1)]
+    tiles = sum(-(-q // 16) for _, q in requests if q > 1)
+    group = nh // nkv
+    per_tile = nkv * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
+    split, nsplit = tile_split(tiles, per_tile, 5037)
+    assert nsplit > 1 and split % 64 == 0 and (nsplit - 1) * split < 5037 <= nsplit * split
+    got, want = run_attention(torch.bfloat16, nh, nkv, hd, ps, requests, seed=11)
+    for g, w in zip(got, want):
+        assert torch.isfinite(g).all()
+        torch.testing.assert_close(g, w, **TOL[torch.bfloat16])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("far", [0, 3, 255, 256, 511, 777])
 def test_a_far_key_among_hundreds_is_found(dtype, far):

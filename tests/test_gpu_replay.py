@@ -18,7 +18,7 @@ LENGTHS = {"A": [5, 17, 33, 100, 128], "B": [1, 9, 40, 70, 201], "C": [2, 31, 64
 def setups(tmp_path_factory):
     root = tmp_path_factory.mktemp("replay")
     out = {}
-    for which in TINIES:
+    for which in LENGTHS:
         folder = make_folder(root, which)
         vocab = TINIES[which]["config"].vocab_size
         requests = {f"r{i}": random_ids(vocab, n, 100 + i) for i, n in enumerate(LENGTHS[which])}

@@ -46,7 +46,7 @@ TINY_E = dict(
 TINY_F = dict(
     config=Qwen3Config("Qwen3ForCausalLM", vocab_size=280, hidden_size=64, num_layers=2,
                        num_attention_heads=6, num_kv_heads=1, head_dim=128, intermediate_size=96,
-                       rms_norm_eps=1e-6, rope_theta=50000.0, max_position_embeddings=1024,
+                       rms_norm_eps=1e-6, rope_theta=50000.0, max_position_embeddings=2048,
                        tie_word_embeddings=False),
     seed=9, matrix_std=0.05, vector_jitter=0.1, page_size=16)
 

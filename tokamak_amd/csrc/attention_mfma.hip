@@ -216,14 +216,24 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 
 // Merge the splits of every (token, head): out = sum_s w_s o_s / sum_s w_s l_s,
 // w_s = exp2(m_s - max m).  Splits that hold no key of the token are skipped by
-// the token's position, so they need not have been written.
+// the token's position, so they need not have been written.  Rows: one per decode
+// item (item_count == nullptr), or sixteen per tile of a prompt portion, of which
+// the tile's first item_count[tile] are tokens.
 template <int HD>
 __global__ __launch_bounds__(64) void attention_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
-    const int* __restrict__ positions, const int* __restrict__ tokens, bf16_t* __restrict__ out,
-    int nsplit, int split_keys, int nh) {
-  const int n = tokens[blockIdx.x], head = blockIdx.y, lane = threadIdx.x;
-  const size_t row = (size_t)blockIdx.x * nh + head;  // partial row (by item)
+    const int* __restrict__ positions, const int* __restrict__ item_token,
+    const int* __restrict__ item_count, bf16_t* __restrict__ out, int nsplit, int split_keys, int nh) {
+  const int head = blockIdx.y, lane = threadIdx.x;
+  int n;
+  if (item_count == nullptr) {
+    n = item_token[blockIdx.x];
+  } else {
+    const int tile = blockIdx.x >> 4, t = blockIdx.x & 15;
+    if (t >= item_count[tile]) return;
+    n = item_token[tile] + t;
+  }
+  const size_t row = (size_t)blockIdx.x * nh + head;  // partial row
   const size_t orow = (size_t)n * nh + head;          // output row (by token)
   const int used = min(nsplit, positions[n] / split_keys + 1);
   const float* ml = part_ml + row * nsplit * 2;
@@ -278,7 +288,8 @@ void attention_prefill_kernel(
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ item_token, const int* __restrict__ item_count,
-    bf16_t* __restrict__ out, int num_items, int nh, int nkv, int ps, float scale_log2) {
+    bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int nsplit,
+    int split_keys, int num_items, int nh, int nkv, int ps, float scale_log2) {
   constexpr int KCH = HD / 32, DBL = HD / 16;
   constexpr int THREADS = kPrefillThreads;
   constexpr int GROUP_PIECES = 2 * HD;         // 16-byte pieces of K (and of V) per 16-key group
@@ -307,6 +318,12 @@ void attention_prefill_kernel(
   const size_t head_off = (size_t)kvh * HD * ps;
   const int c_pos = pos0 + col;
   const bool c_valid = col < count;
+  // With several splits (few tiles over a long context) this block takes the keys
+  // [k_begin, k_begin + split_keys), a multiple of 64, and writes an unnormalised partial.
+  const int split = blockIdx.z;
+  const int k_begin = split * split_keys;
+  if (k_begin > last_pos) return;  // no key of this tile lies in the split (the whole block leaves)
+  const int last_key = min(last_pos, k_begin + split_keys - 1);
 
   bf16x8 qreg[KCH];
   {
@@ -355,7 +372,7 @@ void attention_prefill_kernel(
   // (scalar loads), so their latency is never waited for.
   int page_next[PPT];  // of the 16-key group of this wave's piece i
 #define TK_PAGES(S0)                                                             \
-  if ((S0) <= last_pos) {                                                        \
+  if ((S0) <= last_key) {                                                        \
     _Pragma("unroll") for (int i = 0; i < PPT; ++i) {                            \
       const int c0 = ((S0) + grp[i] * 16 <= last_pos) ? (S0) + grp[i] * 16 : (S0); \
       page_next[i] = table[c0 >> ps_shift];                                      \
@@ -375,15 +392,15 @@ void attention_prefill_kernel(
     TK_PAGES((S0) + 64)                                                                          \
   }
 
-  TK_PAGES(0)
+  TK_PAGES(k_begin)
 #pragma unroll
   for (int b = 0; b < NBUF; ++b)
-    if (b == 0 || b * 64 <= last_pos) TK_FETCH(b * 64, b)
-  for (int sp = 0; sp <= last_pos; sp += 64 * NBUF) {
+    if (b == 0 || k_begin + b * 64 <= last_key) TK_FETCH(k_begin + b * 64, b)
+  for (int sp = k_begin; sp <= last_key; sp += 64 * NBUF) {
 #pragma unroll
    for (int buf = 0; buf < NBUF; ++buf) {
     const int s0 = sp + buf * 64;
-    if (s0 > last_pos) break;
+    if (s0 > last_key) break;
     __syncthreads();  // every wave has read the previous stage
     if (s0 + 63 > last_pos) {
       // keys past the request's end may hold anything (their probability is zero, but
@@ -403,7 +420,7 @@ void attention_prefill_kernel(
       *reinterpret_cast<uint2*>(vs + v_lds[i][1]) = make_uint2(vpre[buf][i][2], vpre[buf][i][3]);
     }
     __syncthreads();
-    if (s0 + 64 * NBUF <= last_pos) TK_FETCH(s0 + 64 * NBUF, buf)
+    if (s0 + 64 * NBUF <= last_key) TK_FETCH(s0 + 64 * NBUF, buf)
     if (!computes) continue;
 
     // S^T for 4 groups of 16 keys
@@ -481,14 +498,27 @@ void attention_prefill_kernel(
   l += __shfl_xor(l, 16, kWave);
   l += __shfl_xor(l, 32, kWave);
   if (c_valid && computes) {
-    const float inv = 1.f / l;
-    bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * HD + kb * 4;
+    if (nsplit == 1) {
+      const float inv = 1.f / l;
+      bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * HD + kb * 4;
 #pragma unroll
-    for (int d = 0; d < DBL; ++d) {
-      uint2 o;
-      o.x = pack_bf16x2(acc[d][0] * inv, acc[d][1] * inv);
-      o.y = pack_bf16x2(acc[d][2] * inv, acc[d][3] * inv);
-      *reinterpret_cast<uint2*>(op + d * 16) = o;
+      for (int d = 0; d < DBL; ++d) {
+        uint2 o;
+        o.x = pack_bf16x2(acc[d][0] * inv, acc[d][1] * inv);
+        o.y = pack_bf16x2(acc[d][2] * inv, acc[d][3] * inv);
+        *reinterpret_cast<uint2*>(op + d * 16) = o;
+      }
+    } else {
+      // partial rows: sixteen per tile, by the token's place in the tile
+      const size_t prow = ((size_t)(item * 16 + col) * nh + head) * nsplit + split;
+      float* po = part_o + prow * HD + kb * 4;
+#pragma unroll
+      for (int d = 0; d < DBL; ++d)
+        *reinterpret_cast<float4*>(po + d * 16) = make_float4(acc[d][0], acc[d][1], acc[d][2], acc[d][3]);
+      if (kb == 0) {
+        part_ml[prow * 2] = m_run;
+        part_ml[prow * 2 + 1] = l;
+      }
     }
   }
 }
@@ -500,14 +530,19 @@ template <int HD, int HPB>
 static int launch_prefill(const void* q, const void* k_cache, const void* v_cache,
                           const int* block_tables, int max_pages, const int* positions,
                           const int* req_of_token, const int* item_token, const int* item_count,
-                          int num_items, void* out, int nh, int nkv, int ps, float scale,
-                          hipStream_t stream) {
+                          int num_items, void* out, float* part_o, float* part_ml, int nsplit,
+                          int split_keys, int nh, int nkv, int ps, float scale, hipStream_t stream) {
   const int G = nh / nkv;
-  dim3 grid(nkv * (G / HPB), num_items);
+  dim3 grid(nkv * (G / HPB), num_items, nsplit);
   attention_prefill_kernel<HD, HPB><<<grid, kPrefillThreads, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
-      positions, req_of_token, item_token, item_count, (bf16_t*)out, num_items, nh, nkv, ps,
-      scale * 1.4426950408889634f);
+      positions, req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit,
+      split_keys, num_items, nh, nkv, ps, scale * 1.4426950408889634f);
+  if (nsplit > 1) {
+    dim3 mgrid(num_items * 16, nh);
+    attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token, item_count,
+                                                         (bf16_t*)out, nsplit, split_keys, nh);
+  }
   return launch_status();
 }
 
@@ -525,14 +560,15 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
       split_keys, nh, nkv, ps, scale * 1.4426950408889634f);
   if (nsplit > 1) {
     dim3 mgrid(num_items, nh);
-    attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token,
+    attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token, nullptr,
                                                          (bf16_t*)out, nsplit, split_keys, nh);
   }
   return launch_status();
 }
 
 // mode 0: heads (every item is one decode token; item_count is ignored)
-// mode 1: tokens (item = up to 16 consecutive tokens of one request; nsplit must be 1)
+// mode 1: tokens (item = up to 16 consecutive tokens of one request; with nsplit > 1 split_keys
+//         is a multiple of 64 and the partial buffers hold 16 rows per item)
 // Returns -2 if this shape is not instantiated (the caller uses the generic kernel).
 TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const void* v_cache,
                              const int* block_tables, int max_pages, const int* positions,
@@ -553,11 +589,12 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
     if (hd == 64) return launch<64, 1>(TK_ARGS);
     return -2;
   }
-  if (nsplit != 1) return -1;
+  // the keys of a tile may be split too: in whole stages of 64 keys, sixteen partial rows a tile
+  if (nsplit > 1 && (split_keys % 64 != 0 || (long)num_items * 16 > 65535)) return -1;
   const int hpb = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
 #define TK_PARGS                                                                                  \
   q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
-      num_items, out, nh, nkv, ps, scale, stream
+      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream
   if (hd == 128) {
     if (hpb == 4) return launch_prefill<128, 4>(TK_PARGS);
     if (hpb == 2) return launch_prefill<128, 2>(TK_PARGS);

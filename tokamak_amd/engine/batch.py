@@ -49,6 +49,7 @@ class StepBatch:
     num_decode: int = 0
     num_tiles: int = 0
     max_decode_len: int = 0                     # longest context among the decode tokens
+    max_tile_len: int = 0                       # longest context (with the portion) among the tiled spans
     # host copies, for choosing kernels and grids
     q_lens: list[int] = field(default_factory=list)
     ctx_lens: list[int] = field(default_factory=list)
@@ -77,6 +78,7 @@ class PackedBatch:
     q_lens: list[int]
     ctx_lens: list[int]
     max_decode_len: int
+    max_tile_len: int = 0
 
 
 def table_width(longest: int, fixed: int | None = None) -> int:
@@ -141,7 +143,8 @@ def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] |
         buf=buf, offsets=offsets, widths=widths, num_tokens=n, num_requests=r, num_logit_rows=m,
         num_decode=nd, num_tiles=nt, q_lens=[len(s.tokens) for s in spans],
         ctx_lens=[s.ctx_len for s in spans],
-        max_decode_len=max((s.ctx_len + 1 for s in spans if len(s.tokens) == 1), default=0))
+        max_decode_len=max((s.ctx_len + 1 for s in spans if len(s.tokens) == 1), default=0),
+        max_tile_len=max((s.ctx_len + len(s.tokens) for s in spans if len(s.tokens) > 1), default=0))
 
 
 def batch_from_device(packed: PackedBatch, dev: torch.Tensor) -> StepBatch:
@@ -155,7 +158,8 @@ def batch_from_device(packed: PackedBatch, dev: torch.Tensor) -> StepBatch:
         block_tables=[parts[NUM_FIXED + g].view(r, widths[g]) for g in range(len(widths))],
         decode_tokens=parts[7], tile_first=parts[8], tile_count=parts[9],
         num_decode=packed.num_decode, num_tiles=packed.num_tiles,
-        max_decode_len=packed.max_decode_len, q_lens=packed.q_lens, ctx_lens=packed.ctx_lens,
+        max_decode_len=packed.max_decode_len, max_tile_len=packed.max_tile_len,
+        q_lens=packed.q_lens, ctx_lens=packed.ctx_lens,
         max_q_len=max(packed.q_lens, default=0),
         max_seq_len=max((c + q for c, q in zip(packed.ctx_lens, packed.q_lens)), default=0),
     )

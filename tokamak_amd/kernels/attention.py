@@ -9,6 +9,9 @@ from tokamak_amd.kernels import ops
 MFMA_HEAD_DIMS = (64, 128)
 SPLIT_KEYS = 256          # fewest keys a split of a decode token's context holds
 TARGET_DECODE_WAVES = 4096  # waves wanted in flight; beyond that splits only cost a merge
+TILE_SPLIT_BELOW_BLOCKS = 256   # a portion with fewer blocks than this has its keys split ...
+TILE_SPLIT_MIN_KEYS = 512       # ... into pieces no shorter than this
+TARGET_TILE_BLOCKS = 1024
 
 
 def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
@@ -27,6 +30,22 @@ def decode_split(num_decode: int, num_kv_heads: int, max_len: int) -> tuple[int,
     return split, max(1, -(-max_len // split))
 
 
+def tile_split(num_tiles: int, blocks_per_tile: int, max_len: int) -> tuple[int, int]:
+    """(keys per split, number of splits) for the 16-token tiles of prompt portions.
+    A block walks its tile's keys 64 at a time, one after the other; a short portion
+    over a long context (the last piece of a long prompt, a small token budget) has
+    few tiles and would leave the GPU idle for hundreds of such steps, so its keys
+    are cut into pieces that run side by side and are merged afterwards."""
+    blocks = num_tiles * blocks_per_tile
+    if blocks >= TILE_SPLIT_BELOW_BLOCKS or max_len < 2 * TILE_SPLIT_MIN_KEYS or num_tiles * 16 > 65535:
+        return 1 << 30, 1
+    nsplit = min(max_len // TILE_SPLIT_MIN_KEYS, -(-TARGET_TILE_BLOCKS // blocks))
+    if nsplit < 2:
+        return 1 << 30, 1
+    split = -(-(-(-max_len // nsplit)) // 64) * 64
+    return split, -(-max_len // split)
+
+
 def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads, num_kv_heads,
                     head_dim, page_size, scale, window=None) -> None:
     """out[n] = softmax(q[n] . K[0..pos_n] * scale) V, per head, over the pages
@@ -34,7 +53,8 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
 
     bfloat16 with head size 64 or 128: the MFMA kernel, once over the single
     (decode) tokens with their context split, once over 16-token tiles of the
-    prompt portions.  Everything else: the generic float32-arithmetic kernel.
+    prompt portions (their keys split too when the tiles are few and the context
+    long).  Everything else: the generic float32-arithmetic kernel.
     """
     if mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, window):
         common = dict(num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
@@ -45,9 +65,12 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
                                batch.req_of_token, batch.decode_tokens, None, batch.num_decode, out,
                                split_keys=split, num_splits=nsplit, **common)
         if batch.num_tiles:
+            group = num_heads // num_kv_heads
+            per_tile = num_kv_heads * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
+            split, nsplit = tile_split(batch.num_tiles, per_tile, batch.max_tile_len)
             ops.attention_mfma("tokens", q, k_cache, v_cache, block_tables, batch.positions,
                                batch.req_of_token, batch.tile_first, batch.tile_count, batch.num_tiles,
-                               out, split_keys=1 << 30, num_splits=1, **common)
+                               out, split_keys=split, num_splits=nsplit, **common)
         return
     ops.paged_attention_generic(
         q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,

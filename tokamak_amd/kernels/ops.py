@@ -374,7 +374,10 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
                    page_size: int, scale: float, split_keys: int = 256, num_splits: int = 1) -> bool:
     """bf16 attention on the matrix cores.  ``mode`` "heads": every item is one
     decode token; "tokens": every item is up to 16 consecutive tokens of one
-    request.  Returns False (nothing launched) if the shape is not instantiated."""
+    request.  With ``num_splits`` > 1 the keys of an item are cut into pieces of
+    ``split_keys`` (a multiple of 16; of 64 in "tokens" mode), each its own block, and a
+    second kernel merges the pieces.  Returns False (nothing launched) if the shape
+    is not instantiated."""
     _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, item_token, item_count, out)
     n = positions.numel()
     _need(q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
@@ -388,12 +391,15 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
           and item_token.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
     _need(item_token.numel() >= num_items and 0 < num_items <= 65535, "bad item list")
     if mode == "tokens":
-        _need(item_count is not None and item_count.dtype == torch.int32 and item_count.numel() >= num_items
-              and num_splits == 1, "tokens mode needs item counts and one split")
+        _need(item_count is not None and item_count.dtype == torch.int32 and item_count.numel() >= num_items,
+              "tokens mode needs item counts")
+        _need(num_splits == 1 or (split_keys % 64 == 0 and num_items * 16 <= 65535),
+              "tokens mode splits keys in multiples of 64, for at most 4095 tiles")
     part_o = part_ml = None
     if num_splits > 1:
-        part_o = torch.empty((num_items * num_heads * num_splits, head_dim), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((num_items * num_heads * num_splits, 2), dtype=torch.float32, device=q.device)
+        rows = num_items * (16 if mode == "tokens" else 1) * num_heads * num_splits
+        part_o = torch.empty((rows, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((rows, 2), dtype=torch.float32, device=q.device)
     status = _fn("attention_mfma", "tk_attention_mfma")(
         0 if mode == "heads" else 1, _p(q), _p(k_cache), _p(v_cache), _p(block_tables),
         block_tables.shape[1], _p(positions), _p(req_of_token), _p(item_token), _p(item_count),
