@@ -6,9 +6,9 @@
 // keeps every logit >= the k-th largest (ties at the threshold survive); top-p
 // sorts descending and drops a token iff the mass ranked before it already
 // reaches top_p (the best token always survives); softmax over what is left;
-// one draw.  No sort is done here: both thresholds are found by bisection over
-// the ordered-integer image of the float values, each probe one pass over the
-// row (which sits in L2).
+// one draw.  No sort is done here: both thresholds are found by radix selection
+// over the ordered-integer image of the float values, three passes over the row
+// each (the row sits in L2).
 #include "common.h"
 
 using namespace tk;
@@ -125,31 +125,99 @@ __device__ __forceinline__ float uniform01(uint64_t seed, uint64_t counter) {
   return (float)(z >> 40) * (1.0f / 16777216.0f);
 }
 
-__device__ __forceinline__ int block_sum_int(int v, int* scratch) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int nw = (blockDim.x + kWave - 1) / kWave;
+constexpr int kSampleThreads = 1024;
+constexpr int kBins = 4096;  // histogram bins of one radix pass (12 bits)
+
+// Prefix sums of one value per thread over the block, threads in index order; `scan`
+// holds kSampleThreads entries.  Returns the sum over the threads before this one;
+// `inclusive` is that plus the thread's own value as the scan computed it (so the
+// ranges [exclusive, inclusive) of the threads tile [0, total) exactly, also in
+// floating point); `total` is the sum over all threads.
+template <typename T>
+__device__ __forceinline__ T block_scan(T v, T* scan, T& inclusive, T& total) {
+  const int tid = threadIdx.x;
   __syncthreads();
-  if (lane == 0) scratch[wave] = v;
+  scan[tid] = v;
   __syncthreads();
-  int t = 0;
-  for (int i = 0; i < nw; ++i) t += scratch[i];
-  return t;
+  for (int step = 1; step < kSampleThreads; step <<= 1) {
+    const T add = tid >= step ? scan[tid - step] : T(0);
+    __syncthreads();
+    scan[tid] += add;
+    __syncthreads();
+  }
+  total = scan[kSampleThreads - 1];
+  inclusive = scan[tid];
+  return tid > 0 ? scan[tid - 1] : T(0);
+}
+
+// Walking the bins from the highest down: the bin in which the running sum first
+// reaches `target` (sum of higher bins < target <= that sum + the bin), and the sum
+// of the higher bins.  Every thread gets the result.  `nbins` is 4096 or 256.
+template <typename T>
+__device__ __forceinline__ void crossing_bin(const T* hist, int nbins, T target, T* scan, int* found_bin,
+                                             T* found_above, int& bin, T& above) {
+  const int tid = threadIdx.x;
+  const int per = nbins / kSampleThreads > 0 ? nbins / kSampleThreads : 1;
+  // thread t owns bins [top - per*t, top - per*t - per + 1], highest first
+  T mine = 0;
+  const int first = nbins - 1 - tid * per;
+  if (first >= 0)
+    for (int j = 0; j < per; ++j) mine += hist[first - j];
+  T total, upto;
+  const T before = block_scan<T>(mine, scan, upto, total);
+  if (tid == 0) {  // target beyond everything (rounding): the lowest bin
+    *found_bin = 0;
+    *found_above = total - hist[0];
+  }
+  __syncthreads();
+  if (first >= 0 && before < target && target <= upto) {
+    T run = before;
+    for (int j = 0; j < per; ++j) {
+      const T h = hist[first - j];
+      if (run + h >= target) {
+        *found_bin = first - j;
+        *found_above = run;
+        break;
+      }
+      run += h;
+    }
+  }
+  __syncthreads();
+  bin = *found_bin;
+  above = *found_above;
+  __syncthreads();
+}
+
+// exp(x - max) as a 32.32 fixed-point number: integer sums do not depend on the
+// order of addition, so thresholds found from them are the same on every run
+__device__ __forceinline__ unsigned long long fixed_mass(float x, float mx) {
+  return (unsigned long long)(expf(x - mx) * 4294967296.f);
 }
 
 // One block per row.  params rows: temperature, top_k, top_p (floats);
 // seeds/counters: the request's seed and how many draws it has made.
 // probs_out (optional, [M, V]) receives the final distribution, for tests.
-__global__ __launch_bounds__(1024) void sample_kernel(
+//
+// Both thresholds are found by radix selection over the ordered-integer image of the
+// scaled logits: three passes over the row (12, 12 and 8 bits), each filling a
+// histogram in LDS (counts for top-k, fixed-point probability mass for top-p) in
+// which the bin that holds the threshold is found; the next pass looks only at the
+// values of that bin.  The row (600 KB for a vocabulary of 152 k) stays in L2.
+__global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p,
     const unsigned long long* __restrict__ seeds, const unsigned long long* __restrict__ counters,
     int* __restrict__ out, float* __restrict__ probs_out) {
   __shared__ float fs[16];
-  __shared__ int is[16];
-  __shared__ float seg_prefix[1025];
-  const int r = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
+  __shared__ unsigned long long hist64[kBins];       // counts use the same memory as 32-bit bins
+  __shared__ unsigned long long scan64[kSampleThreads];
+  __shared__ int found_bin;
+  __shared__ unsigned long long found_above;
+  uint32_t* hist32 = reinterpret_cast<uint32_t*>(hist64);
+  uint32_t* scan32 = reinterpret_cast<uint32_t*>(scan64);
+  float* scanf_ = reinterpret_cast<float*>(scan64);
+
+  const int r = blockIdx.x, tid = threadIdx.x, nt = kSampleThreads;
   if (!(temperature[r] > 0.f)) return;  // greedy row: the argmax pre-pass has written it
   const float* row = logits + (size_t)r * ld;
   const float inv_t = 1.f / temperature[r];
@@ -157,71 +225,100 @@ __global__ __launch_bounds__(1024) void sample_kernel(
   const float p_keep = top_p[r];
 
   float mx = -INFINITY;
+#pragma unroll 8
   for (int i = tid; i < V; i += nt) mx = fmaxf(mx, row[i] * inv_t);
   mx = block_max(mx, fs);
 
-  // top-k: the k-th largest scaled logit, by bisection on the ordered image:
-  // the largest t with count(x >= t) >= k.
+  // top-k: kth = the k-th largest scaled logit (everything >= it survives)
   uint32_t kth = 0;  // ordered(-inf) is > 0, so 0 keeps everything
   if (k > 0 && k < V) {
-    uint32_t lo = 0, hi = 0xffffffffu;  // invariant: count(>= lo) >= k
-    while (lo < hi) {
-      const uint32_t mid = lo + (uint32_t)(((uint64_t)hi - lo + 1) >> 1);
-      int c = 0;
-      for (int i = tid; i < V; i += nt) c += ordered(row[i] * inv_t) >= mid;
-      c = block_sum_int(c, is);
-      if (c >= k) lo = mid; else hi = mid - 1;
+    uint32_t prefix = 0, remaining = (uint32_t)k;
+    // (shift, bits): 20/12, 8/12, 0/8
+    for (int level = 0; level < 3; ++level) {
+      const int shift = level == 0 ? 20 : level == 1 ? 8 : 0;
+      const int nbins = level == 2 ? 256 : kBins;
+      for (int i = tid; i < kBins; i += nt) hist32[i] = 0;
+      __syncthreads();
+#pragma unroll 8
+      for (int i = tid; i < V; i += nt) {
+        const uint32_t o = ordered(row[i] * inv_t);
+        const bool in_bin = level == 0 || (o >> (shift + (level == 1 ? 12 : 8))) == prefix;
+        if (in_bin) atomicAdd(&hist32[(o >> shift) & (uint32_t)(nbins - 1)], 1u);
+      }
+      __syncthreads();
+      int bin;
+      uint32_t above;
+      crossing_bin<uint32_t>(hist32, nbins, remaining, scan32, &found_bin,
+                             reinterpret_cast<uint32_t*>(&found_above), bin, above);
+      remaining -= above;
+      prefix = (prefix << (level == 2 ? 8 : 12)) | (uint32_t)bin;
     }
-    kth = lo;
+    kth = prefix;
   }
 
-  // softmax normaliser over what top-k kept
-  float z = 0.f;
-  for (int i = tid; i < V; i += nt) {
-    const float x = row[i] * inv_t;
-    if (ordered(x) >= kth) z += expf(x - mx);
-  }
-  z = block_sum(z, fs);
-
-  // top-p: keep x iff mass of kept values strictly greater than x is < top_p.
-  // The kept set is {x >= cut}; cut = smallest t with mass(> t) < top_p.
+  // top-p: keep x iff the mass of kept values strictly greater than x is < top_p of
+  // the whole; the kept set is {x >= cut}
   uint32_t cut = kth;
   if (p_keep < 1.f) {
-    uint32_t lo = kth, hi = ordered(mx);  // mass(> hi) = 0 < top_p always
-    while (lo < hi) {
-      const uint32_t mid = lo + ((hi - lo) >> 1);
-      float mass = 0.f;
+    uint32_t prefix = 0;
+    unsigned long long remaining = 0;
+    for (int level = 0; level < 3; ++level) {
+      const int shift = level == 0 ? 20 : level == 1 ? 8 : 0;
+      const int nbins = level == 2 ? 256 : kBins;
+      for (int i = tid; i < kBins; i += nt) hist64[i] = 0;
+      __syncthreads();
+#pragma unroll 8
       for (int i = tid; i < V; i += nt) {
         const float x = row[i] * inv_t;
         const uint32_t o = ordered(x);
-        if (o >= kth && o > mid) mass += expf(x - mx);
+        const bool in_bin = level == 0 || (o >> (shift + (level == 1 ? 12 : 8))) == prefix;
+        if (in_bin && o >= kth) atomicAdd(&hist64[(o >> shift) & (uint32_t)(nbins - 1)], fixed_mass(x, mx));
       }
-      mass = block_sum(mass, fs) / z;
-      if (mass < p_keep) hi = mid; else lo = mid + 1;
+      __syncthreads();
+      if (level == 0) {
+        // the whole mass, then the share of it that top_p allows (at least one unit)
+        unsigned long long mine = 0, upto, whole;
+        for (int i = tid; i < kBins; i += nt) mine += hist64[i];
+        block_scan<unsigned long long>(mine, scan64, upto, whole);
+        const double share = (double)p_keep * (double)whole;
+        remaining = share < 1.0 ? 1ull : (unsigned long long)share;
+      }
+      int bin;
+      unsigned long long above;
+      crossing_bin<unsigned long long>(hist64, nbins, remaining, scan64, &found_bin, &found_above, bin, above);
+      remaining -= above;
+      prefix = (prefix << (level == 2 ? 8 : 12)) | (uint32_t)bin;
     }
-    cut = lo;
+    cut = prefix > kth ? prefix : kth;
   }
 
-  // final distribution over {x >= cut}; contiguous segment per thread so the
-  // draw walks tokens in index order
-  const int seg = (V + nt - 1) / nt;
-  const int b = tid * seg, e = (b + seg < V) ? b + seg : V;
+  // final distribution over {x >= cut}.  The draw walks the tokens in index order: each
+  // wave owns a contiguous chunk of the row (read 64 tokens at a time, coalesced); the
+  // wave whose chunk holds the target walks it again with a prefix sum over the lanes.
+  const int lane = tid & (kWave - 1), wave = tid / kWave;
+  constexpr int kWaves = kSampleThreads / kWave;
+  const int chunk = ((V + kWaves - 1) / kWaves + kWave - 1) / kWave * kWave;
+  const int c_begin = wave * chunk, c_end = min(V, c_begin + chunk);
   float mine = 0.f;
-  for (int i = b; i < e; ++i) {
+#pragma unroll 8
+  for (int i = c_begin + lane; i < c_end; i += kWave) {
     const float x = row[i] * inv_t;
     if (ordered(x) >= cut) mine += expf(x - mx);
   }
+  mine = wave_sum(mine);
   __syncthreads();
-  seg_prefix[tid + 1] = mine;
-  if (tid == 0) seg_prefix[0] = 0.f;
+  if (lane == 0) fs[wave] = mine;
   __syncthreads();
-  if (tid == 0)
-    for (int i = 1; i <= nt; ++i) seg_prefix[i] += seg_prefix[i - 1];
-  __syncthreads();
-  const float total = seg_prefix[nt];
+  float before = 0.f, total = 0.f;
+  for (int w = 0; w < kWaves; ++w) {
+    if (w == wave) before = total;
+    total += fs[w];
+  }
+  const float upto = before + fs[wave];
 
   if (probs_out) {
     float* po = probs_out + (size_t)r * V;
+#pragma unroll 8
     for (int i = tid; i < V; i += nt) {
       const float x = row[i] * inv_t;
       po[i] = (ordered(x) >= cut) ? expf(x - mx) / total : 0.f;
@@ -229,23 +326,55 @@ __global__ __launch_bounds__(1024) void sample_kernel(
   }
 
   const float target = uniform01(seeds[r], counters[r]) * total;
-  // the segment that holds the target; the last non-empty segment catches rounding
-  if (seg_prefix[tid] <= target && (target < seg_prefix[tid + 1] || tid == nt - 1) && b < V) {
-    float run = seg_prefix[tid];
-    int pick = -1, last_kept = -1;
-    for (int i = b; i < e; ++i) {
+  // the chunk that holds the target; the last non-empty chunk catches rounding
+  const bool last_chunk = c_begin < V && c_begin + chunk >= V;
+  if (before <= target && (target < upto || last_chunk) && c_begin < V) {
+    // this wave's chunk holds the target: every lane sums a contiguous run of it, a
+    // prefix sum over the lanes finds the run, and that lane walks its run
+    const int run_len = (c_end - c_begin + kWave - 1) / kWave;
+    const int r_begin = min(c_end, c_begin + lane * run_len), r_end = min(c_end, r_begin + run_len);
+    float mine_run = 0.f;
+    int last_kept = -1;
+    for (int i = r_begin; i < r_end; ++i) {
       const float x = row[i] * inv_t;
       if (ordered(x) >= cut) {
+        mine_run += expf(x - mx);
         last_kept = i;
-        run += expf(x - mx);
-        if (run > target) {
-          pick = i;
-          break;
-        }
       }
     }
-    if (pick < 0) pick = last_kept;
-    if (pick >= 0) out[r] = pick;
+    float incl = mine_run;  // inclusive prefix over the lanes
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const float up = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl += up;
+    }
+    float excl = __shfl_up(incl, 1, kWave);
+    if (lane == 0) excl = 0.f;
+    int pick = -1;
+    if (before + excl <= target && target < before + incl) {
+      float run = before + excl;
+      for (int i = r_begin; i < r_end; ++i) {
+        const float x = row[i] * inv_t;
+        if (ordered(x) >= cut) {
+          run += expf(x - mx);
+          if (run > target) {
+            pick = i;
+            break;
+          }
+        }
+      }
+      if (pick < 0) pick = last_kept;  // rounding at the end of the run
+    }
+    // one lane at most has picked; otherwise (rounding at a chunk's edge) the last kept token
+    int chosen = pick;
+    int fallback = last_kept;
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+      chosen = max(chosen, __shfl_xor(chosen, m, kWave));
+      fallback = max(fallback, __shfl_xor(fallback, m, kWave));
+    }
+    if (chosen < 0) chosen = fallback;
+    if (chosen >= 0 && lane == 0) out[r] = chosen;
   }
 }
 
@@ -257,7 +386,7 @@ TK_API int tk_sample(const float* logits, long ld, int M, int V, const float* te
                      hipStream_t stream) {
   if (M <= 0) return 0;
   if (V <= 0) return -1;
-  sample_kernel<<<M, 1024, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, seeds, counters,
+  sample_kernel<<<M, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, seeds, counters,
                                         out, probs_out);
   return launch_status();
 }

@@ -11,6 +11,7 @@ here, not the same stream.
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from tokamak_amd.kernels import ops
@@ -38,11 +39,19 @@ def sample_tokens(logits: torch.Tensor, params: list[SamplingParams], seeds: lis
     if all(p.is_greedy for p in params) and not return_probs:
         return greedy_tokens(logits)
     dev = logits.device
-    temperature = torch.tensor([p.temperature for p in params], dtype=torch.float32).to(dev)
-    top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32).to(dev)
-    top_p = torch.tensor([p.top_p for p in params], dtype=torch.float32).to(dev)
-    seed_t = torch.tensor([s & 0x7FFFFFFFFFFFFFFF for s in seeds], dtype=torch.int64).to(dev)
-    draw_t = torch.tensor(draws, dtype=torch.int64).to(dev)
+    # one host buffer, one copy: [seeds | draws] int64, then [temperature | top_p] float32 and top_k int32
+    host = np.empty(7 * m, dtype=np.int32)
+    wide = host[:4 * m].view(np.int64)
+    wide[:m] = [s & 0x7FFFFFFFFFFFFFFF for s in seeds]
+    wide[m:] = draws
+    floats = host[4 * m:6 * m].view(np.float32)
+    floats[:m] = [p.temperature for p in params]
+    floats[m:] = [p.top_p for p in params]
+    host[6 * m:] = [p.top_k for p in params]
+    packed = torch.from_numpy(host).to(dev)
+    seed_t, draw_t = packed[:2 * m].view(torch.int64), packed[2 * m:4 * m].view(torch.int64)
+    temperature, top_p = packed[4 * m:5 * m].view(torch.float32), packed[5 * m:6 * m].view(torch.float32)
+    top_k = packed[6 * m:]
     out = torch.empty((m,), dtype=torch.int32, device=dev)
     probs = torch.zeros_like(logits) if return_probs else None
     ops.sample(logits, temperature, top_k, top_p, seed_t, draw_t, out, probs)
