@@ -156,6 +156,24 @@ def test_random_workloads_do_not_depend_on_pool_budget_or_portions(tmp_path, whi
     assert preemptions > 0
 
 
+def test_typed_configuration_gives_the_weights_of_a_written_folder(tmp_path):
+    """``LLM(config, seed=...)`` (random weights without a folder) generates what a
+    folder written by ``write_random_model`` with the same seed generates."""
+    from tiny import TINIES
+    from tokamak_amd import LLM, SamplingParams
+    from tokamak_amd.weights import write_random_model
+
+    cfg = TINIES["B"]["config"]
+    folder = write_random_model(tmp_path / "m", cfg, 5)
+    prompts = [[3, 1, 4, 1, 5, 9, 2, 6], [7]]
+    params = SamplingParams(temperature=0.0, max_new_tokens=10, ignore_eos=True)
+    a = LLM(folder, dtype="float32", block_size=8).generate(prompt_token_ids=prompts, sampling_params=params)
+    b = LLM(cfg, seed=5, dtype="float32", block_size=8).generate(prompt_token_ids=prompts, sampling_params=params)
+    assert [o.output_token_ids for o in a] == [o.output_token_ids for o in b]
+    c = LLM(cfg, seed=6, dtype="float32", block_size=8).generate(prompt_token_ids=prompts, sampling_params=params)
+    assert [o.output_token_ids for o in a] != [o.output_token_ids for o in c]
+
+
 def test_command_line(folders, capsys):
     from tokamak_amd import cli
 

@@ -14,14 +14,15 @@ from pathlib import Path
 
 import torch
 
-from tokamak_amd.config.registry import load_model_description
+from tokamak_amd.config.registry import get_architecture, load_model_description
 from tokamak_amd.engine.outputs import RequestOutput
 from tokamak_amd.engine.runner import ModelRunner, StepEntry, resolve_dtype
 from tokamak_amd.engine.scheduler import ScheduledStep, Scheduler
 from tokamak_amd.engine.sequence import Sequence
 from tokamak_amd.sampling.params import SamplingParams
 from tokamak_amd.sampling.sampler import sample_tokens
-from tokamak_amd.weights.sources import SafetensorsSource
+from tokamak_amd.weights.random_init import expected_tensors_of
+from tokamak_amd.weights.sources import RandomSource, SafetensorsSource
 
 
 class LLM:
@@ -29,7 +30,9 @@ class LLM:
 
     Args (names and meanings as the reference's where it has them,
     src/tokamak/engine/llm.py:64-104):
-        model: folder with ``config.json`` and ``*.safetensors``.
+        model: folder with ``config.json`` and ``*.safetensors``; or an architecture's
+            typed configuration (e.g. ``Qwen3Config``) for seeded random weights
+            (``seed``; the same weights ``write_random_model`` would put in a folder).
         dtype: ``"bfloat16"`` (default) or ``"float32"`` (everything in true 32-bit).
         max_seq_len: cap on one request's context; default the model's maximum.
         block_size: tokens per cache page (a multiple of 8).
@@ -55,7 +58,7 @@ class LLM:
                  max_num_batched_tokens: int = 2048, prefill_chunk: int | None = None,
                  device: str | torch.device = "auto", kv_backend: str = "paged",
                  scheduling: str = "continuous", attention_backend: str = "auto",
-                 attention_policy: str = "full", draft_model=None) -> None:
+                 attention_policy: str = "full", draft_model=None, seed: int = 0) -> None:
         given = {"kv_backend": kv_backend, "scheduling": scheduling, "attention_backend": attention_backend,
                  "attention_policy": attention_policy, "draft_model": draft_model}
         for name, value in given.items():
@@ -72,11 +75,21 @@ class LLM:
             raise ValueError(f"block_size must be >= 1, got {block_size}")
         if max_batch_size < 1:
             raise ValueError(f"max_batch_size must be >= 1, got {max_batch_size}")
-        folder = Path(model)
-        if not folder.is_dir():
-            raise FileNotFoundError(f"model folder {folder} does not exist (no download is attempted)")
         self.dtype = resolve_dtype(dtype)
-        self.architecture, self.model_config, plan = load_model_description(folder)
+        if hasattr(model, "architecture") and not isinstance(model, (str, Path)):
+            # a typed configuration: seeded random weights, no folder
+            folder = None
+            self.architecture = get_architecture(model.architecture)
+            self.model_config = model
+            plan = self.architecture.plan(model)
+            expected = {n: s for n, s in expected_tensors_of(plan).items() if not s.ignored}
+            source = RandomSource(expected, seed)
+        else:
+            folder = Path(model)
+            if not folder.is_dir():
+                raise FileNotFoundError(f"model folder {folder} does not exist (no download is attempted)")
+            self.architecture, self.model_config, plan = load_model_description(folder)
+            source = SafetensorsSource(folder)
         model_max = plan.max_position_embeddings
         self.max_seq_len = min(max_seq_len or model_max, model_max)
         pool_tokens = kv_pool_tokens or self.max_seq_len
@@ -88,10 +101,10 @@ class LLM:
         self.max_num_batched_tokens = max(max_num_batched_tokens, max_batch_size)
         self.prefill_chunk = prefill_chunk
         self.eos_token_ids = tuple(plan.eos_token_ids)
-        self.runner = ModelRunner(plan, SafetensorsSource(folder), dtype=self.dtype,
+        self.runner = ModelRunner(plan, source, dtype=self.dtype,
                                   page_size=block_size, kv_pool_tokens=pool_tokens,
                                   max_requests=max_batch_size, device=device)
-        self.tokenizer = self._load_tokenizer(folder)
+        self.tokenizer = self._load_tokenizer(folder) if folder is not None else None
         self.num_steps = 0
         self.num_preemptions = 0
 
