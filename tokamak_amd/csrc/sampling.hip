@@ -77,7 +77,8 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_segments_kernel(
 
 __global__ __launch_bounds__(kWave) void argmax_pick_kernel(const float* __restrict__ part_v,
                                                             const int* __restrict__ part_i,
-                                                            int* __restrict__ out) {
+                                                            int* __restrict__ out,
+                                                            float* __restrict__ out_value) {
   const int r = blockIdx.x, lane = threadIdx.x;
   float bv = lane < kArgmaxSegments ? part_v[r * kArgmaxSegments + lane] : -INFINITY;
   int bi = lane < kArgmaxSegments ? part_i[r * kArgmaxSegments + lane] : 0x7fffffff;
@@ -87,18 +88,22 @@ __global__ __launch_bounds__(kWave) void argmax_pick_kernel(const float* __restr
     const int oi = __shfl_xor(bi, m, kWave);
     argmax_take(bv, bi, ov, oi);
   }
-  if (lane == 0) out[r] = (bi == 0x7fffffff) ? 0 : bi;
+  if (lane == 0) {
+    out[r] = (bi == 0x7fffffff) ? 0 : bi;
+    if (out_value != nullptr) out_value[r] = bv;
+  }
 }
 
-// part_v, part_i: scratch of M * tk_argmax_segments() floats and ints.
+// part_v, part_i: scratch of M * tk_argmax_segments() floats and ints.  out_value
+// (optional, [M]) receives each row's maximum (-inf if the row holds no number).
 TK_API int tk_argmax_segments() { return kArgmaxSegments; }
 
-TK_API int tk_argmax(const float* logits, int* out, float* part_v, int* part_i, int M, int V, long ld,
-                     hipStream_t stream) {
+TK_API int tk_argmax(const float* logits, int* out, float* out_value, float* part_v, int* part_i, int M,
+                     int V, long ld, hipStream_t stream) {
   if (M <= 0) return 0;
   if (V <= 0 || M > 65535) return -1;
   argmax_segments_kernel<<<dim3(kArgmaxSegments, M), kArgmaxThreads, 0, stream>>>(logits, part_v, part_i, V, ld);
-  argmax_pick_kernel<<<M, kWave, 0, stream>>>(part_v, part_i, out);
+  argmax_pick_kernel<<<M, kWave, 0, stream>>>(part_v, part_i, out, out_value);
   return launch_status();
 }
 
@@ -207,7 +212,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p,
     const unsigned long long* __restrict__ seeds, const unsigned long long* __restrict__ counters,
-    int* __restrict__ out, float* __restrict__ probs_out) {
+    const float* __restrict__ row_max, int* __restrict__ out, float* __restrict__ probs_out) {
   __shared__ float fs[16];
   __shared__ unsigned long long hist64[kBins];       // counts use the same memory as 32-bit bins
   __shared__ unsigned long long scan64[kSampleThreads];
@@ -224,10 +229,10 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   const int k = top_k[r];
   const float p_keep = top_p[r];
 
-  float mx = -INFINITY;
-#pragma unroll 8
-  for (int i = tid; i < V; i += nt) mx = fmaxf(mx, row[i] * inv_t);
-  mx = block_max(mx, fs);
+  // the row's maximum comes from the argmax pass that ran before (temperature > 0
+  // keeps the order); a row without any number has nothing to draw from
+  const float mx = row_max[r] * inv_t;
+  if (!(mx > -INFINITY)) return;
 
   // top-k: kth = the k-th largest scaled logit (everything >= it survives)
   uint32_t kth = 0;  // ordered(-inf) is > 0, so 0 keeps everything
@@ -378,15 +383,16 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   }
 }
 
-// `out` must already hold each row's argmax (tk_argmax): greedy rows keep it, and so
-// does a row whose segment search falls through (rounding at a segment edge).
+// `out` must already hold each row's argmax and `row_max` its maximum (tk_argmax): greedy
+// rows keep the argmax, and so does a row whose search falls through (rounding at an edge).
 TK_API int tk_sample(const float* logits, long ld, int M, int V, const float* temperature,
                      const int* top_k, const float* top_p, const unsigned long long* seeds,
-                     const unsigned long long* counters, int* out, float* probs_out,
-                     hipStream_t stream) {
+                     const unsigned long long* counters, const float* row_max, int* out,
+                     float* probs_out, hipStream_t stream) {
   if (M <= 0) return 0;
   if (V <= 0) return -1;
+  if (row_max == nullptr) return -1;
   sample_kernel<<<M, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, seeds, counters,
-                                        out, probs_out);
+                                                  row_max, out, probs_out);
   return launch_status();
 }

@@ -113,10 +113,10 @@ _SIGS = {
                               c_int, c_int, c_int, c_int, c_float, c_void_p],
     },
     "sampling": {
-        "tk_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+        "tk_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
         "tk_argmax_segments": [],
         "tk_sample": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                      c_void_p, c_void_p, c_void_p, c_void_p],
+                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     },
 }
 _fns: dict[str, ctypes._CFuncPtr] = {}
@@ -411,19 +411,22 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     return True
 
 
-def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
-    """out[m] = index of the first maximum of logits[m]."""
+def argmax(logits: torch.Tensor, out: torch.Tensor, values: torch.Tensor | None = None) -> None:
+    """out[m] = index of the first maximum of logits[m]; ``values`` (optional, float32
+    [M]) receives the maxima."""
     _need(logits.is_cuda and logits.dim() == 2 and logits.stride(1) == 1 and logits.dtype == torch.float32,
           "logits are float32 [M, V] on the GPU")
     _gpu(out)
     m, v = logits.shape
     _need(out.dtype == torch.int32 and out.numel() >= m, "argmax output is int32 [M]")
     _need(m <= 65535, "at most 65535 rows")
+    _need(values is None or (values.is_cuda and values.dtype == torch.float32 and values.numel() >= m
+                             and values.is_contiguous()), "argmax values are float32 [M]")
     segments = _fn("sampling", "tk_argmax_segments")()
     part_v = torch.empty(m * segments, dtype=torch.float32, device=logits.device)
     part_i = torch.empty(m * segments, dtype=torch.int32, device=logits.device)
-    _check(_fn("sampling", "tk_argmax")(_p(logits), _p(out), _p(part_v), _p(part_i), m, v, logits.stride(0),
-                                        _stream()), "argmax")
+    _check(_fn("sampling", "tk_argmax")(_p(logits), _p(out), _p(values), _p(part_v), _p(part_i), m, v,
+                                        logits.stride(0), _stream()), "argmax")
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
@@ -441,7 +444,8 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
         _need(t.numel() >= m, "one sampling parameter per row is required")
     _need(out.dtype == torch.int32, "sample output is int32")
     _need(probs_out is None or (probs_out.dtype == torch.float32 and probs_out.shape == (m, v)), "probs_out is float32 [M, V]")
-    argmax(logits, out)  # greedy rows are done with this; the others overwrite it
+    row_max = torch.empty((m,), dtype=torch.float32, device=logits.device)
+    argmax(logits, out, row_max)  # greedy rows are done with this; the others overwrite it
     _check(_fn("sampling", "tk_sample")(_p(logits), logits.stride(0), m, v, _p(temperature), _p(top_k),
-                                        _p(top_p), _p(seeds), _p(counters), _p(out), _p(probs_out),
-                                        _stream()), "sample")
+                                        _p(top_p), _p(seeds), _p(counters), _p(row_max), _p(out),
+                                        _p(probs_out), _stream()), "sample")
