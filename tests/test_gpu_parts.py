@@ -186,3 +186,22 @@ def test_sampling_vectors_and_seeds():
     assert a[0] == a[1]                     # same seed and draw count: same token
     counts = torch.bincount(torch.tensor(draws(torch.tensor([[0.5, 0.3, 0.2]]).log(), SamplingParams(), 4000)), minlength=3)
     torch.testing.assert_close(counts.float() / 4000, torch.tensor([0.5, 0.3, 0.2]), rtol=0, atol=0.03)
+
+
+def test_sampling_odd_rows():
+    """A NaN or -inf logit is never drawn; a row that holds nothing but those keeps
+    token 0 like the argmax; a vocabulary that is no multiple of four."""
+    from tokamak_amd import SamplingParams
+    from tokamak_amd.sampling.sampler import sample_tokens
+
+    V = 1001
+    logits = torch.randn(4, V, generator=torch.Generator().manual_seed(3))
+    logits[0, ::2] = float("nan")
+    logits[1, 1::2] = float("-inf")
+    logits[2, :] = float("-inf")
+    logits[3, :] = float("nan")
+    logits[3, 777] = -5.0
+    for params in (SamplingParams(temperature=1.5), SamplingParams(temperature=0.7, top_k=30, top_p=0.9)):
+        for draw in range(20):
+            t = sample_tokens(logits.to(DEV), [params] * 4, [11, 12, 13, 14], [draw] * 4).cpu().tolist()
+            assert t[0] % 2 == 1 and t[1] % 2 == 0 and t[2] == 0 and t[3] == 777

@@ -193,6 +193,12 @@ __device__ __forceinline__ void crossing_bin(const T* hist, int nbins, T target,
   __syncthreads();
 }
 
+// logit / temperature; a NaN is treated as -inf (never kept, never drawn), as the argmax does
+__device__ __forceinline__ float scaled(float logit, float inv_t) {
+  const float x = logit * inv_t;
+  return x == x ? x : -INFINITY;
+}
+
 // exp(x - max) as a 32.32 fixed-point number: integer sums do not depend on the
 // order of addition, so thresholds found from them are the same on every run
 __device__ __forceinline__ unsigned long long fixed_mass(float x, float mx) {
@@ -246,7 +252,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
       __syncthreads();
 #pragma unroll 8
       for (int i = tid; i < V; i += nt) {
-        const uint32_t o = ordered(row[i] * inv_t);
+        const uint32_t o = ordered(scaled(row[i], inv_t));
         const bool in_bin = level == 0 || (o >> (shift + (level == 1 ? 12 : 8))) == prefix;
         if (in_bin) atomicAdd(&hist32[(o >> shift) & (uint32_t)(nbins - 1)], 1u);
       }
@@ -274,7 +280,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
       __syncthreads();
 #pragma unroll 8
       for (int i = tid; i < V; i += nt) {
-        const float x = row[i] * inv_t;
+        const float x = scaled(row[i], inv_t);
         const uint32_t o = ordered(x);
         const bool in_bin = level == 0 || (o >> (shift + (level == 1 ? 12 : 8))) == prefix;
         if (in_bin && o >= kth) atomicAdd(&hist64[(o >> shift) & (uint32_t)(nbins - 1)], fixed_mass(x, mx));
@@ -307,7 +313,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   float mine = 0.f;
 #pragma unroll 8
   for (int i = c_begin + lane; i < c_end; i += kWave) {
-    const float x = row[i] * inv_t;
+    const float x = scaled(row[i], inv_t);
     if (ordered(x) >= cut) mine += expf(x - mx);
   }
   mine = wave_sum(mine);
@@ -325,7 +331,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     float* po = probs_out + (size_t)r * V;
 #pragma unroll 8
     for (int i = tid; i < V; i += nt) {
-      const float x = row[i] * inv_t;
+      const float x = scaled(row[i], inv_t);
       po[i] = (ordered(x) >= cut) ? expf(x - mx) / total : 0.f;
     }
   }
@@ -341,7 +347,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     float mine_run = 0.f;
     int last_kept = -1;
     for (int i = r_begin; i < r_end; ++i) {
-      const float x = row[i] * inv_t;
+      const float x = scaled(row[i], inv_t);
       if (ordered(x) >= cut) {
         mine_run += expf(x - mx);
         last_kept = i;
@@ -359,7 +365,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     if (before + excl <= target && target < before + incl) {
       float run = before + excl;
       for (int i = r_begin; i < r_end; ++i) {
-        const float x = row[i] * inv_t;
+        const float x = scaled(row[i], inv_t);
         if (ordered(x) >= cut) {
           run += expf(x - mx);
           if (run > target) {
