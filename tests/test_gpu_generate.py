@@ -174,6 +174,16 @@ def test_typed_configuration_gives_the_weights_of_a_written_folder(tmp_path):
     assert [o.output_token_ids for o in a] != [o.output_token_ids for o in c]
 
 
+def test_default_pool_holds_every_running_request_at_full_length(folders):
+    from tokamak_amd import LLM
+
+    llm = LLM(folders["A"], dtype="float32", max_seq_len=96, max_batch_size=5)
+    assert llm.runner.kv_pool_tokens == 5 * 96
+    assert llm.runner.manager.num_pages() == 5 * 96 // 16
+    with pytest.raises(ValueError, match="kv_pool_tokens"):
+        LLM(folders["A"], dtype="float32", max_seq_len=96, kv_pool_tokens=95)
+
+
 def test_command_line(folders, capsys):
     from tokamak_amd import cli
 

@@ -36,9 +36,11 @@ class LLM:
         dtype: ``"bfloat16"`` (default) or ``"float32"`` (everything in true 32-bit).
         max_seq_len: cap on one request's context; default the model's maximum.
         block_size: tokens per cache page (a multiple of 8).
-        kv_pool_tokens: capacity of the page pool in tokens; default
-            ``max_seq_len``; must be at least ``max_seq_len`` so a request can
-            always finish alone.
+        kv_pool_tokens: capacity of the page pool in tokens; must be at least
+            ``max_seq_len`` so a request can always finish alone.  Default: room for
+            ``max_batch_size`` requests of ``max_seq_len`` tokens, within 90 % of the
+            memory that the weights leave free (the reference's default, ``max_seq_len``,
+            would serve one long request at a time).
         max_batch_size: most sequences running at once.
         max_num_batched_tokens: token budget of one step (new).
         prefill_chunk: longest prompt portion in one step (new; default the budget).
@@ -92,18 +94,20 @@ class LLM:
             source = SafetensorsSource(folder)
         model_max = plan.max_position_embeddings
         self.max_seq_len = min(max_seq_len or model_max, model_max)
-        pool_tokens = kv_pool_tokens or self.max_seq_len
-        if pool_tokens < self.max_seq_len:
+        if kv_pool_tokens is not None and kv_pool_tokens < self.max_seq_len:
             raise ValueError(
-                f"kv_pool_tokens ({pool_tokens}) must be >= max_seq_len ({self.max_seq_len}) "
+                f"kv_pool_tokens ({kv_pool_tokens}) must be >= max_seq_len ({self.max_seq_len}) "
                 f"so any single request can complete alone")
         self.max_batch_size = max_batch_size
         self.max_num_batched_tokens = max(max_num_batched_tokens, max_batch_size)
         self.prefill_chunk = prefill_chunk
         self.eos_token_ids = tuple(plan.eos_token_ids)
         self.runner = ModelRunner(plan, source, dtype=self.dtype,
-                                  page_size=block_size, kv_pool_tokens=pool_tokens,
-                                  max_requests=max_batch_size, device=device)
+                                  page_size=block_size, kv_pool_tokens=kv_pool_tokens,
+                                  max_requests=max_batch_size, device=device,
+                                  min_pool_tokens=self.max_seq_len, tokens_per_request=self.max_seq_len)
+        if self.runner.kv_pool_tokens < self.max_seq_len:
+            raise RuntimeError(f"the GPU has no room for a cache of max_seq_len ({self.max_seq_len}) tokens")
         self.tokenizer = self._load_tokenizer(folder) if folder is not None else None
         self.num_steps = 0
         self.num_preemptions = 0

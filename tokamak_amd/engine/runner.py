@@ -48,8 +48,10 @@ class StepEntry:
 
 class ModelRunner:
     def __init__(self, plan, source, *, dtype="bfloat16", page_size: int = 16,
-                 kv_pool_tokens: int, max_requests: int = 64,
-                 device: str | torch.device = "cuda:0", use_graphs: bool = True) -> None:
+                 kv_pool_tokens: int | None, max_requests: int = 64,
+                 device: str | torch.device = "cuda:0", use_graphs: bool = True,
+                 min_pool_tokens: int = 0, tokens_per_request: int | None = None,
+                 memory_fraction: float = 0.9) -> None:
         self.dtype = resolve_dtype(dtype)
         self.device = torch.device(device)
         if self.device.type != "cuda" or not torch.cuda.is_available():
@@ -60,7 +62,16 @@ class ModelRunner:
         self.page_size = page_size
         self.model = LayeredModel(plan, dtype=self.dtype, device=self.device)
         load_weights(self.model, source, dtype=self.dtype, device=self.device)
-        groups, _ = self.model.cache_layout()
+        groups, layouts = self.model.cache_layout()
+        if kv_pool_tokens is None:
+            # room for every request at full length, within a share of what the weights left free
+            elem = torch.empty((), dtype=self.dtype).element_size()
+            per_token = sum(lay.request.elems_per_token * len(lay.request.arrays) * elem for lay in layouts.values())
+            free, _ = torch.cuda.mem_get_info(self.device)
+            fits = int(free * memory_fraction) // max(per_token, 1)
+            longest = tokens_per_request or plan.max_position_embeddings
+            kv_pool_tokens = max(min_pool_tokens, min(max_requests * longest, fits))
+        self.kv_pool_tokens = int(kv_pool_tokens)
         num_pages = max(1, -(-int(kv_pool_tokens) // page_size))
         self.manager = CacheManager(groups, num_pages, page_size, max_requests)
         self.storage = CacheStorage(self.model, [num_pages] * len(groups), page_size, max_requests,
