@@ -184,6 +184,25 @@ def test_default_pool_holds_every_running_request_at_full_length(folders):
         LLM(folders["A"], dtype="float32", max_seq_len=96, kv_pool_tokens=95)
 
 
+def test_decode_batches_beyond_the_captured_size_run_eagerly(folders):
+    """70 running sequences: decode steps of more than 64 tokens use the library product,
+    which is kept out of HIP graphs; the tokens are those of running each prompt alone."""
+    from tokamak_amd import LLM, SamplingParams
+
+    folder = folders["D"]
+    cfg, _ = plain.read_folder(folder)
+    prompts = [random_ids(cfg["vocab_size"], 3 + i % 5, 300 + i) for i in range(70)]
+    params = SamplingParams(temperature=0.0, max_new_tokens=4, ignore_eos=True)
+    wide = LLM(folder, dtype="bfloat16", max_seq_len=32, max_batch_size=70)
+    got = wide.generate(prompt_token_ids=prompts, sampling_params=params)
+    assert not wide.runner._graphs                      # no step was captured
+    narrow = LLM(folder, dtype="bfloat16", max_seq_len=32, max_batch_size=1)
+    want = narrow.generate(prompt_token_ids=prompts[:6], sampling_params=params)
+    assert narrow.runner._graphs
+    same = sum(a.output_token_ids == b.output_token_ids for a, b in zip(got[:6], want))
+    assert same >= 5                                    # bf16 rounding may flip a near tie
+
+
 def test_command_line(folders, capsys):
     from tokamak_amd import cli
 

@@ -25,6 +25,7 @@ from tokamak_amd.weights.loader import load_weights
 from tokamak_amd.weights.sources import SafetensorsSource
 
 MAX_GRAPHS = 256   # captured decode shapes kept; the one used longest ago goes first
+MAX_GRAPH_BATCH = 64   # larger decode batches use the library product, which is not recorded
 
 DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32,
           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
@@ -175,7 +176,8 @@ class ModelRunner:
         if not entries:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
         with torch.cuda.device(self.device):
-            if (self.use_graphs and all(len(e.tokens) == 1 for e in entries)
+            if (self.use_graphs and len(entries) <= MAX_GRAPH_BATCH
+                    and all(len(e.tokens) == 1 for e in entries)
                     and all(list(e.want) in ([], [0]) for e in entries)):
                 logits = self._graph_step(entries)
             else:
