@@ -136,34 +136,35 @@ def time_decode(runner, cfg, batch, context, steps, warmup):
 
 def run_continuous(args) -> int:
     """Optional extra workload: continuous batching through ``LLM.generate`` (scheduler,
-    portions of prompts beside decode tokens, captured decode steps).  Prompt lengths
-    uniform in [32, 1024], outputs uniform in [16, 256], greedy, seeded."""
+    portions of prompts beside decode tokens, captured decode steps).  Prompt and output
+    lengths uniform in the given ranges, greedy, seeded."""
     import random
-    import tempfile
 
     import torch
 
     from tokamak_amd import LLM, SamplingParams
     from tokamak_amd.models.qwen3 import PRESETS
-    from tokamak_amd.weights import write_random_model
 
-    cfg = dataclasses.replace(PRESETS[args.model], max_position_embeddings=4096)
+    p_lo, p_hi = (int(x) for x in args.prompt_tokens.split(","))
+    o_lo, o_hi = (int(x) for x in args.output_tokens.split(","))
+    max_len = max(4096, p_hi + o_hi)
+    cfg = dataclasses.replace(PRESETS[args.model], max_position_embeddings=max_len)
     rng = random.Random(0)
-    prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(32, 1024))] for _ in range(args.requests)]
-    params = [SamplingParams(temperature=0.0, max_new_tokens=rng.randint(16, 256), ignore_eos=True)
+    prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(p_lo, p_hi))] for _ in range(args.requests)]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=rng.randint(o_lo, o_hi), ignore_eos=True)
               for _ in range(args.requests)]
-    with tempfile.TemporaryDirectory(prefix="tokamak_bench_") as tmp:
-        folder = write_random_model(tmp, cfg, 0)
-        llm = LLM(folder, dtype=args.dtype, max_seq_len=4096, kv_pool_tokens=args.max_batch * 1300,
-                  max_batch_size=args.max_batch, max_num_batched_tokens=2048, prefill_chunk=2048)
-        runs = []
-        for _ in range(2):  # the first run also records the decode graphs
-            steps0 = llm.num_steps
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            outs = llm.generate(prompt_token_ids=prompts, sampling_params=params)
-            torch.cuda.synchronize()
-            runs.append((time.perf_counter() - t0, llm.num_steps - steps0))
+    pool = args.max_batch * (p_hi + o_hi)  # every running request fits at full length
+    llm = LLM(cfg, seed=0, random_weights_on_gpu=True, dtype=args.dtype, max_seq_len=max_len,
+              kv_pool_tokens=max(pool, max_len), max_batch_size=args.max_batch, max_num_batched_tokens=2048,
+              prefill_chunk=2048)
+    runs = []
+    for _ in range(2):  # the first run also records the decode graphs
+        steps0 = llm.num_steps
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        outs = llm.generate(prompt_token_ids=prompts, sampling_params=params)
+        torch.cuda.synchronize()
+        runs.append((time.perf_counter() - t0, llm.num_steps - steps0))
     elapsed, steps = runs[-1]
     out_tokens = sum(len(o.output_token_ids) for o in outs)
     print(json.dumps({
@@ -174,6 +175,7 @@ def run_continuous(args) -> int:
         "data": "synthetic (seeded lengths and token ids, random weights)",
         "config": {"model": f"{args.model}-shaped", "requests": args.requests, "max_batch": args.max_batch,
                    "prompt_tokens": sum(map(len, prompts)), "output_tokens": out_tokens,
+                   "total_tok_per_s": round((sum(map(len, prompts)) + out_tokens) / elapsed, 1),
                    "first_run_s": round(runs[0][0], 3), "preemptions": llm.num_preemptions,
                    "parallelism": "single GPU"},
     }))
@@ -221,6 +223,8 @@ def main() -> int:
                     help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
     ap.add_argument("--requests", type=int, default=256)
     ap.add_argument("--max-batch", type=int, default=64)
+    ap.add_argument("--prompt-tokens", default="32,1024", help="continuous workload: MIN,MAX prompt length")
+    ap.add_argument("--output-tokens", default="16,256", help="continuous workload: MIN,MAX output length")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")

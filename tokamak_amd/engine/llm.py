@@ -32,7 +32,8 @@ class LLM:
     src/tokamak/engine/llm.py:64-104):
         model: folder with ``config.json`` and ``*.safetensors``; or an architecture's
             typed configuration (e.g. ``Qwen3Config``) for seeded random weights
-            (``seed``; the same weights ``write_random_model`` would put in a folder).
+            (``seed``; the same weights ``write_random_model`` would put in a folder, unless
+            ``random_weights_on_gpu`` draws them on the GPU, which is what a large shape needs).
         dtype: ``"bfloat16"`` (default) or ``"float32"`` (everything in true 32-bit).
         max_seq_len: cap on one request's context; default the model's maximum.
         block_size: tokens per cache page (a multiple of 8).
@@ -60,7 +61,8 @@ class LLM:
                  max_num_batched_tokens: int = 2048, prefill_chunk: int | None = None,
                  device: str | torch.device = "auto", kv_backend: str = "paged",
                  scheduling: str = "continuous", attention_backend: str = "auto",
-                 attention_policy: str = "full", draft_model=None, seed: int = 0) -> None:
+                 attention_policy: str = "full", draft_model=None, seed: int = 0,
+                 random_weights_on_gpu: bool = False) -> None:
         given = {"kv_backend": kv_backend, "scheduling": scheduling, "attention_backend": attention_backend,
                  "attention_policy": attention_policy, "draft_model": draft_model}
         for name, value in given.items():
@@ -85,7 +87,9 @@ class LLM:
             self.model_config = model
             plan = self.architecture.plan(model)
             expected = {n: s for n, s in expected_tensors_of(plan).items() if not s.ignored}
-            source = RandomSource(expected, seed)
+            # drawn on the CPU they equal a folder written with the same seed; on the GPU
+            # they differ from that but take seconds for tens of billions of parameters
+            source = RandomSource(expected, seed, device=device if random_weights_on_gpu else "cpu")
         else:
             folder = Path(model)
             if not folder.is_dir():
