@@ -128,6 +128,22 @@ def test_short_portions_over_long_contexts_split_their_keys(nh, nkv, hd, ps):
         torch.testing.assert_close(g, w, **TOL[torch.bfloat16])
 
 
+def test_many_tiles_over_long_contexts_use_the_four_wave_kernel():
+    """Two portions that both start beyond 2,048 cached tokens and fill the GPU without
+    splitting: the dispatcher takes the kernel variant built for four waves a SIMD
+    (checked by its conditions), with the same results."""
+    from tokamak_amd.kernels import attention
+
+    nh, nkv, hd, ps = 32, 8, 128, 16
+    requests = [(2100, 300), (2500, 250)]
+    tiles = sum(-(-q // 16) for _, q in requests)
+    assert attention.tile_split(tiles, nkv, 2800)[1] == 1 and min(c for c, _ in requests) >= attention.DENSE_TILES_FROM
+    got, want = run_attention(torch.bfloat16, nh, nkv, hd, ps, requests, seed=13)
+    for g, w in zip(got, want):
+        assert torch.isfinite(g).all()
+        torch.testing.assert_close(g, w, **TOL[torch.bfloat16])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("far", [0, 3, 255, 256, 511, 777])
 def test_a_far_key_among_hundreds_is_found(dtype, far):

@@ -281,8 +281,11 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(
 // ---------------------------------------------------------------------------
 constexpr int kPrefillThreads = 256;
 
-template <int HD, int HPB>
-__global__ __launch_bounds__(kPrefillThreads) __attribute__((amdgpu_waves_per_eu(2)))
+// OCC: waves a SIMD the compiler must leave room for.  Three (what OCC = 2 gives) are best
+// when tiles differ in length (a prompt from position zero: the longest tile's walk
+// decides); four (a few registers spilled) when every tile walks a long context.
+template <int HD, int HPB, int OCC>
+__global__ __launch_bounds__(kPrefillThreads) __attribute__((amdgpu_waves_per_eu(OCC)))
 void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
@@ -526,7 +529,7 @@ void attention_prefill_kernel(
 #undef TK_FETCH
 #undef TK_PAGES
 
-template <int HD, int HPB>
+template <int HD, int HPB, int OCC>
 static int launch_prefill(const void* q, const void* k_cache, const void* v_cache,
                           const int* block_tables, int max_pages, const int* positions,
                           const int* req_of_token, const int* item_token, const int* item_count,
@@ -534,7 +537,7 @@ static int launch_prefill(const void* q, const void* k_cache, const void* v_cach
                           int split_keys, int nh, int nkv, int ps, float scale, hipStream_t stream) {
   const int G = nh / nkv;
   dim3 grid(nkv * (G / HPB), num_items, nsplit);
-  attention_prefill_kernel<HD, HPB><<<grid, kPrefillThreads, 0, stream>>>(
+  attention_prefill_kernel<HD, HPB, OCC><<<grid, kPrefillThreads, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
       positions, req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit,
       split_keys, num_items, nh, nkv, ps, scale * 1.4426950408889634f);
@@ -569,6 +572,7 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
 // mode 0: heads (every item is one decode token; item_count is ignored)
 // mode 1: tokens (item = up to 16 consecutive tokens of one request; with nsplit > 1 split_keys
 //         is a multiple of 64 and the partial buffers hold 16 rows per item)
+// mode 2: tokens, every tile over a long context (same results; the kernel built for four waves a SIMD)
 // Returns -2 if this shape is not instantiated (the caller uses the generic kernel).
 TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const void* v_cache,
                              const int* block_tables, int max_pages, const int* positions,
@@ -577,6 +581,7 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
                              int split_keys, int nh, int nkv, int hd, int ps, float scale,
                              hipStream_t stream) {
   if (num_items <= 0) return 0;
+  if (mode < 0 || mode > 2) return -1;
   if (nkv <= 0 || nh % nkv != 0 || ps < 16 || (ps & (ps - 1)) != 0 || split_keys % 16 != 0 || nsplit < 1) return -1;
   if (num_items > 65535 || nh > 65535) return -1;
   const int G = nh / nkv;
@@ -595,15 +600,16 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
 #define TK_PARGS                                                                                  \
   q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
       num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream
+  const bool dense = mode == 2;
   if (hd == 128) {
-    if (hpb == 4) return launch_prefill<128, 4>(TK_PARGS);
-    if (hpb == 2) return launch_prefill<128, 2>(TK_PARGS);
-    return launch_prefill<128, 1>(TK_PARGS);
+    if (hpb == 4) return dense ? launch_prefill<128, 4, 4>(TK_PARGS) : launch_prefill<128, 4, 2>(TK_PARGS);
+    if (hpb == 2) return launch_prefill<128, 2, 2>(TK_PARGS);
+    return launch_prefill<128, 1, 2>(TK_PARGS);
   }
   if (hd == 64) {
-    if (hpb == 4) return launch_prefill<64, 4>(TK_PARGS);
-    if (hpb == 2) return launch_prefill<64, 2>(TK_PARGS);
-    return launch_prefill<64, 1>(TK_PARGS);
+    if (hpb == 4) return launch_prefill<64, 4, 2>(TK_PARGS);
+    if (hpb == 2) return launch_prefill<64, 2, 2>(TK_PARGS);
+    return launch_prefill<64, 1, 2>(TK_PARGS);
   }
 #undef TK_PARGS
 #undef TK_ARGS

@@ -50,6 +50,7 @@ class StepBatch:
     num_tiles: int = 0
     max_decode_len: int = 0                     # longest context among the decode tokens
     max_tile_len: int = 0                       # longest context (with the portion) among the tiled spans
+    min_tile_ctx: int = 0                       # shortest cached context among the tiled spans
     # host copies, for choosing kernels and grids
     q_lens: list[int] = field(default_factory=list)
     ctx_lens: list[int] = field(default_factory=list)
@@ -79,6 +80,7 @@ class PackedBatch:
     ctx_lens: list[int]
     max_decode_len: int
     max_tile_len: int = 0
+    min_tile_ctx: int = 0
 
 
 def table_width(longest: int, fixed: int | None = None) -> int:
@@ -144,7 +146,8 @@ def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] |
         num_decode=nd, num_tiles=nt, q_lens=[len(s.tokens) for s in spans],
         ctx_lens=[s.ctx_len for s in spans],
         max_decode_len=max((s.ctx_len + 1 for s in spans if len(s.tokens) == 1), default=0),
-        max_tile_len=max((s.ctx_len + len(s.tokens) for s in spans if len(s.tokens) > 1), default=0))
+        max_tile_len=max((s.ctx_len + len(s.tokens) for s in spans if len(s.tokens) > 1), default=0),
+        min_tile_ctx=min((s.ctx_len for s in spans if len(s.tokens) > 1), default=0))
 
 
 def batch_from_device(packed: PackedBatch, dev: torch.Tensor) -> StepBatch:
@@ -159,6 +162,7 @@ def batch_from_device(packed: PackedBatch, dev: torch.Tensor) -> StepBatch:
         decode_tokens=parts[7], tile_first=parts[8], tile_count=parts[9],
         num_decode=packed.num_decode, num_tiles=packed.num_tiles,
         max_decode_len=packed.max_decode_len, max_tile_len=packed.max_tile_len,
+        min_tile_ctx=packed.min_tile_ctx,
         q_lens=packed.q_lens, ctx_lens=packed.ctx_lens,
         max_q_len=max(packed.q_lens, default=0),
         max_seq_len=max((c + q for c, q in zip(packed.ctx_lens, packed.q_lens)), default=0),

@@ -13,6 +13,7 @@ FEW_DECODE_WAVES = 512      # below this many waves the splits are halved again
 TILE_SPLIT_BELOW_BLOCKS = 256   # a portion with fewer blocks than this has its keys split ...
 TILE_SPLIT_MIN_KEYS = 512       # ... into pieces no shorter than this
 TARGET_TILE_BLOCKS = 1024
+DENSE_TILES_FROM = 2048         # every tiled span starts at least this deep: the four-wave kernel
 
 
 def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
@@ -73,7 +74,8 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
             group = num_heads // num_kv_heads
             per_tile = num_kv_heads * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
             split, nsplit = tile_split(batch.num_tiles, per_tile, batch.max_tile_len)
-            ops.attention_mfma("tokens", q, k_cache, v_cache, block_tables, batch.positions,
+            dense = nsplit == 1 and batch.min_tile_ctx >= DENSE_TILES_FROM
+            ops.attention_mfma("tokens_dense" if dense else "tokens", q, k_cache, v_cache, block_tables, batch.positions,
                                batch.req_of_token, batch.tile_first, batch.tile_count, batch.num_tiles,
                                out, split_keys=split, num_splits=nsplit, **common)
         return

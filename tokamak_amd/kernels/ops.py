@@ -374,7 +374,8 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
                    page_size: int, scale: float, split_keys: int = 256, num_splits: int = 1) -> bool:
     """bf16 attention on the matrix cores.  ``mode`` "heads": every item is one
     decode token; "tokens": every item is up to 16 consecutive tokens of one
-    request.  With ``num_splits`` > 1 the keys of an item are cut into pieces of
+    request ("tokens_dense": the same, with the kernel variant for tiles that all
+    walk a long context).  With ``num_splits`` > 1 the keys of an item are cut into pieces of
     ``split_keys`` (a multiple of 16; of 64 in "tokens" mode), each its own block, and a
     second kernel merges the pieces.  Returns False (nothing launched) if the shape
     is not instantiated."""
@@ -390,18 +391,19 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32 and block_tables.dtype == torch.int32
           and item_token.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
     _need(item_token.numel() >= num_items and 0 < num_items <= 65535, "bad item list")
-    if mode == "tokens":
+    _need(mode in ("heads", "tokens", "tokens_dense"), "mode is heads, tokens or tokens_dense")
+    if mode != "heads":
         _need(item_count is not None and item_count.dtype == torch.int32 and item_count.numel() >= num_items,
               "tokens mode needs item counts")
         _need(num_splits == 1 or (split_keys % 64 == 0 and num_items * 16 <= 65535),
               "tokens mode splits keys in multiples of 64, for at most 4095 tiles")
     part_o = part_ml = None
     if num_splits > 1:
-        rows = num_items * (16 if mode == "tokens" else 1) * num_heads * num_splits
+        rows = num_items * (16 if mode != "heads" else 1) * num_heads * num_splits
         part_o = torch.empty((rows, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((rows, 2), dtype=torch.float32, device=q.device)
     status = _fn("attention_mfma", "tk_attention_mfma")(
-        0 if mode == "heads" else 1, _p(q), _p(k_cache), _p(v_cache), _p(block_tables),
+        {"heads": 0, "tokens": 1, "tokens_dense": 2}[mode], _p(q), _p(k_cache), _p(v_cache), _p(block_tables),
         block_tables.shape[1], _p(positions), _p(req_of_token), _p(item_token), _p(item_count),
         num_items, _p(out), _p(part_o), _p(part_ml), num_splits, split_keys, num_heads, num_kv_heads,
         head_dim, page_size, float(scale), _stream())
