@@ -306,8 +306,9 @@ def gemm_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
     accumulation), for prompt portions too long for the weight-streaming kernels.
     The plan of each shape is kept, and the algorithm of a shape class is chosen by
     timing the library's candidates once (csrc/blas_lt.hip).  Synchronises the first
-    time a shape class is seen, so it must not be recorded into a graph.  Returns
-    False if the library has no algorithm for the shape (nothing was computed)."""
+    time a shape class is seen, so it must not be recorded into a graph.  All calls on a
+    device share one workspace: launch them on one stream at a time (the engine has one).
+    Returns False if the library has no algorithm for the shape (nothing was computed)."""
     for t in (a, w, out):
         _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
         _need(t.dtype == torch.bfloat16 and t.data_ptr() % 16 == 0, "the library product is bfloat16 with 16-byte aligned operands")
