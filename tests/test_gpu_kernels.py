@@ -150,18 +150,25 @@ def test_a_far_key_among_hundreds_is_found(dtype, far):
     """One key (position ``far``) and the query are scaled so that its score
     stands out: the output must be that key's value.  Random weights alone would
     spread the softmax so thin that a skipped key could not be seen."""
-    hd = 128
+    hd, nh, nkv = 128, 8, 2
+    far_values = []
 
     def boost(q, k, v, ctx, qlen):
         direction = torch.nn.functional.normalize(torch.randn(hd, generator=torch.Generator().manual_seed(9)), dim=0)
-        k[far, :, :] = (direction * 12.0).to(k.dtype)
-        q[-1, :, :] = (direction * 12.0).to(q.dtype)
+        k[far, :, :] = (direction * 16.0).to(k.dtype)
+        q[-1, :, :] = (direction * 16.0).to(q.dtype)
+        far_values.append(v[far].float().clone())
 
-    got, want = run_attention(dtype, 8, 2, hd, 16, [(1023, 1), (1000, 24)], boost=boost, seed=4)
-    for g, w in zip(got, want):
+    got, want = run_attention(dtype, nh, nkv, hd, 16, [(1023, 1), (1000, 24)], boost=boost, seed=4)
+    for g, w, v_far in zip(got, want, far_values):
         torch.testing.assert_close(g, w, **TOL[dtype])
-        # and the reference itself says: the last query sees essentially one key
-        assert (w[-1] - w[-1]).abs().max() == 0
+        # the last query's score for the far key is 256 / sqrt(128) = 22.6, a thousand others
+        # lie around zero: its softmax weight is one to 1e-6, so the output is that key's value
+        # for every head of its group.  Should the boost stop dominating, this fails and says
+        # so, instead of leaving a comparison on random data that hides a skipped key.
+        expected = v_far.repeat_interleave(nh // nkv, dim=0)
+        torch.testing.assert_close(w[-1], expected, rtol=0, atol=1e-4)
+        torch.testing.assert_close(g[-1], expected, rtol=0, atol=1e-4 if dtype == torch.float32 else 2e-2)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])

@@ -1,6 +1,14 @@
 """Pins of the plain implementation beside the reference's text: vectors the
 reference's own tests hold, special cases that reduce to a library routine, and
-invariants, each chosen so that a plausible mistake fails it."""
+invariants, each chosen so that a plausible mistake fails it.
+
+The reference's own top test compares its model with the `transformers`
+implementation on a downloaded checkpoint (tests/integration/test_hf_parity.py:25-96).
+Neither a checkpoint nor another project's model code is used here, so parity
+with that implementation is unpinned; what stands in its place are the library
+compositions below (F.linear, F.rms_norm, F.scaled_dot_product_attention with its
+default scale, F.silu), which fix the scale, the place and value of eps, and which
+tensors are normed."""
 
 import math
 
@@ -23,6 +31,24 @@ def test_rmsnorm_formula_and_unit_rms():
     torch.testing.assert_close(out.pow(2).mean(-1).sqrt(), torch.ones(10), rtol=1e-3, atol=1e-3)
     # scale invariance (eps -> 0): a norm that forgot the rsqrt, or used the mean, fails
     torch.testing.assert_close(plain.rmsnorm(7.0 * x, w, 1e-12), plain.rmsnorm(x, w, 1e-12), rtol=1e-5, atol=1e-6)
+
+
+def test_rmsnorm_eps_sits_inside_the_root():
+    """Inputs so small that eps (1e-5) is ten times mean(x^2) (1e-6): with eps added
+    outside the root the result is 2.8 times larger, with eps left out 3.3 times.
+    Closed form, and the library routine that the form reduces to."""
+    torch.manual_seed(10)
+    eps = 1e-5
+    x = torch.randn(7, 96, dtype=torch.float64) * 1e-3
+    w = 1.0 + 0.1 * torch.randn(96, dtype=torch.float64)
+    ms = (x * x).sum(-1, keepdim=True) / 96
+    assert 0.5e-6 < float(ms.mean()) < 2e-6
+    expected = x / torch.sqrt(ms + eps) * w
+    got = plain.rmsnorm(x, w, eps)
+    torch.testing.assert_close(got, expected, rtol=1e-12, atol=0)
+    torch.testing.assert_close(got, F.rms_norm(x, (96,), w, eps), rtol=1e-12, atol=0)
+    outside = x / (torch.sqrt(ms) + eps) * w
+    assert float((outside.abs() / got.abs()).min()) > 2.0          # what the test would catch
 
 
 # -- RoPE (reference tests/unit/test_layers.py:30-68) -------------------------
@@ -160,7 +186,7 @@ def test_tied_head_uses_the_embedding(folders):
     torch.testing.assert_close(plain.logits([1, 2, 3], cfg, w), h @ w["model.embed_tokens.weight"].T)
 
 
-def test_qk_norm_comes_before_rotation_and_v_is_untouched(folders):
+def test_qk_norm_comes_before_rotation(folders):
     cfg, w = folders["B"]
     s = plain.sizes(cfg)
     torch.manual_seed(6)
@@ -173,6 +199,93 @@ def test_qk_norm_comes_before_rotation_and_v_is_untouched(folders):
     cos, sin = plain.rope_tables(torch.arange(4), s["hd"], s["theta"])
     rotated = plain.apply_rope(qn, cos, sin)
     torch.testing.assert_close(rotated.norm(dim=-1), torch.full((4, s["nh"]), math.sqrt(s["hd"])), rtol=1e-4, atol=1e-4)
+
+
+def _library_attention_block(h, w, p, cfg, positions):
+    """The attention sub-layer put together from library routines only: F.linear,
+    F.rms_norm over the head axis with the model's eps, and
+    F.scaled_dot_product_attention with its DEFAULT scale, which is
+    1/sqrt(q.size(-1)), the size of a head as q is laid out, whatever hidden/heads is.
+    Only the rotation comes from the plain implementation (pinned on its own above)."""
+    nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    eps = cfg["rms_norm_eps"]
+    T = h.shape[0]
+    q = F.rms_norm(F.linear(h, w[p + "q_proj.weight"]).view(T, nh, hd), (hd,), w[p + "q_norm.weight"], eps)
+    k = F.rms_norm(F.linear(h, w[p + "k_proj.weight"]).view(T, nkv, hd), (hd,), w[p + "k_norm.weight"], eps)
+    v = F.linear(h, w[p + "v_proj.weight"]).view(T, nkv, hd)
+    cos, sin = plain.rope_tables(positions, hd, float(cfg["rope_theta"]))
+    q, k = plain.apply_rope(q, cos, sin), plain.apply_rope(k, cos, sin)
+    rep = nh // nkv
+    o = F.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.transpose(0, 1).repeat_interleave(rep, 0)[None],
+        v.transpose(0, 1).repeat_interleave(rep, 0)[None], is_causal=True)[0].transpose(0, 1)
+    return F.linear(o.reshape(T, nh * hd), w[p + "o_proj.weight"])
+
+
+def test_attention_block_equals_library_composition_with_default_scale(folders):
+    """Configuration B has head_dim 32 while hidden/heads is 16: a softmax scale taken
+    from hidden/heads differs by sqrt(2) in every score and fails this.  The scores
+    are made large enough (q and k norm weights times 3, so |score| reaches ~10)
+    that the softmax is far from uniform and the scale shows in the output."""
+    cfg, w = folders["B"]
+    s = plain.sizes(cfg)
+    assert s["hd"] == 32 and s["H"] // s["nh"] == 16
+    p = "model.layers.1.self_attn."
+    w = {k: v.double() for k, v in w.items()}
+    w[p + "q_norm.weight"] = w[p + "q_norm.weight"] * 3.0
+    w[p + "k_norm.weight"] = w[p + "k_norm.weight"] * 3.0
+    torch.manual_seed(11)
+    h = torch.randn(19, s["H"], dtype=torch.float64)
+    positions = torch.arange(19)
+    ours = plain.attention_block(h, w, p, s, positions)
+    lib = _library_attention_block(h, w, p, cfg, positions)
+    torch.testing.assert_close(ours, lib, rtol=1e-9, atol=1e-12)
+    # what the pin catches: scores scaled by (hidden/heads)^-0.5 instead (the same as q
+    # norm weights times sqrt(2) here) move the output by far more than the tolerance
+    w_off = dict(w)
+    w_off[p + "q_norm.weight"] = w[p + "q_norm.weight"] * ((s["H"] // s["nh"]) ** -0.5 / s["hd"] ** -0.5)
+    off = plain.attention_block(h, w_off, p, s, positions)
+    assert float((off - lib).abs().max()) > 1e-3 * float(lib.abs().max())
+
+
+def test_qk_norms_use_the_models_eps_inside_the_root(folders):
+    """Hidden states so small that the mean square of a projected head (about 1e-6)
+    lies below eps (1e-5, configuration B): the per-head norms then depend on eps,
+    its place and its value, by a factor of about three.  Against the library
+    composition with F.rms_norm(eps=rms_norm_eps)."""
+    cfg, w = folders["B"]
+    s = plain.sizes(cfg)
+    assert s["eps"] == 1e-5
+    p = "model.layers.0.self_attn."
+    w = {k: v.double() for k, v in w.items()}
+    torch.manual_seed(12)
+    h = torch.randn(9, s["H"], dtype=torch.float64)
+    q = F.linear(h, w[p + "q_proj.weight"])
+    h = h * (1e-3 / float(q.pow(2).mean().sqrt()))                 # projected heads ~ 1e-3
+    positions = torch.arange(9)
+    ours = plain.attention_block(h, w, p, s, positions)
+    lib = _library_attention_block(h, w, p, cfg, positions)
+    torch.testing.assert_close(ours, lib, rtol=1e-9, atol=1e-15)
+    other = _library_attention_block(h, w, p, dict(cfg, rms_norm_eps=1e-6), positions)
+    assert float((other - lib).abs().max()) > 1e-3 * float(lib.abs().max())
+
+
+def test_v_is_not_normed(folders):
+    """Attention is linear in v: three times v_proj gives three times the sub-layer's
+    output.  A norm on v (as q and k have) would undo the factor."""
+    for key in ("A", "B"):
+        cfg, w = folders[key]
+        s = plain.sizes(cfg)
+        p = "model.layers.0.self_attn."
+        w = {k: v.double() for k, v in w.items()}
+        torch.manual_seed(13)
+        h = torch.randn(6, s["H"], dtype=torch.float64)
+        base = plain.attention_block(h, w, p, s, torch.arange(6))
+        w3 = dict(w)
+        w3[p + "v_proj.weight"] = w[p + "v_proj.weight"] * 3.0
+        torch.testing.assert_close(plain.attention_block(h, w3, p, s, torch.arange(6)), 3.0 * base,
+                                   rtol=1e-10, atol=1e-14)
+        assert float(base.abs().max()) > 1e-4
 
 
 def test_float64_agrees_with_float32(folders):
