@@ -10,6 +10,9 @@
 // over the ordered-integer image of the float values, three passes over the row
 // each (the row sits in L2).
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 using namespace tk;
 
@@ -104,6 +107,50 @@ TK_API int tk_argmax(const float* logits, int* out, float* out_value, float* par
   if (V <= 0 || M > 65535) return -1;
   argmax_segments_kernel<<<dim3(kArgmaxSegments, M), kArgmaxThreads, 0, stream>>>(logits, part_v, part_i, V, ld);
   argmax_pick_kernel<<<M, kWave, 0, stream>>>(part_v, part_i, out, out_value);
+  return launch_status();
+}
+
+// The same two kernels with their scratch in a fixed device array (see no_alloc.h).
+// `g_argmax_scratch` names the array for the device compiler; in host code the name is
+// only a handle, so the address each GPU gave its copy is looked up once per device
+// and the kernels get that pointer.
+constexpr int kNoAllocRows = TK_ARGMAX_NO_ALLOC_MAX_ROWS;
+constexpr int kMaxDevices = 64;
+struct ArgmaxScratch {
+  float value[kNoAllocRows * kArgmaxSegments];
+  int index[kNoAllocRows * kArgmaxSegments];
+};
+static __device__ __align__(256) ArgmaxScratch g_argmax_scratch;
+static ArgmaxScratch* g_argmax_scratch_ptr[kMaxDevices] = {};
+static std::mutex g_argmax_scratch_mutex;
+
+static ArgmaxScratch* argmax_scratch_of_current_device() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> guard(g_argmax_scratch_mutex);
+  if (g_argmax_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_argmax_scratch)) != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_argmax_scratch_ptr[device] = static_cast<ArgmaxScratch*>(ptr);
+  }
+  return g_argmax_scratch_ptr[device];
+}
+
+TK_API int tk_argmax_no_alloc_max_rows() { return kNoAllocRows; }
+
+TK_API int tk_argmax_no_alloc(const float* logits, int* out, float* out_value, int M, int V, long ld,
+                              hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (V <= 0 || logits == nullptr || out == nullptr || ld < V) return -1;
+  if (M > kNoAllocRows) return -3;
+  ArgmaxScratch* scratch = argmax_scratch_of_current_device();
+  if (scratch == nullptr) return -4;
+  argmax_segments_kernel<<<dim3(kArgmaxSegments, M), kArgmaxThreads, 0, stream>>>(
+      logits, scratch->value, scratch->index, V, ld);
+  argmax_pick_kernel<<<M, kWave, 0, stream>>>(scratch->value, scratch->index, out, out_value);
   return launch_status();
 }
 
