@@ -33,11 +33,11 @@ def make_runner(cfg, dtype, pool_tokens, max_requests, seed=0):
     import torch
 
     from tokamak_amd.engine.runner import ModelRunner
-    from tokamak_amd.models import qwen3
+    from tokamak_amd.config import get_architecture
     from tokamak_amd.weights.random_init import expected_tensors_of
     from tokamak_amd.weights.sources import RandomSource
 
-    plan = qwen3.plan(cfg)
+    plan = get_architecture(cfg.architecture).plan(cfg)
     expected = {n: s for n, s in expected_tensors_of(plan).items() if not s.ignored}
     tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     source = RandomSource(expected, seed, matrix_std=0.02, vector_jitter=0.0, dtype=tdt, device="cuda:0")
@@ -143,12 +143,12 @@ def run_continuous(args) -> int:
     import torch
 
     from tokamak_amd import LLM, SamplingParams
-    from tokamak_amd.models.qwen3 import PRESETS
+    from tokamak_amd.config import find_preset
 
     p_lo, p_hi = (int(x) for x in args.prompt_tokens.split(","))
     o_lo, o_hi = (int(x) for x in args.output_tokens.split(","))
     max_len = max(4096, p_hi + o_hi)
-    cfg = dataclasses.replace(PRESETS[args.model], max_position_embeddings=max_len)
+    cfg = dataclasses.replace(find_preset(args.model)[1], max_position_embeddings=max_len)
     rng = random.Random(0)
     prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(p_lo, p_hi))] for _ in range(args.requests)]
     params = [SamplingParams(temperature=0.0, max_new_tokens=rng.randint(o_lo, o_hi), ignore_eos=True)
@@ -234,9 +234,9 @@ def main() -> int:
 
     import torch
 
-    from tokamak_amd.models.qwen3 import PRESETS
+    from tokamak_amd.config import find_preset
 
-    full = PRESETS[args.shape]
+    full = find_preset(args.shape)[1]
     cfg = dataclasses.replace(full, num_layers=args.layers or full.num_layers)
     elem = 2 if args.dtype == "bfloat16" else 4
     max_batch = 64 if not (args.no_points or args.phase != "all") else args.batch

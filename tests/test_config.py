@@ -92,21 +92,27 @@ def test_plan_carries_every_number_as_part_parameters():
     cfg = qwen3.parse(raw(), ())
     plan = qwen3.plan(cfg)
     assert len(plan.layers) == 2 and [c.layer for c in plan.order] == [0, 1]
-    mixer = plan.layers[0].mixer
-    assert mixer.kind == "gqa_attention"
+    layer = plan.layers[0]
+    assert [role for role, _ in layer.parts] == ["mixer_norm", "mixer", "feed_forward_norm", "feed_forward", "position"]
+    assert layer.block.kind == "pre_norm"
+    mixer = layer.role("mixer").spec
+    assert mixer.kind == "gqa_attention" and layer.role("mixer").prefix == "self_attn."
     assert mixer["head_dim"] == 32 and mixer["num_kv_heads"] == 2
     assert mixer["softmax_scale"] == 32 ** -0.5   # the configured head_dim, not hidden/heads
     assert mixer["qk_norm_eps"] == 1e-6
-    kind, params = mixer["position"]
-    assert kind == "rotary_half" and dict(params) == {"rotary_dim": 32, "theta": 1e6}
-    assert plan.layers[0].feed_forward["intermediate_size"] == 128
+    position = layer.role("position")
+    assert position.spec.kind == "rotary_half" and position.spec.as_dict() == {"rotary_dim": 32, "theta": 1e6}
+    assert position.shared and position.prefix == ""
+    assert layer.role("feed_forward").spec["intermediate_size"] == 128
+    assert layer.role("mixer_norm").spec["eps"] == 1e-6
     assert plan.head["tied"] is True
 
 
 def test_run_order_is_validated_data():
     spec = qwen3.plan(qwen3.parse(raw(), ()))
     kw = dict(vocab_size=10, hidden_size=8, max_position_embeddings=16, tie_word_embeddings=False,
-              embedding=spec.embedding, layers=spec.layers, final_norm=spec.final_norm, head=spec.head)
+              embedding=spec.embedding, layers=spec.layers, final_norm=spec.final_norm, head=spec.head,
+              embedding_prefix="e.", layer_prefix="l.{}.", final_norm_prefix="n.", head_prefix="h.")
     ModelPlan(order=(LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2), LayerCall(1, 0, writes_cache=False)), **kw)
     with pytest.raises(ValueError, match="names layer 5"):
         ModelPlan(order=(LayerCall(5, 0),), **kw)

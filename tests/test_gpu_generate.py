@@ -38,19 +38,30 @@ def test_greedy_generation_matches_plain(folders, which, lengths, new):
     assert llm.runner.manager.num_free_pages() == llm.runner.manager.num_pages()
 
 
-def test_bfloat16_greedy_runs_and_mostly_agrees(folders):
+def test_bfloat16_greedy_picks_a_token_within_rounding_of_the_best(folders):
+    """Every greedily generated bfloat16 token, checked against the plain float32 logits
+    of the sequence so far: it is the best token, or one whose logit lies within twice
+    the replay tests' bfloat16 bound (2e-3 + 2 % of the row's scale) of the best.  With
+    a vocabulary of 331 and logits spread over the row's scale, a systematic error picks
+    tokens far below that."""
     from tokamak_amd import LLM, SamplingParams
+    from replay_util import TOL
 
     folder = folders["C"]
     cfg, w = plain.read_folder(folder)
     prompts = [random_ids(cfg["vocab_size"], n, 70 + i) for i, n in enumerate([12, 50])]
     llm = LLM(folder, dtype="bfloat16", kv_pool_tokens=1024)
-    outs = llm.generate(prompt_token_ids=prompts, sampling_params=SamplingParams(temperature=0.0, max_new_tokens=4, ignore_eos=True))
+    outs = llm.generate(prompt_token_ids=prompts, sampling_params=SamplingParams(temperature=0.0, max_new_tokens=6, ignore_eos=True))
+    bound = TOL["bfloat16"]
+    exact = 0
     for o, p in zip(outs, prompts):
-        # the first token is decided by logits within bf16 distance of the plain ones
-        logits = plain.logits(p, cfg, w)[-1]
-        top = float(logits.max())
-        assert float(logits[o.output_token_ids[0]]) > top - 0.05 * float(logits.abs().max())
+        assert len(o.output_token_ids) == 6
+        for i, token in enumerate(o.output_token_ids):
+            row = plain.logits(p + o.output_token_ids[:i], cfg, w)[-1]
+            slack = 2 * (bound["tol_abs"] + bound["tol_rel_to_scale"] * float(row.abs().max()))
+            assert float(row[token]) >= float(row.max()) - slack, f"token {i} of a {len(p)}-token prompt"
+            exact += int(token == int(row.argmax()))
+    assert exact >= 9          # near-ties aside, the tokens are the plain implementation's
 
 
 def test_stop_rules(folders, tmp_path):
@@ -249,5 +260,44 @@ def test_captured_decode_steps_equal_eager_ones_on_every_replay(folders, dtype):
         assert torch.equal(a, b), f"replay {i} differs from the eager step"
         for row, r in enumerate(list(last)):
             last[r] = int(a[row].argmax())
-    assert sum(g.replays for g in graphed._graphs.values()) == 40
     assert len(graphed._graphs) >= 2     # batch sizes 3, 4 and 3 again; lengths crossing 256
+    # the step that meets a new shape runs eagerly and is recorded; every later one is a replay
+    assert sum(g.replays for g in graphed._graphs.values()) == 40 - len(graphed._graphs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_queued_without_a_host_sync(folders, dtype):
+    """Forced tokens, nothing wanted, no synchronisation between steps: the host packs
+    descriptor N+1 while the copy of descriptor N may still be queued behind the running
+    graph.  Each descriptor must reach the graph it was packed for: the logits after 24
+    such steps equal the eager runner's, and so does every key that was cached."""
+    from tokamak_amd.engine.runner import ModelRunner, StepEntry
+
+    folder = folders["C"]
+    cfg, _ = plain.read_folder(folder)
+    kw = dict(dtype=dtype, page_size=16, kv_pool_tokens=1024, max_requests=4)
+    graphed = ModelRunner.from_folder(folder, use_graphs=True, **kw)
+    eager = ModelRunner.from_folder(folder, use_graphs=False, **kw)
+    prompts = {r: random_ids(cfg["vocab_size"], n, 70 + r) for r, n in enumerate([21, 5, 40])}
+    forced = {r: random_ids(cfg["vocab_size"], 25, 80 + r) for r in prompts}
+    for runner in (graphed, eager):
+        for r, p in prompts.items():
+            runner.step([StepEntry(r, p, [])])
+    # make the device slow to reach the copies: a long eager step of another request first
+    filler = random_ids(cfg["vocab_size"], 600, 99)
+    graphed.step([StepEntry("filler", filler, [])])
+    for i in range(24):
+        graphed.step([StepEntry(r, [forced[r][i]], []) for r in prompts])
+    a = graphed.step([StepEntry(r, [forced[r][24]], [0]) for r in prompts]).clone()
+    for i in range(24):
+        eager.step([StepEntry(r, [forced[r][i]], []) for r in prompts])
+    b = eager.step([StepEntry(r, [forced[r][24]], [0]) for r in prompts])
+    assert torch.equal(a, b)
+    assert sum(g.replays for g in graphed._graphs.values()) >= 20
+    for slot in range(cfg["num_hidden_layers"]):
+        for name in ("k", "v"):
+            ga, ea = graphed.storage.slot(slot).arrays[name], eager.storage.slot(slot).arrays[name]
+            for r in prompts:
+                pages_g = graphed.manager.block_table(r)
+                pages_e = eager.manager.block_table(r)
+                assert torch.equal(ga[pages_g], ea[pages_e])

@@ -68,8 +68,10 @@ def test_rotary_part_tables(dtype):
 
     rot = get_part("position", "rotary_half")(rotary_dim=48, theta=50000.0, dtype=dtype, device=DEV)
     batch = make_batch([(5, 1000, list(range(70))), (1, 0, [70])])
-    cos, sin = rot.prepare(batch)
-    assert rot.prepare(batch)[0] is cos            # once per step, shared by the layers
+    data = rot.prepare(batch)
+    cos, sin = data.cos, data.sin
+    assert data.rotary_dim == 48 and data.score_slopes is None
+    assert rot.prepare(batch) is data              # once per step, shared by the layers
     positions = torch.tensor([1000, 1001, 1002, 1003, 1004, 0])
     want_cos, want_sin = plain.rope_tables(positions, 48, 50000.0)
     torch.testing.assert_close(cos.cpu(), want_cos[:, :24], rtol=1e-5, atol=2e-6)
@@ -81,13 +83,13 @@ def test_rotary_part_tables(dtype):
 def test_attention_part_whole_and_in_portions(dtype, nh, nkv, hd, H, ps):
     """The mixer alone: one request whole, then the same tokens in portions and a
     final single token, against the plain attention block."""
-    from tokamak_amd.config import PartSpec, get_part
+    from tokamak_amd.config import get_part
     from tokamak_amd.engine.storage import SlotStore
 
-    pos = PartSpec.of("rotary_half", rotary_dim=hd, theta=10000.0)
+    rot = get_part("position", "rotary_half")(rotary_dim=hd, theta=10000.0, dtype=dtype, device=DEV)
     mixer = get_part("mixer", "gqa_attention")(
         hidden_size=H, num_heads=nh, num_kv_heads=nkv, head_dim=hd, qk_norm_eps=1e-6,
-        softmax_scale=hd ** -0.5, position=(pos.kind, pos.params), window=None, dtype=dtype, device=DEV)
+        softmax_scale=hd ** -0.5, window=None, dtype=dtype, device=DEV)
     w = {"a.q_proj.weight": rand(nh * hd, H, seed=1, scale=H ** -0.5), "a.k_proj.weight": rand(nkv * hd, H, seed=2, scale=H ** -0.5),
          "a.v_proj.weight": rand(nkv * hd, H, seed=3, scale=H ** -0.5), "a.o_proj.weight": rand(H, nh * hd, seed=4, scale=(nh * hd) ** -0.5),
          "a.q_norm.weight": 1 + 0.2 * rand(hd, seed=5), "a.k_norm.weight": 1 + 0.2 * rand(hd, seed=6)}
@@ -95,7 +97,8 @@ def test_attention_part_whole_and_in_portions(dtype, nh, nkv, hd, H, ps):
     assert set(mixer.expected_tensors("a.")) == set(w)
     mixer.bind("a.", fetcher(w, dtype))
     req = mixer.cache_request()
-    assert req.arrays == ("k", "v") and req.elems_per_token == nkv * hd and req.window is None
+    assert [(n, a.elems_per_token, a.dtype) for n, a in req.arrays] == [("k", nkv * hd, None), ("v", nkv * hd, None)]
+    assert req.window is None and req.bytes_per_token(dtype) == 2 * nkv * hd * (4 if dtype == torch.float32 else 2)
     T = 45
     x = rand(T, H, seed=7).to(dtype)
     s = dict(nh=nh, nkv=nkv, hd=hd, eps=1e-6, theta=10000.0)
@@ -109,7 +112,7 @@ def test_attention_part_whole_and_in_portions(dtype, nh, nkv, hd, H, ps):
         at, outs = 0, []
         for n in cuts:
             batch = make_batch([(n, at, table)])
-            delta = mixer.forward(x[at:at + n].to(DEV), batch, store)
+            delta = mixer.forward(x[at:at + n].to(DEV), batch, store, True, rot.prepare(batch))
             outs.append(delta.sum(0) if delta.dim() == 3 else delta)   # split-K partial sums
             at += n
         torch.testing.assert_close(torch.cat(outs).cpu().float(), want, **TOL[dtype])
@@ -123,8 +126,11 @@ def test_embedding_and_head_parts(dtype):
     emb = get_part("embedding", "token_embedding")(vocab_size=V, dim=H, dtype=dtype, device=DEV)
     table = rand(V, H, seed=1).to(dtype).float()
     emb.bind("e.", fetcher({"e.weight": table}, dtype))
-    ids = torch.tensor([3, 330, 0, 3], dtype=torch.int32, device=DEV)
-    torch.testing.assert_close(emb.forward(ids).cpu(), table[ids.cpu().long()], rtol=0, atol=0)
+    from tokamak_amd.engine.batch import StepSpan, build_batch
+
+    ids = [3, 330, 0, 3]
+    batch = build_batch([StepSpan(request=0, tokens=ids, ctx_len=0, state_slot=0, tables=[[0]])], 1, DEV)
+    torch.testing.assert_close(emb.forward(batch).cpu(), table[torch.tensor(ids)], rtol=0, atol=0)
     head = get_part("head", "linear_head")(vocab_size=V, dim=H, tied=True, dtype=dtype, device=DEV)
     assert head.expected_tensors("h.")["h.weight"].ignored
     head.tie(emb)

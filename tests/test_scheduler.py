@@ -7,13 +7,13 @@ import random
 import pytest
 
 from tokamak_amd.cache import CacheGroupSpec, CacheManager, OutOfPagesError
+from tokamak_amd.engine.request import FinishReason, Request
 from tokamak_amd.engine.scheduler import Scheduler
-from tokamak_amd.engine.sequence import FinishReason, Sequence, SequenceStatus
 from tokamak_amd.sampling.params import SamplingParams
 
 
-def make_seq(seq_id, prompt_len=4, max_new=8):
-    return Sequence(seq_id, [1] * prompt_len, SamplingParams(max_new_tokens=max_new))
+def make_seq(rid, prompt_len=4, max_new=8):
+    return Request.from_prompt(rid, [1] * prompt_len, SamplingParams(max_new_tokens=max_new))
 
 
 def make(num_pages=16, page_size=4, max_batch=4, budget=64, chunk=None):
@@ -24,45 +24,45 @@ def make(num_pages=16, page_size=4, max_batch=4, budget=64, chunk=None):
 def run_step(step, token=0):
     """What the engine does after a step: advance caches, append sampled tokens."""
     for span in step.spans:
-        assert span.start == span.seq.num_cached
-        span.seq.num_cached = span.start + span.length
+        assert span.start == span.request.cached
+        span.request.advance(span.length)
     for span in step.spans:
         if span.samples:
-            span.seq.append_output_token(token)
+            span.request.tokens.append(token)
 
 
 def finish(seq, manager):
-    seq.finish(FinishReason.STOP)
-    manager.free(seq.seq_id)
+    seq.finish_reason = FinishReason.STOP
+    manager.free(seq.rid)
 
 
 def test_admits_in_fcfs_order_and_batches_prompts_under_the_budget():
     sched, _ = make(budget=10)
     seqs = [make_seq(i) for i in range(3)]
     for s in seqs:
-        sched.add(s)
-    step = sched.schedule()
+        sched.submit(s)
+    step = sched.plan()
     # budget 10: two whole prompts of 4 and the first 2 tokens of the third
-    assert [(s.seq.seq_id, s.start, s.length, s.samples) for s in step.spans] == [
+    assert [(s.request.rid, s.start, s.length, s.samples) for s in step.spans] == [
         (0, 0, 4, True), (1, 0, 4, True), (2, 0, 2, False)]
-    assert all(s.status is SequenceStatus.RUNNING for s in seqs)
+    assert sched.running == seqs and not sched.waiting
     run_step(step)
-    step = sched.schedule()
+    step = sched.plan()
     # decodes of the first two come first, then the rest of the third prompt
-    assert [(s.seq.seq_id, s.start, s.length, s.samples) for s in step.spans] == [
+    assert [(s.request.rid, s.start, s.length, s.samples) for s in step.spans] == [
         (0, 4, 1, True), (1, 4, 1, True), (2, 2, 2, True)]
     run_step(step)
-    step = sched.schedule()
-    assert [(s.seq.seq_id, s.length) for s in step.spans] == [(0, 1), (1, 1), (2, 1)]
+    step = sched.plan()
+    assert [(s.request.rid, s.length) for s in step.spans] == [(0, 1), (1, 1), (2, 1)]
 
 
 def test_prompt_is_cut_into_portions_of_prefill_chunk():
     sched, manager = make(num_pages=32, budget=64, chunk=5)
     seq = make_seq(0, prompt_len=12)
-    sched.add(seq)
+    sched.submit(seq)
     cuts = []
-    while seq.num_output_tokens == 0:
-        step = sched.schedule()
+    while seq.num_generated == 0:
+        step = sched.plan()
         cuts.append((step.spans[0].start, step.spans[0].length, step.spans[0].samples))
         run_step(step)
     assert cuts == [(0, 5, False), (5, 5, False), (10, 2, True)]
@@ -74,16 +74,16 @@ def test_admission_respects_max_batch_size():
     sched, manager = make(max_batch=2)
     seqs = [make_seq(i) for i in range(3)]
     for s in seqs:
-        sched.add(s)
-    step = sched.schedule()
-    assert [s.seq.seq_id for s in step.spans] == [0, 1]
+        sched.submit(s)
+    step = sched.plan()
+    assert [s.request.rid for s in step.spans] == [0, 1]
     run_step(step)
-    step = sched.schedule()
-    assert [s.seq.seq_id for s in step.spans] == [0, 1]      # batch full: third waits
+    step = sched.plan()
+    assert [s.request.rid for s in step.spans] == [0, 1]      # batch full: third waits
     run_step(step)
     finish(seqs[0], manager)
-    step = sched.schedule()
-    assert [(s.seq.seq_id, s.length) for s in step.spans] == [(1, 1), (2, 4)]
+    step = sched.plan()
+    assert [(s.request.rid, s.length) for s in step.spans] == [(1, 1), (2, 4)]
 
 
 def test_no_bypass_of_the_head_of_the_queue():
@@ -91,25 +91,25 @@ def test_no_bypass_of_the_head_of_the_queue():
     sched, manager = make(num_pages=4)
     first, second, third = make_seq(0, 12), make_seq(1, 8), make_seq(2, 3)
     for s in (first, second, third):
-        sched.add(s)
-    step = sched.schedule()
-    assert [s.seq.seq_id for s in step.spans] == [0]
+        sched.submit(s)
+    step = sched.plan()
+    assert [s.request.rid for s in step.spans] == [0]
     run_step(step)
-    step = sched.schedule()
-    assert [s.seq.seq_id for s in step.spans] == [0]
+    step = sched.plan()
+    assert [s.request.rid for s in step.spans] == [0]
     run_step(step)
     finish(first, manager)
-    step = sched.schedule()
-    assert [s.seq.seq_id for s in step.spans] == [1, 2]
+    step = sched.plan()
+    assert [s.request.rid for s in step.spans] == [1, 2]
 
 
 def test_decode_reserves_the_next_tokens_page():
     sched, manager = make(num_pages=8)
     seq = make_seq(0, 4)
-    sched.add(seq)
-    run_step(sched.schedule())
+    sched.submit(seq)
+    run_step(sched.plan())
     assert manager.reserved_tokens(0) == 4
-    sched.schedule()                       # token 5 needs a second page
+    sched.plan()                       # token 5 needs a second page
     assert manager.reserved_tokens(0) == 8
 
 
@@ -117,51 +117,51 @@ def test_pages_run_out_newest_is_preempted_and_requeued_at_the_front():
     sched, manager = make(num_pages=4, max_batch=4)
     old, new = make_seq(0, 8, 16), make_seq(1, 8, 16)
     late = make_seq(2, 4, 4)
-    sched.add(old)
-    sched.add(new)
-    run_step(sched.schedule())             # both prompts, pool now full
-    sched.add(late)
-    step = sched.schedule()                # both need a third page: none free
-    assert [s.seq.seq_id for s in step.spans] == [0]
-    assert step.preempted == [new]
-    assert new.status is SequenceStatus.WAITING and new.num_cached == 0
+    sched.submit(old)
+    sched.submit(new)
+    run_step(sched.plan())             # both prompts, pool now full
+    sched.submit(late)
+    step = sched.plan()                # both need a third page: none free
+    assert [s.request.rid for s in step.spans] == [0]
+    assert step.evicted == [new]
+    assert new not in sched.running and new.cached == 0 and new.evictions == 1
     assert sched.waiting[0] is new and sched.waiting[1] is late   # front, ahead of later arrivals
     assert manager.block_table(1) == []
     run_step(step)
     finish(old, manager)
-    step = sched.schedule()
+    step = sched.plan()
     # the victim resumes over prompt + its generated token, and samples at its end
-    assert (step.spans[0].seq, step.spans[0].start, step.spans[0].length, step.spans[0].samples) == (new, 0, 9, True)
-    assert new.num_tokens == 9
+    assert (step.spans[0].request, step.spans[0].start, step.spans[0].length, step.spans[0].samples) == (new, 0, 9, True)
+    assert len(new.tokens) == 9
 
 
 def test_a_sequence_that_starves_alone_preempts_itself_and_resumes():
     # one page short for the newest: it is its own victim and comes back once there is room
     sched, manager = make(num_pages=3, max_batch=2)
     a, b = make_seq(0, 4, 16), make_seq(1, 8, 16)
-    sched.add(a)
-    sched.add(b)
-    run_step(sched.schedule())              # a: 1 page, b: 2 pages
-    step = sched.schedule()                 # a needs a 2nd page -> b (newest) is evicted
-    assert step.preempted == [b] and [s.seq.seq_id for s in step.spans] == [0]
+    sched.submit(a)
+    sched.submit(b)
+    run_step(sched.plan())              # a: 1 page, b: 2 pages
+    step = sched.plan()                 # a needs a 2nd page -> b (newest) is evicted
+    assert step.evicted == [b] and [s.request.rid for s in step.spans] == [0]
     manager.check()
 
 
 def test_impossible_prompt_raises():
     sched, _ = make(num_pages=2)
-    sched.add(make_seq(0, 12))
+    sched.submit(make_seq(0, 12))
     with pytest.raises(OutOfPagesError, match="pool can ever provide"):
-        sched.schedule()
+        sched.plan()
 
 
 def test_all_finished_returns_none():
     sched, manager = make()
     seq = make_seq(0)
-    sched.add(seq)
-    run_step(sched.schedule())
+    sched.submit(seq)
+    run_step(sched.plan())
     finish(seq, manager)
-    assert not sched.has_unfinished()
-    assert sched.schedule() is None
+    assert not sched.busy
+    assert sched.plan() is None
 
 
 def test_budget_must_cover_the_batch():
@@ -172,11 +172,11 @@ def test_budget_must_cover_the_batch():
 def test_one_token_prompt_is_a_portion_then_decodes():
     sched, _ = make()
     seq = make_seq(0, 1)
-    sched.add(seq)
-    step = sched.schedule()
+    sched.submit(seq)
+    step = sched.plan()
     assert (step.spans[0].start, step.spans[0].length, step.spans[0].samples) == (0, 1, True)
     run_step(step)
-    step = sched.schedule()
+    step = sched.plan()
     assert (step.spans[0].start, step.spans[0].length) == (1, 1)
 
 
@@ -186,25 +186,25 @@ def test_random_workloads_finish_with_every_page_back(seed):
     sched, manager = make(num_pages=12, page_size=4, max_batch=3, budget=16, chunk=7)
     seqs = [make_seq(i, rng.randint(1, 30), rng.randint(1, 12)) for i in range(12)]
     for s in seqs:
-        sched.add(s)
+        sched.submit(s)
     steps = 0
-    while sched.has_unfinished():
-        step = sched.schedule()
+    while sched.busy:
+        step = sched.plan()
         assert step is not None and step.spans
         assert step.num_tokens <= 16 and len(step.spans) <= 3
-        ids = [s.seq.seq_id for s in step.spans]
+        ids = [s.request.rid for s in step.spans]
         assert len(set(ids)) == len(ids)
         for span in step.spans:
             # the pages for the span are there before it runs
-            assert len(manager.block_table(span.seq.seq_id)) * 4 >= span.start + span.length
+            assert len(manager.block_table(span.request.rid)) * 4 >= span.start + span.length
         run_step(step)
         for span in step.spans:
-            seq = span.seq
-            if span.samples and (seq.num_output_tokens >= seq.sampling_params.max_new_tokens
-                                 or seq.num_tokens >= 48):
+            seq = span.request
+            if span.samples and (seq.num_generated >= seq.params.max_new_tokens
+                                 or len(seq.tokens) >= 48):
                 finish(seq, manager)
         manager.check()
         steps += 1
         assert steps < 2000
-    assert all(s.is_finished for s in seqs)
+    assert all(s.finished for s in seqs)
     assert manager.num_free_pages() == 12 and manager.slots.num_free == 3

@@ -118,6 +118,14 @@ class GroupTables:
             self.first_live[request] = hi
         return hi - lo
 
+    def releasable_before(self, request, first_needed_position: int) -> int:
+        """How many pages ``release_before`` would give back now."""
+        table = self.tables.get(request)
+        if table is None:
+            return 0
+        lo = self.first_live.get(request, 0)
+        return min(max(first_needed_position // self.page_size, lo), len(table)) - lo
+
     def free(self, request) -> None:
         table = self.tables.pop(request, None)
         self.first_live.pop(request, None)

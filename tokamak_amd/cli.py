@@ -5,7 +5,8 @@
 
 Options ``--model --prompt --max-new-tokens --temperature --top-p`` and their
 defaults are those of the reference's example (examples/basic_generation.py:14-20);
-the chat template is applied only when the folder has a tokenizer.
+``--prompt`` needs a tokenizer in the folder and goes through the folder's chat template
+(or the architecture's, if the folder has none); ``--prompt-ids`` needs neither.
 """
 
 from __future__ import annotations
@@ -40,13 +41,14 @@ def main(argv: list[str] | None = None) -> int:
     tmp = None
     folder = args.model
     if args.random_weights is not None:
-        from tokamak_amd.models.qwen3 import PRESETS
+        from tokamak_amd.config import find_preset, preset_names
         from tokamak_amd.weights import write_random_model
 
-        if args.random_weights not in PRESETS:
-            parser.error(f"unknown preset {args.random_weights!r}; presets: {sorted(PRESETS)}")
+        if args.random_weights not in preset_names():
+            parser.error(f"unknown preset {args.random_weights!r}; presets: {preset_names()}")
+        _, config = find_preset(args.random_weights)
         tmp = tempfile.TemporaryDirectory(prefix="tokamak_amd_")
-        folder = write_random_model(tmp.name, PRESETS[args.random_weights], args.weights_seed)
+        folder = write_random_model(tmp.name, config, args.weights_seed)
 
     llm = LLM(folder, dtype=args.dtype, block_size=args.page_size, max_seq_len=args.max_seq_len)
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k,
@@ -58,8 +60,7 @@ def main(argv: list[str] | None = None) -> int:
     else:
         if llm.tokenizer is None:
             parser.error("the model folder has no tokenizer.json: use --prompt-ids")
-        text = f"<|im_start|>user\n{args.prompt}<|im_end|>\n<|im_start|>assistant\n<think>\n\n</think>\n\n"
-        outputs = llm.generate(text, params)
+        outputs = llm.generate(llm.chat_prompt(args.prompt), params)
         print(f"\n[prompt]\n{args.prompt}\n")
     out = outputs[0]
     print(f"[completion ({out.finish_reason.value})]")

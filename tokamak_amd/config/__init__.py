@@ -5,13 +5,16 @@ from tokamak_amd.config.model_config import (
     LayerSpec,
     ModelPlan,
     PartSpec,
+    SubPart,
     default_order,
 )
 from tokamak_amd.config.registry import (
     Architecture,
     get_architecture,
+    find_preset,
     get_part,
     load_model_description,
+    preset_names,
     read_eos_token_ids,
     register_architecture,
     register_part,
@@ -24,9 +27,12 @@ __all__ = [
     "LayerSpec",
     "ModelPlan",
     "PartSpec",
+    "SubPart",
     "default_order",
     "get_architecture",
+    "find_preset",
     "get_part",
+    "preset_names",
     "load_model_description",
     "read_eos_token_ids",
     "register_architecture",

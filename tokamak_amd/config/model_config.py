@@ -2,9 +2,9 @@
 
 Two layers of description live here:
 
-* ``ModelPlan`` is what the engine runs: which parts make each layer (mixer,
-  feed-forward, norms, block arrangement), in which order layers are called and
-  which cache slot each call uses.  It is pure data; nothing in it names an
+* ``ModelPlan`` is what the engine runs: which parts make each layer (by role:
+  mixer, feed-forward, norms, position encoding ...) and which block arranges
+  them, in which order layers are called and which cache slot each call uses.  It is pure data; nothing in it names an
   architecture.
 * An architecture's own frozen config dataclass (``Qwen3Config`` in
   ``tokamak_amd.models.qwen3``) is parsed from the keys of its ``config.json``
@@ -51,22 +51,43 @@ class PartSpec:
 
 
 @dataclass(frozen=True)
-class LayerSpec:
-    """One layer: two sub-layers (mixer, feed-forward), each behind a norm.
+class SubPart:
+    """One part of a layer: the registry family it is looked up in, its
+    ``PartSpec``, and the sub-prefix of its checkpoint tensors inside the
+    layer's own prefix.  ``shared``: every sub-part of the model with the same
+    family and spec is one object (for parts without tensors whose per-step work,
+    like a position encoding's tables, should be done once for all layers)."""
 
-    ``block`` names the arrangement (residual topology) that puts them together.
+    family: str
+    spec: PartSpec
+    prefix: str = ""
+    shared: bool = False
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One layer: parts by role, and the block that arranges them.
+
+    ``parts`` maps a role name to a ``SubPart``; which roles exist is between the
+    architecture's plan and the block it names (``block.kind``): the pre-norm block
+    asks for ``mixer_norm``, ``mixer``, ``feed_forward_norm``, ``feed_forward`` and
+    takes an optional ``position``; a block with four norms, with one norm feeding
+    two branches, or with no feed-forward simply names other roles.  Nothing else
+    in the engine knows the role names.
     """
 
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: tuple[tuple[str, SubPart], ...]
     block: PartSpec = field(default_factory=lambda: PartSpec.of("pre_norm"))
-    # checkpoint sub-prefix of each part inside the layer's own prefix
-    mixer_prefix: str = "self_attn."
-    feed_forward_prefix: str = "mlp."
-    mixer_norm_prefix: str = "input_layernorm."
-    feed_forward_norm_prefix: str = "post_attention_layernorm."
+
+    @classmethod
+    def of(cls, block: PartSpec | None = None, **roles: SubPart) -> LayerSpec:
+        return cls(tuple(roles.items()), block if block is not None else PartSpec.of("pre_norm"))
+
+    def role(self, name: str) -> SubPart:
+        for role, part in self.parts:
+            if role == name:
+                return part
+        raise KeyError(name)
 
 
 @dataclass(frozen=True)
@@ -98,12 +119,12 @@ class ModelPlan:
     order: tuple[LayerCall, ...]
     final_norm: PartSpec
     head: PartSpec
-    eos_token_ids: tuple[int, ...] = ()
     # checkpoint names; ``layer_prefix`` is formatted with the layer index
-    embedding_prefix: str = "model.embed_tokens."
-    layer_prefix: str = "model.layers.{}."
-    final_norm_prefix: str = "model.norm."
-    head_prefix: str = "lm_head."
+    embedding_prefix: str
+    layer_prefix: str
+    final_norm_prefix: str
+    head_prefix: str
+    eos_token_ids: tuple[int, ...] = ()
 
     def __post_init__(self) -> None:
         for call in self.order:

@@ -6,6 +6,10 @@ Such a step is recorded once into a HIP graph and replayed: one launch instead
 of several hundred.  The graph reads its descriptor from a static device
 buffer that is refilled (one host-to-device copy) before every replay; nothing
 in it allocates, clears memory or calls a library.
+
+The step that meets a new shape runs eagerly, once, and is recorded afterwards
+without being executed again: a part that advances per-request state sees every
+token exactly once, whether its step was the recorded one or a replay.
 """
 
 from __future__ import annotations
@@ -23,27 +27,43 @@ def pow2_at_least(n: int, floor: int) -> int:
 
 
 class DecodeGraph:
+    """One recorded decode shape.
+
+    The descriptor travels through two pinned host buffers used in turn, each
+    with an event that marks the end of its last copy: a caller may queue
+    several replays without synchronising, and the host never rewrites a buffer
+    whose copy has not run yet.
+    """
+
     def __init__(self, model, storage, packed: PackedBatch, device) -> None:
         self.size = int(packed.buf.size)
-        self.host = torch.empty(self.size, dtype=torch.int32, pin_memory=True)
+        self._host = [torch.empty(self.size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._copied = [torch.cuda.Event(), torch.cuda.Event()]
+        self._turn = 0
         self.dev = torch.empty(self.size, dtype=torch.int32, device=device)
         self.batch = batch_from_device(packed, self.dev)
+        before = torch.cuda.memory_allocated(device)
         self._load(packed)
-        # run once outside the graph: code objects are loaded and buffers exist
-        # before the capture starts (what it writes, the replay writes again)
-        model.forward(self.batch, storage)
+        # this step itself, eagerly: code objects are loaded and the allocator is warm
+        # before the recording starts; the recording executes nothing
+        self.first_logits = model.forward(self.batch, storage)
         torch.cuda.synchronize(device)
         self.batch.memo.clear()
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
             self.logits = model.forward(self.batch, storage)
+        self.bytes = max(0, torch.cuda.memory_allocated(device) - before)
         self.replays = 0
 
     def _load(self, packed: PackedBatch) -> None:
         if packed.buf.size != self.size:
             raise ValueError("descriptor does not have the shape this graph was captured for")
-        self.host.numpy()[:] = packed.buf
-        self.dev.copy_(self.host, non_blocking=True)
+        turn = self._turn
+        self._turn = 1 - turn
+        self._copied[turn].synchronize()       # the copy that last read this buffer has run
+        self._host[turn].numpy()[:] = packed.buf
+        self.dev.copy_(self._host[turn], non_blocking=True)
+        self._copied[turn].record()
 
     def run(self, packed: PackedBatch) -> torch.Tensor:
         """Replay with a new descriptor; the returned logits live in the graph's

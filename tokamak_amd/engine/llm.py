@@ -7,6 +7,7 @@ load once, then ``generate`` runs a scheduler-driven step loop and returns one
 
 from __future__ import annotations
 
+import json
 import random
 import time
 from collections.abc import Sequence as AbcSequence
@@ -17,8 +18,9 @@ import torch
 from tokamak_amd.config.registry import get_architecture, load_model_description
 from tokamak_amd.engine.outputs import RequestOutput
 from tokamak_amd.engine.runner import ModelRunner, StepEntry, resolve_dtype
-from tokamak_amd.engine.scheduler import ScheduledStep, Scheduler
-from tokamak_amd.engine.sequence import Sequence
+from tokamak_amd.kernels import ops
+from tokamak_amd.engine.request import Request
+from tokamak_amd.engine.scheduler import Scheduler, StepPlan
 from tokamak_amd.sampling.params import SamplingParams
 from tokamak_amd.sampling.sampler import sample_tokens
 from tokamak_amd.weights.random_init import expected_tensors_of
@@ -44,6 +46,10 @@ class LLM:
             would serve one long request at a time).
         max_batch_size: most sequences running at once.
         max_num_batched_tokens: token budget of one step (new).
+        tune_library_products: time the library's candidate algorithms for each new
+            shape of a long portion's matrix products and keep the fastest (new; off by
+            default: the library's first choice is taken, so that two runs of the same
+            input compute the same bits).
         prefill_chunk: longest prompt portion in one step (new; default the budget).
         device: ``"auto"`` or a cuda device; there is no CPU path.
         kv_backend, scheduling, attention_backend, attention_policy, draft_model: the
@@ -62,7 +68,7 @@ class LLM:
                  device: str | torch.device = "auto", kv_backend: str = "paged",
                  scheduling: str = "continuous", attention_backend: str = "auto",
                  attention_policy: str = "full", draft_model=None, seed: int = 0,
-                 random_weights_on_gpu: bool = False) -> None:
+                 random_weights_on_gpu: bool = False, tune_library_products: bool = False) -> None:
         given = {"kv_backend": kv_backend, "scheduling": scheduling, "attention_backend": attention_backend,
                  "attention_policy": attention_policy, "draft_model": draft_model}
         for name, value in given.items():
@@ -106,12 +112,15 @@ class LLM:
         self.max_num_batched_tokens = max(max_num_batched_tokens, max_batch_size)
         self.prefill_chunk = prefill_chunk
         self.eos_token_ids = tuple(plan.eos_token_ids)
+        ops.set_library_tuning(tune_library_products)
         self.runner = ModelRunner(plan, source, dtype=self.dtype,
                                   page_size=block_size, kv_pool_tokens=kv_pool_tokens,
                                   max_requests=max_batch_size, device=device,
-                                  min_pool_tokens=self.max_seq_len, tokens_per_request=self.max_seq_len)
+                                  min_pool_tokens=self.max_seq_len, tokens_per_request=self.max_seq_len,
+                                  max_step_tokens=self.max_num_batched_tokens)
         if self.runner.kv_pool_tokens < self.max_seq_len:
             raise RuntimeError(f"the GPU has no room for a cache of max_seq_len ({self.max_seq_len}) tokens")
+        self.folder = folder
         self.tokenizer = self._load_tokenizer(folder) if folder is not None else None
         self.num_steps = 0
         self.num_preemptions = 0
@@ -127,139 +136,146 @@ class LLM:
             return None
         return Tokenizer.from_file(str(path))
 
+    def chat_prompt(self, user_text: str) -> str:
+        """``user_text`` as a single user turn, ready to tokenize.  The folder's own
+        chat template (``tokenizer_config.json``, rendered in a sandbox with
+        ``enable_thinking=False`` as the reference's example asks,
+        examples/basic_generation.py:25-30) when it has one; else the architecture's."""
+        template = None
+        if self.folder is not None and (self.folder / "tokenizer_config.json").is_file():
+            template = json.loads((self.folder / "tokenizer_config.json").read_text()).get("chat_template")
+        if isinstance(template, str):
+            from jinja2.sandbox import ImmutableSandboxedEnvironment
+
+            env = ImmutableSandboxedEnvironment(trim_blocks=True, lstrip_blocks=True)
+            return env.from_string(template).render(
+                messages=[{"role": "user", "content": user_text}], add_generation_prompt=True,
+                enable_thinking=False)
+        if self.architecture.chat_prompt is not None:
+            return self.architecture.chat_prompt(user_text)
+        return user_text
+
     # ------------------------------------------------------------------
     def generate(self, prompts: str | AbcSequence[str] | None = None,
                  sampling_params: SamplingParams | AbcSequence[SamplingParams] | None = None, *,
                  prompt_token_ids: AbcSequence[AbcSequence[int]] | None = None,
                  use_tqdm: bool = False) -> list[RequestOutput]:
         """One completion per prompt, in input order
-        (reference: src/tokamak/engine/llm.py:265-334)."""
-        texts, token_lists = self._resolve_prompts(prompts, prompt_token_ids)
-        params_list = self._broadcast_params(sampling_params, len(token_lists))
-        arrival = time.perf_counter()
-        sequences = []
-        for i, (ids, params) in enumerate(zip(token_lists, params_list)):
-            seq = Sequence(i, list(ids), params)
-            seq.arrival_time = arrival
-            seq.seed = params.seed if params.seed is not None else random.getrandbits(62)
-            self._validate_fits(seq)
-            sequences.append(seq)
-
-        manager = self.runner.manager
-        scheduler = Scheduler(manager, self.max_batch_size, self.max_num_batched_tokens, self.prefill_chunk)
-        for seq in sequences:
-            scheduler.add(seq)
-        try:
-            while scheduler.has_unfinished():
-                step = scheduler.schedule()
-                if step is None:
-                    raise RuntimeError("scheduler returned no work but is unfinished")
-                self._run(step)
-        finally:
-            self.runner.end_all()
-        return [self._to_output(seq, texts[seq.seq_id] if texts else None) for seq in sequences]
-
-    def _run(self, step: ScheduledStep) -> None:
-        for victim in step.preempted:
-            self.runner.forget(victim.seq_id)  # the scheduler has already freed its pages
-            self.num_preemptions += 1
-        entries = []
-        sampling = []
-        for span in step.spans:
-            seq = span.seq
-            if span.start != self.runner.cached_tokens(seq.seq_id):
-                raise RuntimeError(f"sequence {seq.seq_id}: span starts at {span.start}, cache holds "
-                                   f"{self.runner.cached_tokens(seq.seq_id)}")
-            tokens = seq.tokens_between(span.start, span.start + span.length)
-            entries.append(StepEntry(seq.seq_id, tokens, [span.length - 1] if span.samples else []))
-            if span.samples:
-                sampling.append(seq)
-        logits = self.runner.step(entries)
-        self.num_steps += 1
-        for span in step.spans:
-            span.seq.num_cached = span.start + span.length
-        if not sampling:
-            return
-        chosen = sample_tokens(logits, [s.sampling_params for s in sampling],
-                               [s.seed for s in sampling], [s.num_output_tokens for s in sampling])
-        now = None
-        for seq, token in zip(sampling, chosen.tolist()):
-            finished = seq.append_checked(token, eos_token_ids=self.eos_token_ids,
-                                          max_total_tokens=self._max_total_tokens(seq))
-            if seq.first_token_time is None:
-                now = now or time.perf_counter()
-                seq.first_token_time = now
-            if finished:
-                seq.finish_time = time.perf_counter()
-                self.runner.end(seq.seq_id)
-
-    # ------------------------------------------------------------------
-    def _max_total_tokens(self, seq: Sequence) -> int:
-        """reference: src/tokamak/engine/llm.py:483-485"""
-        return min(self.max_seq_len, seq.num_prompt_tokens + seq.sampling_params.max_new_tokens)
-
-    def _validate_fits(self, seq: Sequence) -> None:
-        """reference: src/tokamak/engine/llm.py:487-499"""
-        if seq.num_prompt_tokens >= self.max_seq_len:
-            raise ValueError(
-                f"Prompt of {seq.num_prompt_tokens} tokens does not fit in "
-                f"max_seq_len={self.max_seq_len} (room for generation is required)")
-        vocab = self.runner.plan.vocab_size
-        if min(seq.prompt_token_ids) < 0 or max(seq.prompt_token_ids) >= vocab:
-            raise ValueError(f"prompt {seq.seq_id} has a token id outside [0, {vocab})")
-        manager = self.runner.manager
-        needed = manager.pages_needed(self._max_total_tokens(seq))
-        for g in range(len(manager.groups)):
-            if needed > manager.num_pages(g):
-                raise ValueError(
-                    f"Request needs {needed} cache pages but the pool has {manager.num_pages(g)}; "
-                    f"raise kv_pool_tokens")
-
-    def _resolve_prompts(self, prompts, prompt_token_ids):
+        (interface of reference: src/tokamak/engine/llm.py:265-334)."""
         if (prompts is None) == (prompt_token_ids is None):
             raise ValueError("provide exactly one of `prompts` or `prompt_token_ids`")
+        texts: list[str | None]
         if prompt_token_ids is not None:
-            return None, [list(ids) for ids in prompt_token_ids]
-        if isinstance(prompts, str):
-            prompts = [prompts]
-        texts = list(prompts)
-        if self.tokenizer is None:
-            raise ValueError("the model folder has no tokenizer.json: pass prompt_token_ids")
-        return texts, [self.tokenizer.encode(t).ids for t in texts]
+            id_lists = [list(ids) for ids in prompt_token_ids]
+            texts = [None] * len(id_lists)
+        else:
+            if self.tokenizer is None:
+                raise ValueError("the model folder has no tokenizer.json: pass prompt_token_ids")
+            texts = [prompts] if isinstance(prompts, str) else list(prompts)
+            id_lists = [self.tokenizer.encode(t).ids for t in texts]
+        if sampling_params is None or isinstance(sampling_params, SamplingParams):
+            per_request = [sampling_params or SamplingParams()] * len(id_lists)
+        else:
+            per_request = list(sampling_params)
+            if len(per_request) != len(id_lists):
+                raise ValueError(f"Got {len(per_request)} SamplingParams for {len(id_lists)} prompts")
 
-    def _decode(self, ids: list[int]) -> str | None:
-        if self.tokenizer is None:
-            return None
-        return self.tokenizer.decode(ids, skip_special_tokens=True)
+        now = time.perf_counter()
+        requests = []
+        for rid, (ids, params) in enumerate(zip(id_lists, per_request)):
+            seed = params.seed if params.seed is not None else random.getrandbits(62)
+            request = Request.from_prompt(rid, ids, params, seed)
+            request.arrived_at = now
+            self._check_request(request)
+            requests.append(request)
 
-    def _to_output(self, seq: Sequence, prompt_text: str | None) -> RequestOutput:
-        if seq.finish_reason is None:
-            raise RuntimeError(f"Sequence {seq.seq_id} completed without a finish reason")
-        ttft = latency = None
-        if seq.arrival_time is not None:
-            if seq.first_token_time is not None:
-                ttft = seq.first_token_time - seq.arrival_time
-            if seq.finish_time is not None:
-                latency = seq.finish_time - seq.arrival_time
+        scheduler = Scheduler(self.runner.manager, self.max_batch_size, self.max_num_batched_tokens,
+                              self.prefill_chunk)
+        for request in requests:
+            scheduler.submit(request)
+        try:
+            while scheduler.busy:
+                plan = scheduler.plan()
+                if plan is None:
+                    raise RuntimeError("the scheduler has unfinished requests but plans no step")
+                self._run(plan)
+        finally:
+            # also what the scheduler reserved for requests that never reached a step
+            self.runner.end_all()
+            for request in scheduler.live_requests():
+                self.runner.manager.free(request.rid)
+        return [self._output(request, text) for request, text in zip(requests, texts)]
+
+    def _run(self, plan: StepPlan) -> None:
+        for victim in plan.evicted:
+            self.runner.forget(victim.rid)      # the scheduler has already freed its pages
+            self.num_preemptions += 1
+        entries, sampling = [], []
+        for span in plan.spans:
+            request = span.request
+            held = self.runner.cached_tokens(request.rid)
+            if span.start != held or span.start != request.cached:
+                raise RuntimeError(f"request {request.rid}: span starts at {span.start}, the cache holds {held}")
+            entries.append(StepEntry(request.rid, request.span(span.length), [span.length - 1] if span.samples else []))
+            if span.samples:
+                sampling.append(request)
+        logits = self.runner.step(entries)
+        self.num_steps += 1
+        for span in plan.spans:
+            span.request.advance(span.length)
+        if not sampling:
+            return
+        chosen = sample_tokens(logits, [r.params for r in sampling], [r.seed for r in sampling],
+                               [r.num_generated for r in sampling]).tolist()
+        stamp = time.perf_counter()
+        for request, token in zip(sampling, chosen):
+            if request.first_token_at is None:
+                request.first_token_at = stamp
+            if request.accept(token, eos_token_ids=self.eos_token_ids, context_limit=self._context_limit(request)):
+                request.finished_at = stamp
+                self.runner.end(request.rid)
+
+    # ------------------------------------------------------------------
+    def _context_limit(self, request: Request) -> int:
+        """Most tokens the request may ever hold: its prompt plus ``max_new_tokens``,
+        within ``max_seq_len`` (reference: src/tokamak/engine/llm.py:483-485)."""
+        return min(self.max_seq_len, request.prompt_len + request.params.max_new_tokens)
+
+    def _check_request(self, request: Request) -> None:
+        """Refuse at submission what could never finish: a prompt that leaves no room
+        to generate, ids outside the vocabulary, more pages than the pool has
+        (reference: src/tokamak/engine/llm.py:487-499)."""
+        if request.prompt_len >= self.max_seq_len:
+            raise ValueError(f"prompt {request.rid} has {request.prompt_len} tokens and does not fit "
+                             f"max_seq_len={self.max_seq_len}: at least one token must be generated")
+        vocab = self.runner.plan.vocab_size
+        if min(request.tokens) < 0 or max(request.tokens) >= vocab:
+            raise ValueError(f"prompt {request.rid} has a token id outside [0, {vocab})")
+        manager = self.runner.manager
+        pages = manager.pages_needed(self._context_limit(request))
+        smallest = min(manager.num_pages(g) for g in range(len(manager.groups))) if manager.groups else pages
+        if pages > smallest:
+            raise ValueError(f"prompt {request.rid} may grow to {pages} cache pages, the pool has {smallest}: "
+                             f"raise kv_pool_tokens or lower max_new_tokens")
+
+    def _text(self, ids: list[int]) -> str | None:
+        return None if self.tokenizer is None else self.tokenizer.decode(ids, skip_special_tokens=True)
+
+    def _output(self, request: Request, prompt_text: str | None) -> RequestOutput:
+        if not request.finished:
+            raise RuntimeError(f"request {request.rid} left the step loop unfinished")
+        since = request.arrived_at
+
+        def elapsed(t):
+            return None if t is None or since is None else t - since
+
         return RequestOutput(
-            request_id=seq.seq_id,
-            prompt=prompt_text if prompt_text is not None else self._decode(seq.prompt_token_ids),
-            prompt_token_ids=seq.prompt_token_ids,
-            output_text=self._decode(seq.output_token_ids),
-            output_token_ids=seq.output_token_ids,
-            finish_reason=seq.finish_reason,
-            ttft_s=ttft,
-            latency_s=latency,
+            request_id=request.rid,
+            prompt=prompt_text if prompt_text is not None else self._text(request.prompt),
+            prompt_token_ids=request.prompt,
+            output_text=self._text(request.generated),
+            output_token_ids=request.generated,
+            finish_reason=request.finish_reason,
+            ttft_s=elapsed(request.first_token_at),
+            latency_s=elapsed(request.finished_at),
         )
-
-    @staticmethod
-    def _broadcast_params(sampling_params, num_prompts: int) -> list[SamplingParams]:
-        """reference: src/tokamak/engine/llm.py:544-556"""
-        if sampling_params is None:
-            return [SamplingParams()] * num_prompts
-        if isinstance(sampling_params, SamplingParams):
-            return [sampling_params] * num_prompts
-        params_list = list(sampling_params)
-        if len(params_list) != num_prompts:
-            raise ValueError(f"Got {len(params_list)} SamplingParams for {num_prompts} prompts")
-        return params_list

@@ -9,12 +9,8 @@ import torch
 from tokamak_amd.cache.pages import CacheGroupSpec
 from tokamak_amd.config.model_config import ModelPlan, PartSpec
 from tokamak_amd.config.registry import get_part
-from tokamak_amd.parts.base import Block, CacheRequest
+from tokamak_amd.parts.base import Block, CacheRequest, Part, StateArray
 from tokamak_amd.weights.spec import TensorSpec
-
-
-def _build(family: str, spec: PartSpec, dtype, device):
-    return get_part(family, spec.kind)(**spec.as_dict(), dtype=dtype, device=device)
 
 
 @dataclass
@@ -29,37 +25,43 @@ class LayeredModel:
     """Embedding, layers run in the plan's order, final norm, head.
 
     ``forward`` runs exactly the tokens of the batch against the cache and
-    returns float32 logits at ``batch.logit_rows``.
+    returns float32 logits at ``batch.logit_rows``.  Sub-parts marked ``shared``
+    with equal family and spec (position encodings) are built once, so what they
+    prepare for a step is prepared once.
     """
 
     def __init__(self, plan: ModelPlan, *, dtype: torch.dtype, device: str | torch.device) -> None:
         self.plan = plan
         self.dtype = dtype
         self.device = torch.device(device)
-        self.embedding = _build("embedding", plan.embedding, dtype, device)
+        self._shared: dict[tuple[str, PartSpec], Part] = {}
+        self.embedding = self._build("embedding", plan.embedding)
         self.blocks: list[Block] = []
         for spec in plan.layers:
-            block_cls = get_part("block", spec.block.kind)
-            self.blocks.append(block_cls(
-                _build("mixer", spec.mixer, dtype, device),
-                _build("feed_forward", spec.feed_forward, dtype, device),
-                _build("norm", spec.mixer_norm, dtype, device),
-                _build("norm", spec.feed_forward_norm, dtype, device),
-                **spec.block.as_dict(),
-            ))
-        self.final_norm = _build("norm", plan.final_norm, dtype, device)
-        self.head = _build("head", plan.head, dtype, device)
+            parts = {role: self._build(sub.family, sub.spec, shared=sub.shared) for role, sub in spec.parts}
+            self.blocks.append(get_part("block", spec.block.kind)(parts, **spec.block.as_dict()))
+        self.final_norm = self._build("norm", plan.final_norm)
+        self.head = self._build("head", plan.head)
+
+    def _build(self, family: str, spec: PartSpec, shared: bool = False) -> Part:
+        if shared and (family, spec) in self._shared:
+            return self._shared[(family, spec)]
+        part = get_part(family, spec.kind)(**spec.as_dict(), dtype=self.dtype, device=self.device)
+        if shared:
+            self._shared[(family, spec)] = part
+        return part
+
+    def _all_parts(self):
+        yield self.embedding
+        for block in self.blocks:
+            yield from block.parts.values()
+        yield self.final_norm
+        yield self.head
 
     @property
     def capturable(self) -> bool:
         """Whether a decode step of this model may be recorded into a HIP graph."""
-        parts = [self.embedding, self.final_norm, self.head]
-        for block in self.blocks:
-            parts += [block.mixer, block.feed_forward, block.mixer_norm, block.feed_forward_norm]
-            position = getattr(block.mixer, "position", None)
-            if position is not None:
-                parts.append(position)
-        return all(getattr(p, "capturable", False) for p in parts)
+        return all(getattr(p, "capturable", False) for p in self._all_parts())
 
     # -- weights -------------------------------------------------------------
     def _named_parts(self):
@@ -67,10 +69,8 @@ class LayeredModel:
         yield p.embedding_prefix, self.embedding
         for i, (spec, block) in enumerate(zip(p.layers, self.blocks)):
             base = p.layer_prefix.format(i)
-            yield base + spec.mixer_norm_prefix, block.mixer_norm
-            yield base + spec.mixer_prefix, block.mixer
-            yield base + spec.feed_forward_norm_prefix, block.feed_forward_norm
-            yield base + spec.feed_forward_prefix, block.feed_forward
+            for role, sub in spec.parts:
+                yield base + sub.prefix, block.parts[role]
         yield p.final_norm_prefix, self.final_norm
         yield p.head_prefix, self.head
 
@@ -90,13 +90,17 @@ class LayeredModel:
             self.head.tie(self.embedding)
 
     # -- cache ---------------------------------------------------------------
+    def _mixer_of(self, call):
+        return self.blocks[call.layer].mixer
+
     def cache_layout(self) -> tuple[list[CacheGroupSpec], dict[int, SlotLayout]]:
         """Cache groups (slots that share a retention rule) and each slot's layout."""
         requests: dict[int, CacheRequest] = {}
         for call in self.plan.order:
-            if not call.writes_cache:
+            mixer = self._mixer_of(call)
+            if not call.writes_cache or mixer is None:
                 continue
-            req = self.blocks[call.layer].mixer.cache_request()
+            req = mixer.cache_request()
             if req is None:
                 continue
             if call.cache in requests and requests[call.cache] != req:
@@ -118,18 +122,21 @@ class LayeredModel:
         slots = {s: SlotLayout(windows.index(r.window), r) for s, r in requests.items()}
         return groups, slots
 
-    def state_shapes(self) -> dict[int, tuple[int, ...]]:
-        """Cache slot -> shape of the fixed-size per-request state its mixer keeps."""
-        out: dict[int, tuple[int, ...]] = {}
+    def state_requests(self) -> dict[int, dict[str, StateArray]]:
+        """Cache slot -> arrays of the fixed-size per-request state its mixer keeps."""
+        out: dict[int, dict[str, StateArray]] = {}
         for call in self.plan.order:
-            shape = self.blocks[call.layer].mixer.state_shape()
-            if shape is not None and call.writes_cache:
-                out[call.cache] = tuple(shape)
+            mixer = self._mixer_of(call)
+            if mixer is None or not call.writes_cache:
+                continue
+            request = mixer.state_request()
+            if request:
+                out[call.cache] = dict(request)
         return out
 
     # -- compute -------------------------------------------------------------
     def forward(self, batch, storage) -> torch.Tensor:
-        resid = self.embedding.forward(batch.token_ids)
+        resid = self.embedding.forward(batch)
         pending = None
         for call in self.plan.order:
             pending = self.blocks[call.layer].forward(

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
-from tokamak_amd.engine.sequence import FinishReason
+from tokamak_amd.engine.request import FinishReason
 
 
 @dataclass(frozen=True)

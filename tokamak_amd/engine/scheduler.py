@@ -1,18 +1,18 @@
 """Iteration-level scheduler: admission, prompt portions under a token budget,
-decode, preemption when pages run out.
+decode, eviction when pages run out.
 
 Policy kept from the reference (src/tokamak/engine/scheduler.py:67-188):
-first come first served; no bypass of the head of the waiting queue; when the
-pool cannot cover a running sequence's next tokens the newest arrival is
-preempted by recomputation (pages freed, generated tokens kept, back to the
-*front* of the waiting queue); an impossible prompt raises.
+first come first served; nothing overtakes the head of the waiting queue; when
+the pool cannot cover a running request's next token the newest arrival is
+evicted by recomputation (pages freed, generated tokens kept, back to the
+*front* of the waiting queue); a prompt the pool can never hold raises.
 
 Different from the reference, which runs either one whole prompt or one decode
-token of every running sequence: every step takes one token of each decoding
-sequence first, then fills what is left of ``max_num_batched_tokens`` with
-portions (at most ``prefill_chunk`` tokens) of sequences whose prompt is not
-yet cached, then admits from the waiting queue while slots, budget and pages
-allow.  Pages are reserved per portion.
+token of every running request: every step takes one token of each decoding
+request first, then fills what is left of ``max_num_batched_tokens`` with
+portions (at most ``prefill_chunk`` tokens) of requests whose tokens are not yet
+all cached, then admits from the waiting queue while slots, budget and pages
+allow.  Pages are reserved portion by portion.
 """
 
 from __future__ import annotations
@@ -22,24 +22,24 @@ from dataclasses import dataclass, field
 
 from tokamak_amd.cache.manager import CacheManager
 from tokamak_amd.cache.pages import OutOfPagesError
-from tokamak_amd.engine.sequence import Sequence, SequenceStatus
+from tokamak_amd.engine.request import Request
 
 
 @dataclass
-class ScheduledSpan:
-    """Run ``seq``'s tokens [start, start + length); ``samples`` when the span
-    reaches the sequence's last token, so a next token is drawn from it."""
+class Span:
+    """Run ``request.tokens[start : start + length]``; ``samples``: the span ends
+    at the request's last token, so a next token is drawn from its last row."""
 
-    seq: Sequence
+    request: Request
     start: int
     length: int
     samples: bool
 
 
 @dataclass
-class ScheduledStep:
-    spans: list[ScheduledSpan]
-    preempted: list[Sequence] = field(default_factory=list)
+class StepPlan:
+    spans: list[Span]
+    evicted: list[Request] = field(default_factory=list)
 
     @property
     def num_tokens(self) -> int:
@@ -54,121 +54,112 @@ class Scheduler:
         if max_num_batched_tokens < max_batch_size:
             raise ValueError(
                 f"max_num_batched_tokens ({max_num_batched_tokens}) must be >= max_batch_size "
-                f"({max_batch_size}) so every running sequence can decode in one step")
+                f"({max_batch_size}) so every running request can decode in one step")
         if prefill_chunk is not None and prefill_chunk < 1:
             raise ValueError(f"prefill_chunk must be >= 1, got {prefill_chunk}")
-        self._manager = manager
-        self._max_batch_size = max_batch_size
-        self._budget = max_num_batched_tokens
-        self._chunk = prefill_chunk or max_num_batched_tokens
-        self.waiting: deque[Sequence] = deque()
-        self.running: list[Sequence] = []
+        self.manager = manager
+        self.max_batch_size = max_batch_size
+        self.token_budget = max_num_batched_tokens
+        self.chunk = prefill_chunk or max_num_batched_tokens
+        self.waiting: deque[Request] = deque()
+        self.running: list[Request] = []        # oldest first
 
-    def add(self, seq: Sequence) -> None:
-        seq.status = SequenceStatus.WAITING
-        self.waiting.append(seq)
+    def submit(self, request: Request) -> None:
+        self.waiting.append(request)
 
-    def has_unfinished(self) -> bool:
-        return bool(self.waiting) or any(not s.is_finished for s in self.running)
+    @property
+    def busy(self) -> bool:
+        return bool(self.waiting) or any(not r.finished for r in self.running)
+
+    def live_requests(self) -> list[Request]:
+        """Every request that may hold pages or a slot."""
+        return [*self.running, *self.waiting]
 
     # ------------------------------------------------------------------
-    def schedule(self) -> ScheduledStep | None:
-        """Plan the next step; None when everything is finished."""
-        self.running = [s for s in self.running if not s.is_finished]
-        preempted: list[Sequence] = []
+    def plan(self) -> StepPlan | None:
+        """The next step, or None when nothing is left to do."""
+        self.running = [r for r in self.running if not r.finished]
+        evicted: list[Request] = []
         while True:
-            spans: list[ScheduledSpan] = []
-            budget = self._budget
-            budget = self._schedule_decodes(spans, budget, preempted)
-            budget = self._schedule_portions(spans, budget)
-            self._admit(spans, budget)
+            spans = self._fill(evicted)
             if spans:
-                return ScheduledStep(spans, preempted)
+                return StepPlan(spans, evicted)
             if self.running:
-                # every running sequence waits for pages: make room
-                victim = self.running[-1]
-                self._preempt(victim)
-                preempted.append(victim)
-                continue
-            if self.waiting:
-                head = self.waiting[0]
+                # nobody could move: every running request waits for pages
+                evicted.append(self._evict_newest())
+            elif self.waiting:
                 raise OutOfPagesError(
-                    f"sequence {head.seq_id} needs more pages than the pool can ever provide")
-            return None
+                    f"request {self.waiting[0].rid} needs more pages than the pool can ever provide")
+            else:
+                return None
 
-    # ------------------------------------------------------------------
-    def _schedule_decodes(self, spans, budget, preempted) -> int:
-        for seq in list(self.running):
-            if seq not in self.running or seq.num_uncached != 1 or seq.num_cached == 0:
-                continue
-            while True:
-                try:
-                    self._manager.ensure_capacity(seq.seq_id, seq.num_tokens)
-                    spans.append(ScheduledSpan(seq, seq.num_cached, 1, True))
-                    budget -= 1
-                    break
-                except OutOfPagesError:
-                    victim = self.running[-1]  # newest arrival = lowest priority
-                    self._preempt(victim)
-                    preempted.append(victim)
-                    spans[:] = [s for s in spans if s.seq is not victim]
-                    if victim is seq:
-                        break
-        return budget
-
-    def _portion(self, seq: Sequence, budget: int) -> int:
-        """Largest portion of ``seq`` that budget, chunk size and free pages allow."""
-        want = min(seq.num_uncached, self._chunk, budget)
-        if want <= 0:
-            return 0
-        ps = self._manager.page_size
-        have = len(self._manager.block_table(seq.seq_id)) * ps
-        room = have + min(self._manager.num_free_pages(g) for g in range(len(self._manager.groups))) * ps
-        return max(0, min(want, room - seq.num_cached))
-
-    def _schedule_portions(self, spans, budget) -> int:
-        for seq in self.running:
-            if budget <= 0:
+    def _fill(self, evicted: list[Request]) -> list[Span]:
+        spans: list[Span] = []
+        left = self.token_budget
+        # 1. a token for every decoding request, oldest first.  When the pool cannot give
+        # one its page the newest running request makes room; walking from the old end and
+        # evicting from the new end, a victim never has a span in this step yet.
+        at = 0
+        while at < len(self.running):
+            request = self.running[at]
+            if not request.decoding:
+                at += 1
+            elif self._reserve(request, 1):
+                spans.append(Span(request, request.cached, 1, True))
+                left -= 1
+                at += 1
+            else:
+                evicted.append(self._evict_newest())     # may be ``request`` itself
+        # 2. portions of running requests whose tokens are not all cached yet
+        for request in self.running:
+            if left <= 0:
                 break
-            if seq.num_uncached <= 1 and seq.num_cached > 0:
-                continue  # decoding; handled above
-            if any(s.seq is seq for s in spans):
+            if request.decoding:
                 continue
-            length = self._portion(seq, budget)
-            if length <= 0:
-                continue
-            self._manager.ensure_capacity(seq.seq_id, seq.num_cached + length)
-            spans.append(ScheduledSpan(seq, seq.num_cached, length,
-                                       seq.num_cached + length == seq.num_tokens))
-            budget -= length
-        return budget
-
-    def _admit(self, spans, budget) -> int:
-        while self.waiting and len(self.running) < self._max_batch_size and budget > 0:
+            length = self._affordable(request, left)
+            if length > 0 and self._reserve(request, length):
+                spans.append(Span(request, request.cached, length, length == request.pending))
+                left -= length
+        # 3. newcomers, in arrival order, never past a head that does not fit
+        while self.waiting and left > 0 and len(self.running) < self.max_batch_size:
             head = self.waiting[0]
-            # admit only when the pool could hold everything the sequence has so far
-            # (reference: scheduler.py:144-148), but reserve only the first portion
-            if not self._manager.can_hold(head.seq_id, head.num_tokens):
+            # the pool must be able to hold all the request has so far (reference:
+            # scheduler.py:144-148); only its first portion is reserved
+            if not self.manager.can_hold(head.rid, len(head.tokens)):
                 break
-            if self._manager.slots.num_free == 0 and self._manager.slots.slot_of(head.seq_id) is None:
+            if self.manager.slots.num_free == 0 and self.manager.slots.slot_of(head.rid) is None:
                 break
-            length = self._portion(head, budget)
+            length = self._affordable(head, left)
             if length <= 0:
                 break
             self.waiting.popleft()
-            self._manager.admit(head.seq_id)
-            self._manager.ensure_capacity(head.seq_id, length)
-            head.status = SequenceStatus.RUNNING
-            head.num_cached = 0
+            self.manager.admit(head.rid)
+            self.manager.ensure_capacity(head.rid, length)
             self.running.append(head)
-            spans.append(ScheduledSpan(head, 0, length, length == head.num_tokens))
-            budget -= length
-        return budget
+            spans.append(Span(head, 0, length, length == head.pending))
+            left -= length
+        return spans
 
-    def _preempt(self, victim: Sequence) -> None:
-        """Evict by recomputation: free pages and slot, requeue at the front."""
-        self._manager.free(victim.seq_id)
-        self.running.remove(victim)
-        victim.status = SequenceStatus.WAITING
-        victim.num_cached = 0
+    def _reserve(self, request: Request, length: int) -> bool:
+        try:
+            self.manager.ensure_capacity(request.rid, request.cached + length)
+        except OutOfPagesError:
+            return False
+        return True
+
+    def _affordable(self, request: Request, left: int) -> int:
+        """Longest next portion of ``request`` within budget, chunk and free pages."""
+        manager = self.manager
+        page = manager.page_size
+        reserved = len(manager.block_table(request.rid)) * page
+        free = min(manager.num_free_pages(g) for g in range(len(manager.groups))) * page
+        return max(0, min(request.pending, self.chunk, left, reserved + free - request.cached))
+
+    def _evict_newest(self) -> Request:
+        """Free the newest running request's pages and slot; it keeps its tokens and
+        goes to the front of the queue (it is older than anything waiting)."""
+        victim = self.running.pop()
+        self.manager.free(victim.rid)
+        victim.rewind()
         self.waiting.appendleft(victim)
+        return victim

@@ -10,14 +10,15 @@ import torch
 @dataclass
 class SlotStore:
     """What one mixer call sees: the paged arrays of its cache slot
-    (``arrays[name]`` is [num_pages, elems_per_token * page_size]), its group's
-    index into ``batch.block_tables``, and its per-request state
-    ([num_state_slots, *shape]) if it keeps any."""
+    (``arrays[name]`` is [num_pages, elems_per_token * page_size], each with the
+    width and dtype its mixer asked for), its group's index into
+    ``batch.block_tables``, and its per-request state arrays
+    (``state[name]`` is [num_state_slots, *shape]) if it keeps any."""
 
     group: int = 0
     page_size: int = 0
     arrays: dict[str, torch.Tensor] = field(default_factory=dict)
-    state: torch.Tensor | None = None
+    state: dict[str, torch.Tensor] = field(default_factory=dict)
 
 
 class CacheStorage:
@@ -27,15 +28,16 @@ class CacheStorage:
         self.page_size = page_size
         self._slots: dict[int, SlotStore] = {}
         for slot, layout in layouts.items():
-            elems = layout.request.elems_per_token * page_size
             arrays = {
-                name: torch.zeros((pages_per_group[layout.group], elems), dtype=dtype, device=device)
-                for name in layout.request.arrays
+                name: torch.zeros((pages_per_group[layout.group], array.elems_per_token * page_size),
+                                  dtype=array.dtype or dtype, device=device)
+                for name, array in layout.request.arrays
             }
             self._slots[slot] = SlotStore(layout.group, page_size, arrays)
-        for slot, shape in model.state_shapes().items():
+        for slot, request in model.state_requests().items():
             store = self._slots.setdefault(slot, SlotStore(0, page_size))
-            store.state = torch.zeros((num_state_slots, *shape), dtype=torch.float32, device=device)
+            store.state = {name: torch.zeros((num_state_slots, *array.shape), dtype=array.dtype, device=device)
+                           for name, array in request.items()}
         self._empty = SlotStore(0, page_size)
 
     def slot(self, index: int) -> SlotStore:
@@ -44,14 +46,12 @@ class CacheStorage:
     def reset_state(self, state_slot: int) -> None:
         """Zero the fixed-size state of one request slot (on admission)."""
         for store in self._slots.values():
-            if store.state is not None:
-                store.state[state_slot].zero_()
+            for array in store.state.values():
+                array[state_slot].zero_()
 
     def bytes(self) -> int:
         total = 0
         for store in self._slots.values():
-            for t in store.arrays.values():
+            for t in (*store.arrays.values(), *store.state.values()):
                 total += t.numel() * t.element_size()
-            if store.state is not None:
-                total += store.state.numel() * 4
         return total

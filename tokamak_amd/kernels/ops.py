@@ -197,13 +197,14 @@ def rope_tables(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tens
 
 
 def qknorm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor | None,
-                      k_weight: torch.Tensor | None, cos: torch.Tensor, sin: torch.Tensor,
+                      k_weight: torch.Tensor | None, cos: torch.Tensor | None, sin: torch.Tensor | None,
                       positions: torch.Tensor, req_of_token: torch.Tensor,
                       block_tables: torch.Tensor, q_out: torch.Tensor,
                       k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, *, num_heads: int,
                       num_kv_heads: int, head_dim: int, rotary_dim: int, page_size: int, eps: float,
                       store: bool = True) -> None:
-    """Per-head norm + rotation of q (and k), q written to q_out, k/v into pages."""
+    """Per-head norm + rotation of q (and k), q written to q_out, k/v into pages.
+    ``rotary_dim`` 0 (then ``cos`` and ``sin`` may be None): no rotation."""
     _gpu(qkv, q_weight, k_weight, cos, sin, positions, req_of_token, block_tables, q_out, k_cache, v_cache)
     n = positions.numel()
     nkv_in = num_kv_heads if store else 0
@@ -212,7 +213,9 @@ def qknorm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor | None,
     _need(q_out.numel() >= n * num_heads * head_dim, "q_out too small")
     _need(head_dim % 16 == 0 and head_dim <= 512 and page_size % 8 == 0, "head_dim must be a multiple of 16 (at most 512), page_size a multiple of 8")
     _need(rotary_dim % 2 == 0 and rotary_dim <= head_dim, "rotary_dim must be even and <= head_dim")
-    _need(cos.numel() >= n * (rotary_dim // 2) and sin.numel() >= n * (rotary_dim // 2), "rotary tables too small")
+    _need(rotary_dim == 0 or (cos is not None and sin is not None and cos.dtype == torch.float32
+                               and sin.dtype == torch.float32 and cos.numel() >= n * (rotary_dim // 2)
+                               and sin.numel() >= n * (rotary_dim // 2)), "rotary tables missing, not float32 or too small")
     for w in (q_weight, k_weight):
         _need(w is None or (w.dtype == torch.float32 and w.numel() == head_dim), "q/k norm weights are float32 [head_dim]")
     _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32
@@ -297,16 +300,31 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> N
 
 
 LT_WORKSPACE_BYTES = 128 << 20
-LT_TUNE_CANDIDATES = 16     # of the library's candidates, timed once per shape class
+LT_TUNE_CANDIDATES = 16     # of the library's candidates, timed once per shape class when tuning is on
 _lt_workspace: dict[torch.device, torch.Tensor] = {}
+_lt_tune = 1                # 1: take the library's first choice (the same in every process)
+
+
+def set_library_tuning(on: bool) -> None:
+    """Whether the library product times its candidate algorithms for each new shape
+    class and keeps the fastest.  Off (the default) every process takes the library's
+    first choice, so identical input gives identical bits from run to run; on, prompt
+    portions run up to 2x faster on some shapes, the choice depends on timing noise, and
+    the first step that meets a new shape class pays for some 60 extra products."""
+    global _lt_tune
+    _lt_tune = LT_TUNE_CANDIDATES if on else 1
+
+
+if __import__("os").environ.get("TOKAMAK_AMD_LT_TUNE", "") not in ("", "0"):
+    _lt_tune = LT_TUNE_CANDIDATES
 
 
 def gemm_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
     """out[M, N] = a[M, K] @ w[N, K]^T through hipBLASLt (bf16 in and out, float32
     accumulation), for prompt portions too long for the weight-streaming kernels.
-    The plan of each shape is kept, and the algorithm of a shape class is chosen by
-    timing the library's candidates once (csrc/blas_lt.hip).  Synchronises the first
-    time a shape class is seen, so it must not be recorded into a graph.  All calls on a
+    The plan of each shape is kept; the algorithm is the library's first choice, or with
+    ``set_library_tuning(True)`` the fastest of its candidates, timed once per shape class
+    (csrc/blas_lt.hip; that synchronises, so the call must not be recorded into a graph).  All calls on a
     device share one workspace: launch them on one stream at a time (the engine has one).
     Returns False if the library has no algorithm for the shape (nothing was computed)."""
     for t in (a, w, out):
@@ -319,7 +337,7 @@ def gemm_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
     if ws is None:
         ws = _lt_workspace[a.device] = torch.empty(LT_WORKSPACE_BYTES, dtype=torch.uint8, device=a.device)
     status = _fn("blas_lt", "tk_lt_gemm")(_p(a), _p(w), _p(out), m, n, k, a.stride(0), w.stride(0), out.stride(0),
-                                          _p(ws), ws.numel(), LT_TUNE_CANDIDATES, _stream())
+                                          _p(ws), ws.numel(), _lt_tune, _stream())
     if status == -2:
         return False
     _check(status, "gemm_library")

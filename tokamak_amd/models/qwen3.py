@@ -16,6 +16,7 @@ from tokamak_amd.config.model_config import (
     LayerSpec,
     ModelPlan,
     PartSpec,
+    SubPart,
     default_order,
 )
 from tokamak_amd.config.registry import Architecture, register_architecture
@@ -151,14 +152,19 @@ def plan(cfg: Qwen3Config) -> ModelPlan:
         head_dim=cfg.head_dim,
         qk_norm_eps=cfg.rms_norm_eps,
         softmax_scale=float(cfg.head_dim) ** -0.5,
-        position=(position.kind, position.params),
         window=None,
     )
     feed_forward = PartSpec.of(
         "swiglu", hidden_size=cfg.hidden_size, intermediate_size=cfg.intermediate_size
     )
-    layer = LayerSpec(
-        mixer=mixer, feed_forward=feed_forward, mixer_norm=norm, feed_forward_norm=norm
+    # checkpoint names as the reference's module tree gives them (transformer.py:1-6)
+    layer = LayerSpec.of(
+        PartSpec.of("pre_norm"),
+        mixer_norm=SubPart("norm", norm, "input_layernorm."),
+        mixer=SubPart("mixer", mixer, "self_attn."),
+        feed_forward_norm=SubPart("norm", norm, "post_attention_layernorm."),
+        feed_forward=SubPart("feed_forward", feed_forward, "mlp."),
+        position=SubPart("position", position, shared=True),
     )
     return ModelPlan(
         vocab_size=cfg.vocab_size,
@@ -171,8 +177,21 @@ def plan(cfg: Qwen3Config) -> ModelPlan:
         final_norm=norm,
         head=PartSpec.of("linear_head", vocab_size=cfg.vocab_size, dim=cfg.hidden_size,
                          tied=cfg.tie_word_embeddings),
+        embedding_prefix="model.embed_tokens.",
+        layer_prefix="model.layers.{}.",
+        final_norm_prefix="model.norm.",
+        head_prefix="lm_head.",
         eos_token_ids=cfg.eos_token_ids,
     )
+
+
+def chat_prompt(user_text: str) -> str:
+    """A single user turn in the ChatML form Qwen3 checkpoints are trained on, with
+    the empty think block that switches reasoning off (what the reference's example
+    asks its tokenizer's template for with enable_thinking=False,
+    examples/basic_generation.py:25-30).  Used when the model folder brings no
+    template of its own."""
+    return f"<|im_start|>user\n{user_text}<|im_end|>\n<|im_start|>assistant\n<think>\n\n</think>\n\n"
 
 
 def _shape(vocab, hidden, layers, heads, kv, hd, inter, theta, max_pos, tied, eps=1e-6) -> Qwen3Config:
@@ -189,4 +208,5 @@ PRESETS = {
 }
 
 
-register_architecture(Architecture(name=NAME, parse=parse, plan=plan, to_json=to_config_json))
+register_architecture(Architecture(name=NAME, parse=parse, plan=plan, to_json=to_config_json,
+                                   presets=PRESETS, chat_prompt=chat_prompt))

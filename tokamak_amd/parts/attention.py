@@ -4,17 +4,18 @@ from __future__ import annotations
 
 import torch
 
-from tokamak_amd.config.registry import get_part, register_part
+from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels import ops
 from tokamak_amd.kernels.attention import paged_attention
 from tokamak_amd.kernels.linear import linear
-from tokamak_amd.parts.base import CacheRequest, Fetch, Mixer
+from tokamak_amd.parts.base import CacheRequest, Fetch, Mixer, PositionData
 from tokamak_amd.weights.spec import TensorSpec
 
 
 class GQAAttention(Mixer):
-    """q/k/v projections, optional per-head RMSNorm of q and k, position
-    encoding, causal softmax attention over the request's pages, o projection
+    """q/k/v projections, optional per-head RMSNorm of q and k, rotation of q and k
+    by the tables the layer's position encoding prepared (none: no rotation),
+    causal softmax attention over the request's pages, o projection
     (reference: src/tokamak/model/transformer.py:22-86).
 
     Query head a reads kv head a // (num_heads / num_kv_heads).  Keys are cached
@@ -26,7 +27,7 @@ class GQAAttention(Mixer):
     capturable = True
 
     def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
-                 qk_norm_eps: float | None, softmax_scale: float, position, window: int | None,
+                 qk_norm_eps: float | None, softmax_scale: float, window: int | None,
                  dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)
         if num_heads % num_kv_heads:
@@ -38,8 +39,6 @@ class GQAAttention(Mixer):
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.softmax_scale = float(softmax_scale)
         self.window = None if window is None else int(window)
-        kind, params = position
-        self.position = get_part("position", kind)(**dict(params), dtype=dtype, device=device)
         self.qkv: torch.Tensor | None = None
         self.o: torch.Tensor | None = None
         self.q_norm: torch.Tensor | None = None
@@ -66,21 +65,28 @@ class GQAAttention(Mixer):
             self.k_norm = fetch(prefix + "k_norm.weight")
 
     def cache_request(self) -> CacheRequest:
-        return CacheRequest(arrays=("k", "v"), elems_per_token=self.num_kv_heads * self.head_dim,
-                            window=self.window)
+        width = self.num_kv_heads * self.head_dim
+        return CacheRequest.of(window=self.window, k=width, v=width)
 
-    def forward(self, h: torch.Tensor, batch, store, writes_cache: bool = True) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, batch, store, writes_cache: bool = True,
+                position: PositionData | None = None) -> torch.Tensor:
         nh, nkv, hd = self.num_heads, self.num_kv_heads, self.head_dim
         n = h.shape[0]
         weight = self.qkv if writes_cache else self.qkv[: nh * hd]
         qkv = linear(h, weight, allow_partials=True)
-        cos, sin = self.position.prepare(batch)
+        cos = sin = None
+        rotary_dim = 0
+        if position is not None:
+            if position.score_slopes is not None:
+                raise ops.KernelError("this attention part has no kernel for a bias on the scores; "
+                                      "it takes rotary tables or no position data")
+            cos, sin, rotary_dim = position.cos, position.sin, position.rotary_dim
         tables = batch.block_tables[store.group]
         q = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
         ops.qknorm_rope_store(
             qkv, self.q_norm, self.k_norm, cos, sin, batch.positions, batch.req_of_token, tables, q,
             store.arrays["k"], store.arrays["v"], num_heads=nh, num_kv_heads=nkv, head_dim=hd,
-            rotary_dim=self.position.rotary_dim, page_size=store.page_size,
+            rotary_dim=rotary_dim, page_size=store.page_size,
             eps=self.qk_norm_eps or 0.0, store=writes_cache)
         attended = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
         paged_attention(q, store.arrays["k"], store.arrays["v"], tables, batch, attended,

@@ -6,22 +6,27 @@ them (``bind``) and computes (``forward``).  No part knows which model it is
 in: sizes and constants arrive as parameters, checkpoint names arrive as a
 prefix, and everything about the running batch arrives in the ``StepBatch``.
 
+* ``Embedding.forward(batch)``: the float32 residual stream [N, H] of the step's
+  tokens (token rows; an absolute position encoding would be added here, from
+  ``batch.positions``).
 * ``Norm.forward(resid, delta, ...)``: adds ``delta`` into the float32 residual
   stream and returns the normed activations in the compute dtype.  ``delta`` is
   a sub-layer's output: [N, H] in the compute dtype or float32, or float32
   partial sums [P, N, H] of a split-K product, which the norm adds.
-* ``Mixer.forward(h, batch, store, writes_cache)``: token mixing.  It may own
-  paged cache (``cache_request``) and/or fixed-size per-request state
-  (``state_shape``); it sees its own storage only.
+* ``PositionEncoding.prepare(batch)``: per-step ``PositionData`` (rotary tables,
+  per-head score slopes), computed once per step and shared by every layer whose
+  encoding has the same parameters.  The block hands it to its mixer.
+* ``Mixer.forward(h, batch, store, writes_cache, position)``: token mixing.  It
+  may own paged cache (``cache_request``) and/or fixed-size per-request state
+  (``state_request``); it sees its own storage only.
 * ``FeedForward.forward(h, batch)``: token-wise map [N, H] -> [N, H].
-* ``PositionEncoding.prepare(batch)``: per-step data (e.g. rotary tables),
-  computed once per step and shared by every layer that uses the same encoding.
-* ``Block.forward(resid, pending, ...)``: the arrangement of the above.
+* ``Block.forward(resid, pending, ...)``: the arrangement of a layer's parts,
+  which it receives as a dict by role.
 """
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Callable
 
 import torch
@@ -54,16 +59,72 @@ class Part:
 
 
 @dataclass(frozen=True)
+class PagedArray:
+    """One paged array of a mixer: elements per token, and its dtype (None: the
+    engine's compute dtype)."""
+
+    elems_per_token: int
+    dtype: torch.dtype | None = None
+
+
+@dataclass(frozen=True)
 class CacheRequest:
     """What a mixer asks of the paged cache for one cache slot.
 
-    ``arrays``: name -> elements per page as a function of the page size is
-    fixed by the mixer: ``page_elems(page_size)`` per array.  ``window``: None to
-    keep every token, W if only the last W positions are ever read."""
+    ``arrays``: (name, PagedArray) pairs; the arrays of one request may differ in
+    width and dtype (keys and values of unlike sizes, a compressed latent beside
+    its rotary part).  The mixer reads ``store.arrays[name]``, laid out
+    [num_pages, elems_per_token * page_size].  ``window``: None to keep every
+    token, W if only the last W positions are ever read."""
 
-    arrays: tuple[str, ...]
-    elems_per_token: int
+    arrays: tuple[tuple[str, PagedArray], ...]
     window: int | None = None
+
+    @classmethod
+    def of(cls, window: int | None = None, **arrays: int | PagedArray) -> CacheRequest:
+        return cls(tuple((n, a if isinstance(a, PagedArray) else PagedArray(int(a))) for n, a in arrays.items()),
+                   window)
+
+    def bytes_per_token(self, default_dtype: torch.dtype) -> int:
+        return sum(a.elems_per_token * torch.empty((), dtype=a.dtype or default_dtype).element_size()
+                   for _, a in self.arrays)
+
+
+@dataclass(frozen=True)
+class StateArray:
+    """One array of a mixer's fixed-size per-request state."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class PositionData:
+    """What a position encoding hands to a mixer for one step.
+
+    ``cos``/``sin``: float32 [N, rotary_dim / 2] tables for a mixer that rotates
+    queries and keys (half-split pairing), or None.  ``score_slopes``: float32
+    [heads] for a mixer that adds ``slope * (key position - query position)`` to its
+    scores, or None.  A mixer refuses what it has no kernel for."""
+
+    cos: torch.Tensor | None = None
+    sin: torch.Tensor | None = None
+    rotary_dim: int = 0
+    score_slopes: torch.Tensor | None = None
+    extra: dict = field(default_factory=dict)
+
+
+class Embedding(Part):
+    def forward(self, batch) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def tie(self, embedding: Embedding) -> None:
+        raise NotImplementedError
 
 
 class Norm(Part):
@@ -73,7 +134,7 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    def prepare(self, batch) -> object:
+    def prepare(self, batch) -> PositionData:
         raise NotImplementedError
 
 
@@ -82,11 +143,14 @@ class Mixer(Part):
         """Paged storage per token, or None."""
         return None
 
-    def state_shape(self) -> tuple[int, ...] | None:
-        """Shape of the fixed-size per-request state, or None."""
+    def state_request(self) -> dict[str, StateArray] | None:
+        """Arrays of the fixed-size per-request state by name, or None.  The mixer
+        reads ``store.state[name][batch.state_slots[r]]``; every array is zero when
+        a request is admitted."""
         return None
 
-    def forward(self, h: torch.Tensor, batch, store, writes_cache: bool = True) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, batch, store, writes_cache: bool = True,
+                position: PositionData | None = None) -> torch.Tensor:
         raise NotImplementedError
 
 
@@ -96,15 +160,32 @@ class FeedForward(Part):
 
 
 class Block:
-    """Arrangement of one layer's parts."""
+    """Arrangement of one layer's parts.
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
-                 feed_forward_norm: Norm) -> None:
-        self.mixer = mixer
-        self.feed_forward = feed_forward
-        self.mixer_norm = mixer_norm
-        self.feed_forward_norm = feed_forward_norm
+    ``roles``: names of the parts it needs; ``optional``: of those it can do
+    without.  ``parts`` holds the built parts by role.  At most one
+    part of a block is a mixer: it owns the cache slot of the layer call.
+    """
+
+    roles: tuple[str, ...] = ()
+    optional: tuple[str, ...] = ()
+
+    def __init__(self, parts: dict[str, Part]) -> None:
+        missing = [r for r in self.roles if r not in parts]
+        unknown = [r for r in parts if r not in self.roles and r not in self.optional]
+        if missing or unknown:
+            raise ValueError(f"{type(self).__name__} needs parts {sorted(self.roles)} "
+                             f"(optional: {sorted(self.optional)}); missing {missing}, unknown {unknown}")
+        mixers = [p for p in parts.values() if isinstance(p, Mixer)]
+        if len(mixers) > 1:
+            raise ValueError(f"{type(self).__name__}: a layer has one cache slot, so at most one mixer")
+        self.parts = dict(parts)
+        self.mixer: Mixer | None = mixers[0] if mixers else None
 
     def forward(self, resid: torch.Tensor, pending: torch.Tensor | None, batch, store,
-                writes_cache: bool) -> torch.Tensor:
+                writes_cache: bool) -> torch.Tensor | None:
+        """Run the layer on the residual stream ``resid`` (float32, updated in
+        place by the norms); ``pending`` is the previous layer's last sub-layer
+        output, not yet added.  Returns this layer's last sub-layer output, to be
+        added by whoever norms next."""
         raise NotImplementedError

@@ -7,11 +7,11 @@ import torch
 from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels import ops
 from tokamak_amd.kernels.linear import linear
-from tokamak_amd.parts.base import Fetch, Part
+from tokamak_amd.parts.base import Embedding, Fetch, Head
 from tokamak_amd.weights.spec import TensorSpec
 
 
-class TokenEmbedding(Part):
+class TokenEmbedding(Embedding):
     """Plain row gather into the float32 residual stream, no scaling
     (reference: src/tokamak/model/transformer.py:140)."""
 
@@ -28,13 +28,13 @@ class TokenEmbedding(Part):
     def bind(self, prefix: str, fetch: Fetch) -> None:
         self.weight = fetch(prefix + "weight")
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
-        resid = torch.empty((token_ids.numel(), self.dim), dtype=torch.float32, device=self.device)
-        ops.embed_gather(self.weight, token_ids, resid)
+    def forward(self, batch) -> torch.Tensor:
+        resid = torch.empty((batch.num_tokens, self.dim), dtype=torch.float32, device=self.device)
+        ops.embed_gather(self.weight, batch.token_ids, resid)
         return resid
 
 
-class LinearHead(Part):
+class LinearHead(Head):
     """logits = h @ W^T in float32; a tied head uses the embedding matrix itself
     (reference: src/tokamak/model/transformer.py:154-156,173-176)."""
 

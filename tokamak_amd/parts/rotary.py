@@ -6,7 +6,7 @@ import torch
 
 from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels import ops
-from tokamak_amd.parts.base import PositionEncoding
+from tokamak_amd.parts.base import PositionData, PositionEncoding
 
 
 class RotaryHalf(PositionEncoding):
@@ -31,15 +31,15 @@ class RotaryHalf(PositionEncoding):
         self.inv_freq = inv_freq.to(self.device)
         self.key = ("rotary_half", self.rotary_dim, self.theta)
 
-    def prepare(self, batch) -> tuple[torch.Tensor, torch.Tensor]:
-        """(cos, sin), each float32 [N, rotary_dim/2]; computed once per step."""
+    def prepare(self, batch) -> PositionData:
+        """cos and sin, each float32 [N, rotary_dim/2]; computed once per step."""
         cached = batch.memo.get(self.key)
         if cached is None:
             n, half = batch.num_tokens, self.rotary_dim // 2
             cos = torch.empty((n, half), dtype=torch.float32, device=self.device)
             sin = torch.empty((n, half), dtype=torch.float32, device=self.device)
             ops.rope_tables(batch.positions, self.inv_freq, cos, sin)
-            cached = batch.memo[self.key] = (cos, sin)
+            cached = batch.memo[self.key] = PositionData(cos=cos, sin=sin, rotary_dim=self.rotary_dim)
         return cached
 
 
