@@ -124,3 +124,82 @@ def test_partspec_is_hashable_and_frozen():
     a = PartSpec.of("x", b=2, a=[1, 2])
     assert a == PartSpec.of("x", a=(1, 2), b=2) and hash(a) == hash(PartSpec.of("x", a=(1, 2), b=2))
     assert a.as_dict() == {"a": (1, 2), "b": 2}
+
+
+# -- where the EOS ids come from (reference src/tokamak/engine/llm.py:244-263) ---------
+def _folder(tmp_path, generation=None, config_eos=..., tokenizer=False):
+    from tokamak_amd.config import read_eos_token_ids
+
+    cfg = qwen3.to_config_json(qwen3.parse(raw(), ()))
+    if config_eos is not ...:
+        cfg["eos_token_id"] = config_eos
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    if generation is not None:
+        (tmp_path / "generation_config.json").write_text(json.dumps(generation))
+    if tokenizer:
+        (tmp_path / "tokenizer_config.json").write_text(json.dumps({"eos_token": "<|end|>"}))
+        (tmp_path / "tokenizer.json").write_text(json.dumps(
+            {"added_tokens": [{"id": 901, "content": "<|end|>"}], "model": {"vocab": {"a": 0}}}))
+    return read_eos_token_ids(tmp_path)
+
+
+def test_eos_from_generation_config_int_or_list(tmp_path):
+    assert _folder(tmp_path, generation={"eos_token_id": 5}, config_eos=9, tokenizer=True) == (5,)
+    assert _folder(tmp_path, generation={"eos_token_id": [5, 6]}) == (5, 6)
+
+
+def test_eos_falls_back_to_config_json_then_to_the_tokenizer(tmp_path):
+    assert _folder(tmp_path, generation={"temperature": 0.6}, config_eos=[9, 10], tokenizer=True) == (9, 10)
+    (tmp_path / "generation_config.json").unlink()
+    assert _folder(tmp_path, config_eos=9, tokenizer=True) == (9,)
+    assert _folder(tmp_path, tokenizer=True) == (901,)          # the tokenizer's eos_token, looked up by text
+    assert load_model_description(tmp_path)[2].eos_token_ids == (901,)
+
+
+def test_no_eos_anywhere_means_requests_stop_on_length(tmp_path):
+    assert _folder(tmp_path) == ()
+    assert _folder(tmp_path, generation={"eos_token_id": True}) == ()     # a bool is no token id
+
+
+# -- presets and the chat prompt come through the registry -------------------------------
+def test_presets_are_found_by_name_through_the_registry():
+    from tokamak_amd.config import find_preset, preset_names
+
+    assert {"tiny-a", "tiny-b", "qwen3-0.6b", "qwen3-8b", "qwen3-32b"} <= set(preset_names())
+    arch, cfg = find_preset("qwen3-8b")
+    assert arch.name == "Qwen3ForCausalLM" and cfg.hidden_size == 4096 and cfg.num_layers == 36
+    with pytest.raises(ValueError, match="unknown preset 'nope'.*tiny-a"):
+        find_preset("nope")
+
+
+def test_architecture_brings_its_chat_prompt():
+    text = get_architecture("Qwen3ForCausalLM").chat_prompt("hi")
+    assert text.startswith("<|im_start|>user\nhi<|im_end|>") and text.endswith("<think>\n\n</think>\n\n")
+
+
+def test_entry_points_name_no_architecture():
+    """The command line and the benchmark reach shapes and models through the registry."""
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parent.parent
+    for file in (root / "tokamak_amd" / "cli.py", root / "bench.py", root / "bin" / "trace_run",
+                 root / "tokamak_amd" / "engine" / "llm.py", root / "tokamak_amd" / "engine" / "runner.py"):
+        assert "models.qwen3" not in file.read_text() and "import qwen3" not in file.read_text(), file
+
+
+def test_a_block_says_which_parts_it_needs():
+    import torch
+
+    from tokamak_amd.config import LayerSpec, SubPart
+    from tokamak_amd.engine.model import LayeredModel
+
+    plan = qwen3.plan(qwen3.parse(raw(), ()))
+    layer = plan.layers[0]
+    broken = LayerSpec(tuple((r, p) for r, p in layer.parts if r != "feed_forward_norm")
+                       + (("extra", SubPart("norm", layer.role("mixer_norm").spec, "x.")),), layer.block)
+    import dataclasses
+    with pytest.raises(ValueError, match="missing \\['feed_forward_norm'\\], unknown \\['extra'\\]"):
+        LayeredModel(dataclasses.replace(plan, layers=(broken, broken)), dtype=torch.float32, device="meta")
+    model = LayeredModel(plan, dtype=torch.float32, device="meta")
+    assert model.blocks[0].parts["position"] is model.blocks[1].parts["position"]      # shared: one table a step
+    assert model.blocks[0].parts["mixer"] is not model.blocks[1].parts["mixer"]

@@ -42,10 +42,21 @@ class KernelBuildError(RuntimeError):
 
 
 def sources_of(name: str) -> list[Path]:
+    """The library's source and the headers of this folder that it includes (directly
+    or through another of them)."""
     src = CSRC / f"{name}.hip"
     if not src.is_file():
         raise KernelBuildError(f"no kernel source {src}")
-    return [src, *sorted(CSRC.glob("*.h"))]
+    found, todo = [src], [src]
+    while todo:
+        for line in todo.pop().read_text().splitlines():
+            line = line.strip()
+            if line.startswith("#include \""):
+                header = CSRC / line.split('"')[1]
+                if header.is_file() and header not in found:
+                    found.append(header)
+                    todo.append(header)
+    return [src, *sorted(found[1:])]
 
 
 def _digest(name: str) -> str:
