@@ -1,19 +1,31 @@
 """Decode and prefill throughput of a Qwen3-8B-shaped model with random weights.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 36]
+    python bench.py [--gpus 1] [--steps 256] [--warmup 8] [--batch 8] [--prompt 2048]
+                    [--context C] [--layers L] [--shape PRESET] [--profile]
 
-Prints one JSON line.  A "step" is one decode step of the whole batch through
-the engine's own step function and greedy sampler, each request holding
-``context`` tokens at the end of the timed steps.  ``value`` is decoded tokens
-per second.  ``prefill`` is one 2,048-token prompt in one step; ``roofline``
-prices the decode step against HBM: every weight it uses once plus the cache of
-the live requests, divided by its time.  Peaks: HBM 8 TB/s, dense bf16 MFMA
-2.5 PFLOP/s (MI355X, published).
+Prints one JSON line.  The default workload is the headline one as written: every
+request of the batch has a 2,048-token random prompt and generates 256 tokens
+greedily; a "step" is one decode step of the whole batch through the engine's own
+step function and sampler; all ``--steps`` steps after the prompt are timed, three
+times over (fresh requests each time), and the median run is reported.  ``--warmup``
+steps of the same workload run untimed before (they also record the decode graph).
+``--context C`` instead times the last ``--steps`` steps before each request holds C
+tokens (a longer context than the headline's).
+
+``value`` is decoded tokens per second.  ``prefill`` is one 2,048-token prompt in one
+step.  ``roofline`` prices the decode step against HBM: every weight it uses once plus
+the cache of the live requests at the mean context of the timed steps, divided by its
+time.  Fractions are of the published peaks (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s);
+``peaks`` holds what two microbenchmarks of this program reach on this GPU (streaming
+reads and copies of 4 GiB; back-to-back MFMA from registers), and ``frac_of_measured``
+the same fractions of those.  ``--profile`` adds ``kernels``: one decode step and one
+prefill step with every kernel call timed by events, summed by kind of call.
 """
 
 from __future__ import annotations
 
 import argparse
+import ctypes
 import dataclasses
 import json
 import statistics
@@ -26,44 +38,121 @@ sys.path.insert(0, str(Path(__file__).resolve().parent))
 HBM_PEAK = 8.0e12
 MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 PREFILL_TOKENS = 2048
-SHAPE_NAMES = {"qwen3-0.6b": "Qwen3-0.6B", "qwen3-8b": "Qwen3-8B", "qwen3-32b": "Qwen3-32B"}
+PAGE_SIZE = 16
 
 
-def make_runner(cfg, dtype, pool_tokens, max_requests, seed=0):
+# ---------------------------------------------------------------------------
+# what this GPU reaches
+# ---------------------------------------------------------------------------
+def measure_peaks() -> dict:
+    """Streaming read and copy of 4 GiB (far beyond every cache) and bf16 MFMA from
+    registers, each the best of five launches after an untimed one."""
+    import torch
+
+    from tokamak_amd.kernels.build import load_library
+
+    lib = load_library("peaks")
+    c_void_p, c_size_t, c_int = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    lib.tk_peak_read.argtypes = [c_void_p, c_size_t, c_void_p, c_int, c_void_p]
+    lib.tk_peak_copy.argtypes = [c_void_p, c_void_p, c_size_t, c_int, c_void_p]
+    lib.tk_peak_mfma.argtypes = [c_int, c_int, c_int, c_void_p, ctypes.POINTER(ctypes.c_double), c_void_p]
+    stream = c_void_p(torch.cuda.current_stream().cuda_stream)
+    nbytes = 4 << 30
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").fill_(1)
+    dst = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
+    sink = torch.zeros(65536, dtype=torch.float32, device="cuda:0")
+
+    def best(launch) -> float:
+        times = []
+        for _ in range(6):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            assert launch() == 0
+            e1.record()
+            e1.synchronize()
+            times.append(e0.elapsed_time(e1) * 1e-3)
+        return min(times[1:])
+
+    blocks = 256 * 16
+    read_s = best(lambda: lib.tk_peak_read(src.data_ptr(), nbytes, sink.data_ptr(), blocks, stream))
+    copy_s = best(lambda: lib.tk_peak_copy(src.data_ptr(), dst.data_ptr(), nbytes, blocks, stream))
+    mfma = {}
+    for shape, name in ((0, "16x16x32"), (1, "32x32x16")):
+        flops = ctypes.c_double(0.0)
+        seconds = best(lambda: lib.tk_peak_mfma(shape, 256 * 8, 20000, sink.data_ptr(), ctypes.byref(flops), stream))
+        mfma[name] = flops.value / seconds
+    del src, dst
+    torch.cuda.empty_cache()
+    return {"hbm_read_measured": round(nbytes / read_s / 1e9, 1),
+            "hbm_copy_measured": round(2 * nbytes / copy_s / 1e9, 1),
+            "mfma_bf16_measured": round(max(mfma.values()) / 1e12, 1),
+            "mfma_bf16_16x16x32": round(mfma["16x16x32"] / 1e12, 1),
+            "hbm_published": HBM_PEAK / 1e9, "mfma_bf16_published": MFMA_PEAK["bf16"] / 1e12,
+            "units": "GB/s, TFLOP/s"}
+
+
+# ---------------------------------------------------------------------------
+# the model and what a step has to move and compute, from the plan
+# ---------------------------------------------------------------------------
+def make_runner(arch, cfg, dtype, pool_tokens, max_requests, seed=0):
     import torch
 
     from tokamak_amd.engine.runner import ModelRunner
-    from tokamak_amd.config import get_architecture
     from tokamak_amd.weights.random_init import expected_tensors_of
     from tokamak_amd.weights.sources import RandomSource
 
-    plan = get_architecture(cfg.architecture).plan(cfg)
+    plan = arch.plan(cfg)
     expected = {n: s for n, s in expected_tensors_of(plan).items() if not s.ignored}
     tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     source = RandomSource(expected, seed, matrix_std=0.02, vector_jitter=0.0, dtype=tdt, device="cuda:0")
-    return ModelRunner(plan, source, dtype=dtype, page_size=16, kv_pool_tokens=pool_tokens,
+    return ModelRunner(plan, source, dtype=dtype, page_size=PAGE_SIZE, kv_pool_tokens=pool_tokens,
                        max_requests=max_requests)
 
 
-def weight_bytes(cfg, elem):
-    per_layer = ((cfg.num_attention_heads + 2 * cfg.num_kv_heads) * cfg.head_dim * cfg.hidden_size
-                 + cfg.hidden_size * cfg.num_attention_heads * cfg.head_dim
-                 + 3 * cfg.hidden_size * cfg.intermediate_size)
-    return (per_layer * cfg.num_layers + cfg.vocab_size * cfg.hidden_size) * elem
+class StepCost:
+    """Bytes and flops of steps of the model a runner holds, from its own tensors and
+    cache layout (nothing here names an architecture)."""
+
+    def __init__(self, runner) -> None:
+        model, plan = runner.model, runner.plan
+        elem = 2 if runner.dtype.itemsize == 2 else 4
+        tensors = {n: s for n, s in model.expected_tensors().items() if not s.ignored}
+        size = {n: (4 if s.role != "matrix" else elem) for n, s in tensors.items()}
+        numel = {n: _prod(s.shape) for n, s in tensors.items()}
+        embedding = set(model.embedding.expected_tensors(plan.embedding_prefix))
+        head = {n for n in model.head.expected_tensors(plan.head_prefix) if n in tensors}
+        self.hidden = plan.hidden_size
+        self.elem = elem
+        # every tensor a decode step reads whole: all but the embedding table (a row a token),
+        # unless the head is tied to it
+        self.weight_bytes = sum(numel[n] * size[n] for n in tensors if n not in embedding or plan.tie_word_embeddings)
+        self.embedding_row_bytes = plan.hidden_size * elem
+        self.matrix_params = sum(numel[n] for n, s in tensors.items()
+                                 if s.role == "matrix" and n not in embedding and n not in head)
+        self.head_params = plan.vocab_size * plan.hidden_size
+        _, layouts = model.cache_layout()
+        self.kv_bytes_per_token = sum(lay.request.bytes_per_token(runner.dtype) for lay in layouts.values())
+        # attention flops of a layer call: 4 * heads * head_dim per (query, visible key) pair
+        self.pair_flops = 0.0
+        for call in plan.order:
+            for _, sub in plan.layers[call.layer].parts:
+                params = sub.spec.as_dict()
+                if sub.family == "mixer" and "num_heads" in params and "head_dim" in params:
+                    self.pair_flops += 4.0 * params["num_heads"] * params["head_dim"]
+
+    def decode_bytes(self, batch: int, mean_keys: float) -> float:
+        return self.weight_bytes + batch * (self.embedding_row_bytes + mean_keys * self.kv_bytes_per_token)
+
+    def prefill_flops(self, tokens: int) -> float:
+        return (2.0 * tokens * self.matrix_params + self.pair_flops * tokens * (tokens + 1) / 2
+                + 2.0 * self.head_params)
 
 
-def kv_bytes_per_token(cfg, elem):
-    return 2 * cfg.num_layers * cfg.num_kv_heads * cfg.head_dim * elem
-
-
-def prefill_flops(cfg, t):
-    per_layer = ((cfg.num_attention_heads + 2 * cfg.num_kv_heads) * cfg.head_dim * cfg.hidden_size
-                 + cfg.hidden_size * cfg.num_attention_heads * cfg.head_dim
-                 + 3 * cfg.hidden_size * cfg.intermediate_size)
-    linear = 2.0 * t * per_layer * cfg.num_layers
-    attention = 4.0 * cfg.num_attention_heads * cfg.head_dim * (t * (t + 1) / 2) * cfg.num_layers
-    head = 2.0 * cfg.vocab_size * cfg.hidden_size
-    return linear + attention + head
+def _prod(shape) -> int:
+    out = 1
+    for d in shape:
+        out *= int(d)
+    return out
 
 
 def random_prompt(vocab, n, seed):
@@ -84,14 +173,17 @@ def fill(runner, request, tokens, chunk=2048):
     return logits
 
 
-def time_prefill(runner, cfg, repeats=5):
+# ---------------------------------------------------------------------------
+# timing
+# ---------------------------------------------------------------------------
+def time_prefill(runner, vocab, repeats=5):
     import torch
 
     from tokamak_amd.engine.runner import StepEntry
 
     times = []
-    for i in range(repeats + 2):  # the first two are untimed (kernel choice of the library products, clocks)
-        ids = random_prompt(cfg.vocab_size, PREFILL_TOKENS, 1000 + i)
+    for i in range(repeats + 2):  # the first two are untimed (plans of the library products, clocks)
+        ids = random_prompt(vocab, PREFILL_TOKENS, 1000 + i)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         runner.step([StepEntry("prefill", ids, [PREFILL_TOKENS - 1])])
@@ -101,39 +193,109 @@ def time_prefill(runner, cfg, repeats=5):
     return statistics.median(times[2:])
 
 
-def time_decode(runner, cfg, batch, context, steps, warmup):
-    """``batch`` requests reach ``context`` tokens at the end of the timed steps."""
+def decode_pass(runner, vocab, batch, prompt_tokens, steps, seed):
+    """``batch`` fresh requests with ``prompt_tokens``-token prompts, then ``steps`` greedy
+    decode steps of the whole batch; seconds for those steps."""
     import torch
 
     from tokamak_amd.engine.runner import StepEntry
     from tokamak_amd.sampling.sampler import greedy_tokens
 
-    start = context - steps - warmup
-    assert start >= 1
     last = []
     for r in range(batch):
-        logits = fill(runner, r, random_prompt(cfg.vocab_size, start, 7 + r))
+        logits = fill(runner, r, random_prompt(vocab, prompt_tokens, seed * 1000 + r))
         last.append(int(greedy_tokens(logits).item()))
-
-    def one_step():
-        nonlocal last
-        logits = runner.step([StepEntry(r, [last[r]], [0]) for r in range(batch)])
-        last = greedy_tokens(logits).tolist()
-
-    for _ in range(warmup):
-        one_step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        one_step()
+        logits = runner.step([StepEntry(r, [last[r]], [0]) for r in range(batch)])
+        last = greedy_tokens(logits).tolist()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    mean_ctx = context - (steps + 1) / 2.0
     for r in range(batch):
         runner.end(r)
-    return elapsed / steps, mean_ctx
+    return elapsed
 
 
+def time_decode(runner, vocab, batch, prompt_tokens, steps, warmup, repeats):
+    """Median seconds per step over ``repeats`` timed passes, after one untimed pass of
+    ``warmup`` steps; and every pass's figure."""
+    if warmup > 0:
+        decode_pass(runner, vocab, batch, prompt_tokens, warmup, seed=0)
+    runs = [decode_pass(runner, vocab, batch, prompt_tokens, steps, seed=1 + i) / steps for i in range(repeats)]
+    return statistics.median(runs), runs
+
+
+def profile_step(runner, entries, blocker):
+    """One step, eagerly, every kernel call between two events.  A few long copies are
+    queued first so that the step's launches are all in the queue before the first runs:
+    what the events bracket is then the kernels, not the host's launch gaps."""
+    from tokamak_amd.kernels import ops
+
+    graphs, runner.use_graphs = runner.use_graphs, False
+    try:
+        blocker()
+        with ops.KernelProfile() as prof:
+            runner.step(entries)
+        return prof.rows()
+    finally:
+        runner.use_graphs = graphs
+
+
+def kernel_table(rows, key, top=14):
+    out = []
+    for row in rows[:top]:
+        seconds = row["us"] * 1e-6
+        rec = {"name": row["name"], "calls": row["calls"], "us": round(row["us"], 1)}
+        if row["bytes"]:
+            rec["GBps"] = round(row["bytes"] / seconds / 1e9, 1)
+        if row["flops"]:
+            rec["TFLOPs"] = round(row["flops"] / seconds / 1e12, 1)
+        fracs = [row["bytes"] / seconds / HBM_PEAK, row["flops"] / seconds / MFMA_PEAK[key]]
+        rec["frac"] = round(max(fracs), 3)
+        rec["bound"] = "hbm" if fracs[0] >= fracs[1] else "mfma"
+        out.append(rec)
+    rest = rows[top:]
+    if rest:
+        out.append({"name": f"{len(rest)} other kinds", "calls": sum(r["calls"] for r in rest),
+                    "us": round(sum(r["us"] for r in rest), 1)})
+    return out
+
+
+def profile_kernels(runner, vocab, batch, prompt_tokens, key, blocker):
+    from tokamak_amd.engine.runner import StepEntry
+
+    for r in range(batch):
+        fill(runner, r, random_prompt(vocab, prompt_tokens + 127, 77 + r))
+    graphs, runner.use_graphs = runner.use_graphs, False
+    runner.step([StepEntry(r, [1 + r], [0]) for r in range(batch)])          # untimed: code objects, allocator
+    runner.use_graphs = graphs
+    decode = profile_step(runner, [StepEntry(r, [2 + r], [0]) for r in range(batch)], blocker)
+    for r in range(batch):
+        runner.end(r)
+    ids = random_prompt(vocab, PREFILL_TOKENS, 5)
+    prefill = profile_step(runner, [StepEntry("prefill", ids, [PREFILL_TOKENS - 1])], blocker)
+    runner.end("prefill")
+    return {"decode": kernel_table(decode, key), "prefill": kernel_table(prefill, key),
+            "decode_sum_us": round(sum(r["us"] for r in decode), 1),
+            "prefill_sum_us": round(sum(r["us"] for r in prefill), 1)}
+
+
+def make_blocker():
+    """A callable that queues ~25 ms of copies on the current stream."""
+    import torch
+
+    a = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0")
+    b = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0")
+
+    def blocker():
+        for _ in range(40):
+            b.copy_(a)
+
+    return blocker
+
+
+# ---------------------------------------------------------------------------
 def run_continuous(args) -> int:
     """Optional extra workload: continuous batching through ``LLM.generate`` (scheduler,
     portions of prompts beside decode tokens, captured decode steps).  Prompt and output
@@ -156,7 +318,7 @@ def run_continuous(args) -> int:
     pool = args.max_batch * (p_hi + o_hi)  # every running request fits at full length
     llm = LLM(cfg, seed=0, random_weights_on_gpu=True, dtype=args.dtype, max_seq_len=max_len,
               kv_pool_tokens=max(pool, max_len), max_batch_size=args.max_batch, max_num_batched_tokens=2048,
-              prefill_chunk=2048)
+              prefill_chunk=2048, tune_library_products=not args.no_tune)
     runs = []
     for _ in range(2):  # the first run also records the decode graphs
         steps0 = llm.num_steps
@@ -177,49 +339,34 @@ def run_continuous(args) -> int:
                    "prompt_tokens": sum(map(len, prompts)), "output_tokens": out_tokens,
                    "total_tok_per_s": round((sum(map(len, prompts)) + out_tokens) / elapsed, 1),
                    "first_run_s": round(runs[0][0], 3), "preemptions": llm.num_preemptions,
-                   "parallelism": "single GPU"},
-    }))
-    return 0
-
-
-def run_phase(args, runner, cfg, full) -> int:
-    """One part alone, so that a profile of the run holds that part's kernels only
-    (the decode part still has to fill the requests' caches first)."""
-    key = "bf16" if args.dtype == "bfloat16" else "fp32"
-    if args.phase == "prefill":
-        seconds = time_prefill(runner, cfg, repeats=max(args.steps, 1))
-        value, steps, what = PREFILL_TOKENS / seconds, max(args.steps, 1), f"prefill tok/s at {PREFILL_TOKENS} tokens"
-    else:
-        seconds, _ = time_decode(runner, cfg, args.batch, args.context, args.steps, args.warmup)
-        value, steps, what = args.batch / seconds, args.steps, f"decode tok/s at batch {args.batch}"
-    print(json.dumps({
-        "metric": f"{what} ({SHAPE_NAMES[args.shape]}-shaped, random weights)", "value": round(value, 1), "unit": "tokens/s",
-        "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": round(seconds * 1e3, 3),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": key,
-        "data": "synthetic (uniform random token ids, seeded random weights)",
-        "config": {"model": f"{args.shape}-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers,
-                   "global_batch": args.batch, "seq_len": args.context, "phase": args.phase,
-                   "parallelism": "single GPU"},
+                   "tuned_products": not args.no_tune, "parallelism": "single GPU"},
     }))
     return 0
 
 
 def main() -> int:
-    ap = argparse.ArgumentParser()
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--steps", type=int, default=256, help="timed decode steps of a pass (the headline workload: 256)")
+    ap.add_argument("--warmup", type=int, default=8, help="untimed decode steps before the timed passes")
+    ap.add_argument("--repeats", type=int, default=3, help="timed passes; the median is reported")
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prompt", type=int, default=2048, help="prompt tokens of every request")
+    ap.add_argument("--context", type=int, default=None,
+                    help="instead of --prompt: the timed steps end when each request holds this many tokens")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the microbenchmarks of this GPU's peaks")
+    ap.add_argument("--no-tune", action="store_true",
+                    help="take the library's first algorithm for long portions' products instead of timing its candidates")
+    ap.add_argument("--profile", action="store_true", help="add per-kernel times of one decode and one prefill step")
     ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
-                    help="run only one part (for profiles); the other part's figures are null")
+                    help="run only one part (for an external profiler); the other part's figures are null")
     ap.add_argument("--workload", default="decode", choices=["decode", "continuous"],
                     help="decode: the headline measurement; continuous: LLM.generate over many requests")
     ap.add_argument("--model", default="qwen3-0.6b", help="preset shape of the continuous workload")
-    ap.add_argument("--shape", default="qwen3-8b", choices=["qwen3-0.6b", "qwen3-8b", "qwen3-32b"],
+    ap.add_argument("--shape", default="qwen3-8b",
                     help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
     ap.add_argument("--requests", type=int, default=256)
     ap.add_argument("--max-batch", type=int, default=64)
@@ -232,59 +379,80 @@ def main() -> int:
     if args.workload == "continuous":
         return run_continuous(args)
 
-    import torch
-
     from tokamak_amd.config import find_preset
+    from tokamak_amd.kernels import ops
 
-    full = find_preset(args.shape)[1]
+    arch, full = find_preset(args.shape)
     cfg = dataclasses.replace(full, num_layers=args.layers or full.num_layers)
-    elem = 2 if args.dtype == "bfloat16" else 4
-    max_batch = 64 if not (args.no_points or args.phase != "all") else args.batch
-    pool = max(max_batch, args.batch) * (args.context + 16)
-    runner = make_runner(cfg, args.dtype, pool, max(max_batch, args.batch))
-
-    if args.phase != "all":
-        return run_phase(args, runner, cfg, full)
-    prefill_s = time_prefill(runner, cfg)
-    step_s, mean_ctx = time_decode(runner, cfg, args.batch, args.context, args.steps, args.warmup)
-    points = {}
-    if not args.no_points:
-        for b, k in ((1, min(args.steps, 64)), (64, min(args.steps, 32))):
-            s, _ = time_decode(runner, cfg, b, args.context, k, min(args.warmup, 4))
-            points[f"decode_b{b}"] = round(b / s, 1)
-
-    step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
-    achieved = step_bytes / step_s
     key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    prompt_tokens = args.prompt if args.context is None else args.context - args.steps
+    if prompt_tokens < 1:
+        ap.error("--context must exceed --steps")
+    final_context = prompt_tokens + args.steps
+    want_points = not args.no_points and args.phase == "all"
+    max_batch = max(64 if want_points else 1, args.batch)
+    peaks = None if args.no_peaks else measure_peaks()
+    ops.set_library_tuning(not args.no_tune)
+    pool = max_batch * (-(-(final_context + 1) // PAGE_SIZE) * PAGE_SIZE + PAGE_SIZE)
+    runner = make_runner(arch, cfg, args.dtype, max(pool, PREFILL_TOKENS + PAGE_SIZE), max_batch)
+    cost = StepCost(runner)
+    vocab = runner.plan.vocab_size
+
+    prefill_s = time_prefill(runner, vocab) if args.phase in ("all", "prefill") else None
+    step_s = runs = None
+    if args.phase in ("all", "decode"):
+        step_s, runs = time_decode(runner, vocab, args.batch, prompt_tokens, args.steps, args.warmup, args.repeats)
+    points = {}
+    if want_points:
+        for b in (1, 64):
+            s, _ = time_decode(runner, vocab, b, prompt_tokens, args.steps, min(args.warmup, 4), args.repeats)
+            keys = prompt_tokens + (args.steps + 1) / 2.0
+            points[f"decode_b{b}"] = round(b / s, 1)
+            points[f"decode_b{b}_hbm_frac"] = round(cost.decode_bytes(b, keys) / s / HBM_PEAK, 4)
+    kernels = None
+    if args.profile:
+        kernels = profile_kernels(runner, vocab, args.batch, prompt_tokens, key, make_blocker())
+
+    sizes = arch.to_json(cfg) if arch.to_json else {}
+    config = {"model": f"{args.shape}-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers}
+    for name, short in (("hidden_size", "hidden_size"), ("num_attention_heads", "heads"),
+                        ("num_key_value_heads", "kv_heads"), ("head_dim", "head_dim"),
+                        ("intermediate_size", "intermediate_size"), ("vocab_size", "vocab_size")):
+        if name in sizes:
+            config[short] = sizes[name]
+    config.update({"global_batch": args.batch, "prompt_tokens": prompt_tokens, "generated_tokens": args.steps,
+                   "seq_len": final_context, "page_size": PAGE_SIZE, "repeats": args.repeats,
+                   "tuned_products": not args.no_tune, "sampling": "greedy", "parallelism": "single GPU"})
+    what = (f"decode tok/s at batch {args.batch} ({args.shape}-shaped, random weights, {prompt_tokens}-token prompts "
+            f"+ {args.steps} generated); prefill tok/s at {PREFILL_TOKENS} tokens")
     result = {
-        "metric": f"decode tok/s at batch {args.batch} ({SHAPE_NAMES[args.shape]}-shaped, random weights); prefill tok/s at 2,048 tokens",
-        "value": round(args.batch / step_s, 1),
-        "unit": "tokens/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(step_s * 1e3, 3),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": key,
+        "metric": what, "value": None, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": key,
         "data": "synthetic (uniform random token ids, seeded random weights N(0, 0.02), norm weights 1)",
-        "config": {
-            "model": f"{args.shape}-shaped", "layers": cfg.num_layers, "layers_of_model": full.num_layers,
-            "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_kv_heads,
-            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size,
-            "vocab_size": cfg.vocab_size, "global_batch": args.batch, "seq_len": args.context,
-            "page_size": 16, "sampling": "greedy", "parallelism": "single GPU",
-        },
-        "prefill": {
-            "value": round(PREFILL_TOKENS / prefill_s, 1), "tokens": PREFILL_TOKENS,
-            "ms": round(prefill_s * 1e3, 3),
-            "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / prefill_s / MFMA_PEAK[key], 4),
-        },
-        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)},
-        "points": points,
+        "config": config,
     }
+    if step_s is not None:
+        mean_keys = prompt_tokens + (args.steps + 1) / 2.0
+        achieved = cost.decode_bytes(args.batch, mean_keys) / step_s
+        result.update({"value": round(args.batch / step_s, 1), "ms_per_step": round(step_s * 1e3, 3),
+                       "runs_ms_per_step": [round(r * 1e3, 3) for r in runs]})
+        result["roofline"] = {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9,
+                              "unit": "GB/s", "frac": round(achieved / HBM_PEAK, 4)}
+        if peaks:
+            result["roofline"]["frac_of_measured"] = round(achieved / 1e9 / peaks["hbm_read_measured"], 4)
+    if prefill_s is not None:
+        flops = cost.prefill_flops(PREFILL_TOKENS)
+        result["prefill"] = {"value": round(PREFILL_TOKENS / prefill_s, 1), "tokens": PREFILL_TOKENS,
+                             "ms": round(prefill_s * 1e3, 3), "frac": round(flops / prefill_s / MFMA_PEAK[key], 4)}
+        if peaks and key == "bf16":
+            result["prefill"]["frac_of_measured"] = round(flops / prefill_s / 1e12 / peaks["mfma_bf16_measured"], 4)
+        if step_s is None:
+            result.update({"value": result["prefill"]["value"], "ms_per_step": result["prefill"]["ms"], "steps": 5})
+    result["points"] = points
+    if peaks:
+        result["peaks"] = peaks
+    if kernels:
+        result["kernels"] = kernels
     print(json.dumps(result))
     return 0
 

@@ -62,11 +62,21 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     prompt portions (their keys split too when the tiles are few and the context
     long).  Everything else: the generic float32-arithmetic kernel.
     """
+    profiling = ops._profile is not None
+    if profiling:
+        # keys each query sees; the cache bytes of a request are read once per kv head
+        decode_keys = sum(c + 1 for c, n in zip(batch.ctx_lens, batch.q_lens) if n == 1)
+        tile_pairs = sum(n * c + n * (n + 1) // 2 for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
+        tile_keys = sum(c + n for c, n in zip(batch.ctx_lens, batch.q_lens) if n > 1)
+        kv_token_bytes = 2 * num_kv_heads * head_dim * q.element_size()
+        flops_per_pair = 4.0 * num_heads * head_dim
     if mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, window):
         common = dict(num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
                       page_size=page_size, scale=scale)
         if batch.num_decode:
             split, nsplit = decode_split(batch.num_decode, num_kv_heads, batch.max_decode_len)
+            if profiling:
+                ops._note(f"decode {batch.num_decode} tokens", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
             ops.attention_mfma("heads", q, k_cache, v_cache, block_tables, batch.positions,
                                batch.req_of_token, batch.decode_tokens, None, batch.num_decode, out,
                                split_keys=split, num_splits=nsplit, **common)
@@ -75,10 +85,15 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
             per_tile = num_kv_heads * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
             split, nsplit = tile_split(batch.num_tiles, per_tile, batch.max_tile_len)
             dense = nsplit == 1 and batch.min_tile_ctx >= DENSE_TILES_FROM
+            if profiling:
+                ops._note(f"portions {batch.num_tiles} tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
             ops.attention_mfma("tokens_dense" if dense else "tokens", q, k_cache, v_cache, block_tables, batch.positions,
                                batch.req_of_token, batch.tile_first, batch.tile_count, batch.num_tiles,
                                out, split_keys=split, num_splits=nsplit, **common)
         return
+    if profiling:
+        ops._note(f"{batch.num_tokens} tokens", (decode_keys + tile_keys) * kv_token_bytes,
+                  (decode_keys + tile_pairs) * flops_per_pair)
     ops.paged_attention_generic(
         q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
         num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,

@@ -120,6 +120,60 @@ _SIGS = {
     },
 }
 _fns: dict[str, ctypes._CFuncPtr] = {}
+_profile: "KernelProfile | None" = None
+
+
+class KernelProfile:
+    """Times every kernel entry point called inside the ``with`` block with a pair
+    of events on the current stream, and keeps what each call says about itself
+    (shape, bytes it has to move, flops).  ``rows()`` gives one record per kind of
+    call, summed.  Meant for one step at a time; the events add a few microseconds
+    a launch, so the sum is above the step's time without them."""
+
+    def __init__(self) -> None:
+        self.calls: list[tuple[str, torch.cuda.Event, torch.cuda.Event, float, float]] = []
+        self._note: tuple[str, float, float] | None = None
+
+    def __enter__(self) -> "KernelProfile":
+        global _profile
+        self._before, _profile = _profile, self
+        return self
+
+    def __exit__(self, *exc) -> bool:
+        global _profile
+        _profile = self._before
+        return False
+
+    def note(self, shape: str, nbytes: float = 0.0, flops: float = 0.0) -> None:
+        self._note = (shape, float(nbytes), float(flops))
+
+    def timed(self, name: str, fn, args):
+        shape, nbytes, flops = self._note or ("", 0.0, 0.0)
+        self._note = None
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        status = fn(*args)
+        e1.record()
+        self.calls.append((f"{name[3:]} {shape}".strip(), e0, e1, nbytes, flops))
+        return status
+
+    def rows(self) -> list[dict]:
+        """[{name, calls, us, bytes, flops}], longest first; synchronises."""
+        torch.cuda.synchronize()
+        merged: dict[str, dict] = {}
+        for name, e0, e1, nbytes, flops in self.calls:
+            row = merged.setdefault(name, {"name": name, "calls": 0, "us": 0.0, "bytes": 0.0, "flops": 0.0})
+            row["calls"] += 1
+            row["us"] += e0.elapsed_time(e1) * 1e3
+            row["bytes"] += nbytes
+            row["flops"] += flops
+        return sorted(merged.values(), key=lambda r: -r["us"])
+
+
+def _note(shape: str, nbytes: float = 0.0, flops: float = 0.0) -> None:
+    """What the next kernel call is, for a running ``KernelProfile`` (else nothing)."""
+    if _profile is not None:
+        _profile.note(shape, nbytes, flops)
 
 
 def _fn(library: str, name: str):
@@ -132,6 +186,9 @@ def _fn(library: str, name: str):
         fn.argtypes = _SIGS[library][name]
         fn.restype = c_int
         _fns[name] = fn
+    if _profile is not None and name not in ("tk_argmax_segments",):
+        profile = _profile
+        return lambda *args: profile.timed(name, fn, args)
     return fn
 
 
@@ -144,6 +201,7 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, resid: torch.Tensor) ->
     _need(ids.dtype == torch.int32, "token ids must be int32")
     _need(resid.dtype == torch.float32 and resid.shape[-1] == h and resid.numel() >= n * h,
           "residual buffer must be float32 [>=N, H]")
+    _note(f"{n}x{h}", n * h * (table.element_size() + 4))
     _check(_fn("elementwise", "tk_embed_gather")(_code(table.dtype), _p(table), _p(ids), _p(resid),
                                                  n, h, v, _stream()), "embed_gather")
 
@@ -180,6 +238,8 @@ def add_rmsnorm(resid: torch.Tensor, delta: torch.Tensor | None, weight: torch.T
               "row-indexed rmsnorm cannot write the residual")
         write_resid = False
     is_f32, parts, stride = _partials(delta, resid.shape[0], h, out.dtype, "delta")
+    _note(f"{m}x{h}", m * h * (4 + (8 if write_resid else 0) + out.element_size())
+          + (0 if delta is None else parts * m * h * delta.element_size()))
     _check(_fn("elementwise", "tk_add_rmsnorm")(_code(out.dtype), _p(resid), _p(delta), is_f32, parts, stride,
                                                 _p(rows), _p(weight), _p(out), m, h, float(eps),
                                                 int(bool(write_resid)), _stream()), "add_rmsnorm")
@@ -227,6 +287,7 @@ def qknorm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor | None,
         _need(k_cache is not None and v_cache is not None and k_cache.dtype == q_out.dtype
               and v_cache.dtype == q_out.dtype, "cache dtype must match activations")
         _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
+    _note(f"{n}x{width}", n * width * (qkv.element_size() * parts + q_out.element_size()))
     _check(_fn("elementwise", "tk_qknorm_rope_store")(
         _code(q_out.dtype), _p(qkv), in_f32, parts, stride, _p(q_weight), _p(k_weight), _p(cos), _p(sin), _p(positions),
         _p(req_of_token), _p(block_tables), _p(q_out), _p(k_cache), _p(v_cache), n, num_heads,
@@ -239,6 +300,7 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _gpu(gate_up, out)
     n, two_i = gate_up.shape
     _need(two_i % 2 == 0 and out.shape == (n, two_i // 2) and out.dtype == gate_up.dtype, "silu_mul shapes disagree")
+    _note(f"{n}x{two_i // 2}", n * two_i * out.element_size() * 1.5)
     _check(_fn("elementwise", "tk_silu_mul")(_code(out.dtype), _p(gate_up), _p(out), n, two_i // 2,
                                              _stream()), "silu_mul")
 
@@ -252,6 +314,7 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     _need(w.shape[1] == k and out.shape == (m, n), f"gemm shapes disagree: {tuple(a.shape)} x {tuple(w.shape)}^T -> {tuple(out.shape)}")
     _need(a.dtype == w.dtype, "gemm inputs must share a dtype")
     _need(m <= 64 * 65535, "too many rows for one launch")
+    _note(f"{m}x{n}x{k}", (n * k + m * k) * a.element_size() + m * n * out.element_size(), 2.0 * m * n * k)
     _check(_fn("gemm_tiled", "tk_gemm_tiled")(_code(a.dtype), _code(out.dtype), _p(a), _p(w), _p(out),
                                               m, n, k, a.stride(0), w.stride(0), out.stride(0),
                                               _stream()), "gemm_tiled")
@@ -278,6 +341,7 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
         _need(1 < splits <= 64 and out.dtype == torch.float32 and out.shape == (splits, m, n) and out.is_contiguous(),
               "with splits the output is contiguous float32 [splits, M, N]")
         ldc, stride = n, m * n
+    _note(f"{m}x{n}x{k}", (n * k + m * k) * 2 + splits * m * n * out.element_size(), 2.0 * m * n * k)
     used = _fn("gemm_mfma", "tk_gemm_stream")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
                                               w.stride(0), ldc, splits, stride, _stream())
     if used < 1:
@@ -295,6 +359,7 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> N
     _need(a.dtype == w.dtype == out.dtype == torch.bfloat16, "the gated product is bfloat16")
     _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gated product needs M <= 64 and 16-byte aligned rows")
+    _note(f"{m}x{w.shape[0]}x{k}", (w.shape[0] * k + m * k) * 2 + m * w.shape[0], 2.0 * m * w.shape[0] * k)
     _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
                                                      w.stride(0), out.stride(0), _stream()), "gemm_stream_swiglu")
 
@@ -336,6 +401,7 @@ def gemm_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
     ws = _lt_workspace.get(a.device)
     if ws is None:
         ws = _lt_workspace[a.device] = torch.empty(LT_WORKSPACE_BYTES, dtype=torch.uint8, device=a.device)
+    _note(f"{m}x{n}x{k}", (n * k + m * k + m * n) * 2, 2.0 * m * n * k)
     status = _fn("blas_lt", "tk_lt_gemm")(_p(a), _p(w), _p(out), m, n, k, a.stride(0), w.stride(0), out.stride(0),
                                           _p(ws), ws.numel(), _lt_tune, _stream())
     if status == -2:
@@ -357,6 +423,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, row_tile
     _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "skinny product needs M <= 64 and 16-byte aligned rows")
     _need(row_tiles in (1, 2, 4) and 1 <= waves <= 16, "row_tiles in (1, 2, 4), waves in 1..16")
+    _note(f"{m}x{n}x{k}", (n * k + m * k) * 2 + m * n * out.element_size(), 2.0 * m * n * k)
     _check(_fn("gemm_mfma", "tk_gemm_skinny")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
                                               w.stride(0), out.stride(0), row_tiles, waves, _stream()), "gemm_skinny")
 
