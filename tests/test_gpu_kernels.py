@@ -72,7 +72,7 @@ def run_attention(dtype, nh, nkv, hd, ps, requests, *, window=None, poison=True,
 SHAPES = [
     (4, 2, 16, 8), (7, 1, 16, 16), (16, 8, 128, 16), (32, 8, 128, 16), (8, 2, 64, 32), (5, 5, 48, 16),
     (6, 2, 256, 16), (24, 2, 64, 16), (3, 1, 128, 16), (14, 2, 128, 16), (8, 2, 128, 64), (4, 4, 64, 128),
-    (2, 1, 128, 24),
+    (2, 1, 128, 24), (16, 1, 128, 16), (20, 2, 128, 32),
 ]
 MIXES = {
     "decode": [(48, 1), (15, 1), (0, 1), (300, 1), (16, 1)],

@@ -1,10 +1,12 @@
 // Paged causal attention on the matrix cores (bf16 in, float32 softmax and
 // accumulation) for head sizes 64 and 128 and page sizes 16, 32, 64, ... (powers of two).
 //
-// Decode tokens (attention_decode_kernel): one 64-lane wave owns one token, one kv
-// head and a range of that request's keys (a split); its 16 "columns" are the
-// query heads of the group.
-// Keys are taken 16 at a time (one MFMA tile, never across a page edge):
+// Decode tokens (attention_decode_kernel): a block of sixteen waves owns one token, one kv
+// head and a range of that request's keys (a split); the waves take contiguous shares
+// of the range and merge through LDS.  A wave's 16 "columns" are the query heads of the
+// group.  Keys are taken 16 at a time (one MFMA tile, never across a page edge); a tile's
+// keys are reloaded for the wave's next tile as soon as the scores are taken, its values
+// as soon as they are multiplied:
 //   S^T[key][col] = K[key][:] . Q[col][:]      v_mfma_f32_16x16x32_bf16, K rows as A
 //   P^T = exp2(S^T * c - m[col])               float32, one column per lane
 //   O^T[d][col] += V^T[d][key] * P^T[key][col] v_mfma_f32_16x16x16_bf16, V^T rows as A
@@ -13,7 +15,7 @@
 // are loaded straight from the pages (K page [nkv][hd/8][ps][8], V page
 // [nkv][hd/16][ps/4][16][4]) in contiguous 16- and 8-byte pieces.
 //
-// With more than one split the wave writes an unnormalised partial (o, m, l) and
+// With more than one split the block writes an unnormalised partial (o, m, l) and
 // a second kernel merges the splits of each (token, head).
 #include "common.h"
 
@@ -39,8 +41,12 @@ union Frag4 {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-template <int HD, int NSETS>
-__global__ __launch_bounds__(64) void attention_decode_kernel(
+constexpr int kDecodeWaves = 16;
+
+// WAVES: waves of a block (they share a split's keys and merge through LDS); D: tiles of
+// 16 keys a wave keeps in flight.
+template <int HD, int WAVES, int D>
+__global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
@@ -49,167 +55,185 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     int split_keys, int nh, int nkv, int ps, float scale_log2) {
   constexpr int KCH = HD / 32;  // 32-wide chunks of the head dim (QK^T steps)
   constexpr int DBL = HD / 16;  // 16-wide blocks of the head dim (PV outputs)
-  const int lane = threadIdx.x, col = lane & 15, kb = lane >> 4;
+  // LDS: the waves' accumulators of the group's heads [WAVES][G][HD], then their (m, l) [WAVES][16] each
+  extern __shared__ __attribute__((aligned(16))) float s_dyn[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, kb = lane >> 4;
   const int split = blockIdx.x, item = blockIdx.z;
   const int G = nh / nkv;
   const int kvh = blockIdx.y;
 
   const int n0 = item_token[item];
-  const int count = 1;
-  const int pos0 = positions[n0];
-  const int last_pos = pos0 + count - 1;
+  const int pos0 = positions[n0];  // the token's position: it sees keys 0 .. pos0
   const int k_begin = split * split_keys;
-  const int k_end = min(last_pos + 1, k_begin + split_keys);
-  if (k_begin >= k_end) return;
+  const int k_end = min(pos0 + 1, k_begin + split_keys);
+  if (k_begin >= k_end) return;  // the whole block: this split holds no key of the token
   const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
   const size_t page_elems = (size_t)nkv * HD * ps;
   const size_t head_off = (size_t)kvh * HD * ps;
 
-  // which (token, head) this lane's column is, per set
-  int c_token[NSETS], c_head[NSETS];
-  bool c_valid[NSETS];
-  const int c_pos = pos0;
-#pragma unroll
-  for (int s = 0; s < NSETS; ++s) {
-    c_token[s] = n0;
-    c_head[s] = kvh * G + s * 16 + col;
-    c_valid[s] = s * 16 + col < G;
-  }
+  // the split's tiles of 16 keys, in contiguous shares of the waves
+  const int tiles = (k_end - k_begin + 15) >> 4;
+  const int per = (tiles + WAVES - 1) / WAVES;
+  const int t_begin = wave * per, t_end = min(tiles, t_begin + per);
+
+  // this lane's column is query head `col` of the group
+  const int c_head = kvh * G + col;
+  const bool c_valid = col < G;
 
   // Q as B operand: lane (col, kb) holds Q[col][c*32 + kb*8 .. +8]
-  bf16x8 qreg[NSETS][KCH];
-#pragma unroll
-  for (int s = 0; s < NSETS; ++s) {
-    const bf16_t* qp = q + ((size_t)c_token[s] * nh + c_head[s]) * HD + kb * 8;
+  bf16x8 qreg[KCH];
+  {
+    const bf16_t* qp = q + ((size_t)n0 * nh + c_head) * HD + kb * 8;
 #pragma unroll
     for (int c = 0; c < KCH; ++c) {
       Frag8 f;
-      f.u = c_valid[s] ? *reinterpret_cast<const uint4*>(qp + c * 32) : make_uint4(0, 0, 0, 0);
-      qreg[s][c] = f.v;
+      f.u = c_valid ? *reinterpret_cast<const uint4*>(qp + c * 32) : make_uint4(0, 0, 0, 0);
+      qreg[c] = f.v;
     }
   }
 
-  float m_run[NSETS], l_run[NSETS];
-  float4v acc[NSETS][DBL];
+  float m_run = -INFINITY, l_run = 0.f;
+  float4v acc[DBL];
 #pragma unroll
-  for (int s = 0; s < NSETS; ++s) {
-    m_run[s] = -INFINITY;
-    l_run[s] = 0.f;
-#pragma unroll
-    for (int d = 0; d < DBL; ++d) acc[s][d] = float4v{0.f, 0.f, 0.f, 0.f};
+  for (int d = 0; d < DBL; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  Frag8 kreg[D][KCH];
+  Frag4 vreg[D][DBL];
+#define TK_TILE_ADDR(T_)                                                  \
+    const int c0_ = k_begin + (T_) * 16;                                    \
+    const int page_ = table[c0_ / ps];                                      \
+    const int off_ = c0_ % ps;
+#define TK_LOAD_K(SLOT_, T_)                                                                          \
+  {                                                                                                   \
+    TK_TILE_ADDR(T_)                                                                                  \
+    const bf16_t* kp_ = k_cache + (size_t)page_ * page_elems + head_off + (size_t)(off_ + col) * 8;   \
+    _Pragma("unroll") for (int c = 0; c < KCH; ++c) kreg[SLOT_][c].w = __builtin_nontemporal_load(    \
+        reinterpret_cast<const u32x4*>(kp_ + (size_t)(c * 4 + kb) * ps * 8));                         \
+  }
+  // V page [hd/16][ps/4][16][4]: lane (dim col, quad kb) of block d reads 8 bytes, the wave 512
+  // contiguous bytes
+#define TK_LOAD_V(SLOT_, T_)                                                                          \
+  {                                                                                                   \
+    TK_TILE_ADDR(T_)                                                                                  \
+    const bf16_t* vp_ =                                                                               \
+        v_cache + (size_t)page_ * page_elems + head_off + (size_t)((off_ >> 2) + kb) * 64 + col * 4;  \
+    _Pragma("unroll") for (int d = 0; d < DBL; ++d) vreg[SLOT_][d].w = __builtin_nontemporal_load(    \
+        reinterpret_cast<const u32x2*>(vp_ + (size_t)d * (ps >> 2) * 64));                            \
   }
 
-  Frag8 kreg[KCH];
-  Frag4 vreg[DBL];
-  auto load_tile = [&](int c0) {
-    const int page = table[c0 / ps];
-    const int off = c0 % ps;
-    const bf16_t* kp = k_cache + (size_t)page * page_elems + head_off + (size_t)(off + col) * 8;
 #pragma unroll
-    for (int c = 0; c < KCH; ++c)
-      kreg[c].w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp + (size_t)(c * 4 + kb) * ps * 8));
-    // V page [hd/16][ps/4][16][4]: lane (dim col, quad kb) of block d reads 8 bytes, the
-    // wave 512 contiguous bytes
-    const bf16_t* vp = v_cache + (size_t)page * page_elems + head_off + (size_t)((off >> 2) + kb) * 64 + col * 4;
-#pragma unroll
-    for (int d = 0; d < DBL; ++d)
-      vreg[d].w = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(vp + (size_t)d * (ps >> 2) * 64));
-  };
-
-  load_tile(k_begin);
-  for (int c0 = k_begin; c0 < k_end; c0 += 16) {
-    Frag8 kc[KCH];
-    Frag4 vc[DBL];
-#pragma unroll
-    for (int c = 0; c < KCH; ++c) kc[c] = kreg[c];
-#pragma unroll
-    for (int d = 0; d < DBL; ++d) vc[d] = vreg[d];
-    if (c0 + 16 < k_end) load_tile(c0 + 16);  // next tile's loads fly while this one computes
-
-    const bool edge = c0 + 15 > pos0;  // some key of this tile is hidden from some column
-    if (c0 + 15 > last_pos) {
-      // keys past the request's end may hold anything (NaN included): zero their values
-#pragma unroll
-      for (int d = 0; d < DBL; ++d) {
-        short4v t = vc[d].v;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (c0 + kb * 4 + i > last_pos) t[i] = 0;
-        vc[d].v = t;
-      }
+  for (int i = 0; i < D; ++i)
+    if (t_begin + i < t_end) {
+      TK_LOAD_K(i, t_begin + i)
+      TK_LOAD_V(i, t_begin + i)
     }
+
+  for (int t0 = t_begin; t0 < t_end; t0 += D) {
 #pragma unroll
-    for (int s = 0; s < NSETS; ++s) {
+    for (int i = 0; i < D; ++i) {
+      const int t = t0 + i;
+      if (t >= t_end) break;  // the same for every lane of the wave
+      const int c0 = k_begin + t * 16;
+      const bool edge = c0 + 15 > pos0;  // some key of this tile lies past the token's position
       float4v sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < KCH; ++c)
-        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kc[c].v, qreg[s][c], sc, 0, 0, 0);
+      for (int c = 0; c < KCH; ++c) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[i][c].v, qreg[c], sc, 0, 0, 0);
+      // the slot's keys have been used: its next tile's keys fly while the others are multiplied
+      if (t + D < t_end) TK_LOAD_K(i, t + D)
       float sv[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        sv[i] = sc[i] * scale_log2;
-        if (edge) {
-          const int key = c0 + kb * 4 + i;
-          if (key > c_pos || key > last_pos) sv[i] = -INFINITY;
-        }
+      for (int e = 0; e < 4; ++e) {
+        sv[e] = sc[e] * scale_log2;
+        if (edge && c0 + kb * 4 + e > pos0) sv[e] = -INFINITY;
       }
       float tmax = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-      const float m_new = fmaxf(m_run[s], tmax);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fast_exp2(m_run[s] - m_safe);
-      m_run[s] = m_new;
-      float p[4];
+      const float m_new = fmaxf(m_run, tmax);  // finite: a tile's first key is never past the position
+      const float alpha = fast_exp2(m_run - m_new);
+      m_run = m_new;
+      float pr[4];
       float psum = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        p[i] = fast_exp2(sv[i] - m_safe);
-        psum += p[i];
+      for (int e = 0; e < 4; ++e) {
+        pr[e] = fast_exp2(sv[e] - m_new);
+        psum += pr[e];
       }
-      l_run[s] = l_run[s] * alpha + psum;
+      l_run = l_run * alpha + psum;
       Frag4 pb;
-      pb.u = make_uint2(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]));
+      pb.u = make_uint2(pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3]));
 #pragma unroll
       for (int d = 0; d < DBL; ++d) {
-        float4v a = acc[s][d];
+        short4v tv = vreg[i][d].v;
+        if (edge) {
+          // keys past the request's end may hold anything (NaN included): zero their values
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (c0 + kb * 4 + e > pos0) tv[e] = 0;
+        }
+        float4v a = acc[d];
         a[0] *= alpha;
         a[1] *= alpha;
         a[2] *= alpha;
         a[3] *= alpha;
-        acc[s][d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vc[d].v, pb.v, a, 0, 0, 0);
+        acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(tv, pb.v, a, 0, 0, 0);
       }
+      if (t + D < t_end) TK_LOAD_V(i, t + D)
     }
   }
+#undef TK_LOAD_V
+#undef TK_LOAD_K
+#undef TK_TILE_ADDR
 
-  // acc[s][d][i] = O^T[dim = d*16 + kb*4 + i][col]
+  // The waves' shares meet in LDS: acc[d][e] = O^T[dim = d*16 + kb*4 + e][col], unnormalised,
+  // relative to the wave's own maximum m_run (-inf and zeros for a wave without a tile).
+  float* s_acc = s_dyn;                         // [WAVES][G][HD]
+  float* s_m = s_dyn + (size_t)WAVES * G * HD;  // [WAVES][16]
+  float* s_l = s_m + WAVES * 16;                // [WAVES][16]
+  float l = l_run;
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  if (c_valid) {
+    float* mine = s_acc + ((size_t)wave * G + col) * HD + kb * 4;
 #pragma unroll
-  for (int s = 0; s < NSETS; ++s) {
-    float l = l_run[s];
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
-    if (!c_valid[s]) continue;
-    const size_t row = (size_t)c_token[s] * nh + c_head[s];
-    const size_t prow = (size_t)item * nh + c_head[s];  // partials are indexed by item, not token
-    if (nsplit == 1) {
-      const float inv = 1.f / l;
-      bf16_t* op = out + row * HD + kb * 4;
+    for (int d = 0; d < DBL; ++d)
+      *reinterpret_cast<float4*>(mine + d * 16) = make_float4(acc[d][0], acc[d][1], acc[d][2], acc[d][3]);
+  }
+  if (kb == 0) {
+    s_m[wave * 16 + col] = m_run;
+    s_l[wave * 16 + col] = l;
+  }
+  __syncthreads();
+  // thread t sums four dims of one head over the waves
+  const int t = threadIdx.x;
+  if (t >= G * (HD / 4)) return;
+  const int head = t / (HD / 4), dim = (t % (HD / 4)) * 4;
+  float m_all = s_m[head];
 #pragma unroll
-      for (int d = 0; d < DBL; ++d) {
-        *reinterpret_cast<uint2*>(op + d * 16) =
-            make_uint2(pack_bf16x2(acc[s][d][0] * inv, acc[s][d][1] * inv),
-                       pack_bf16x2(acc[s][d][2] * inv, acc[s][d][3] * inv));
-      }
-    } else {
-      float* po = part_o + (prow * nsplit + split) * HD + kb * 4;
+  for (int w = 1; w < WAVES; ++w) m_all = fmaxf(m_all, s_m[w * 16 + head]);  // finite: wave 0 has a tile
+  float l_all = 0.f;
+  float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-      for (int d = 0; d < DBL; ++d)
-        *reinterpret_cast<float4*>(po + d * 16) =
-            make_float4(acc[s][d][0], acc[s][d][1], acc[s][d][2], acc[s][d][3]);
-      if (kb == 0) {
-        part_ml[(prow * nsplit + split) * 2] = m_run[s];
-        part_ml[(prow * nsplit + split) * 2 + 1] = l;
-      }
+  for (int w = 0; w < WAVES; ++w) {
+    const float weight = fast_exp2(s_m[w * 16 + head] - m_all);  // exp2(-inf) = 0 for a wave without a tile
+    l_all = fmaf(weight, s_l[w * 16 + head], l_all);
+    const float4 v = *reinterpret_cast<const float4*>(s_acc + ((size_t)w * G + head) * HD + dim);
+    o.x = fmaf(weight, v.x, o.x);
+    o.y = fmaf(weight, v.y, o.y);
+    o.z = fmaf(weight, v.z, o.z);
+    o.w = fmaf(weight, v.w, o.w);
+  }
+  const size_t row = (size_t)n0 * nh + kvh * G + head;
+  const size_t prow = ((size_t)item * nh + kvh * G + head) * nsplit + split;  // partials are indexed by item, not token
+  if (nsplit == 1) {
+    const float inv = 1.f / l_all;
+    *reinterpret_cast<uint2*>(out + row * HD + dim) =
+        make_uint2(pack_bf16x2(o.x * inv, o.y * inv), pack_bf16x2(o.z * inv, o.w * inv));
+  } else {
+    *reinterpret_cast<float4*>(part_o + prow * HD + dim) = o;
+    if (dim == 0) {
+      part_ml[prow * 2] = m_all;
+      part_ml[prow * 2 + 1] = l_all;
     }
   }
 }
@@ -549,18 +573,33 @@ static int launch_prefill(const void* q, const void* k_cache, const void* v_cach
   return launch_status();
 }
 
-template <int HD, int NSETS>
+template <int HD>
 static int launch(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                   int max_pages, const int* positions, const int* req_of_token,
                   const int* item_token, const int* item_count, int num_items, void* out,
                   float* part_o, float* part_ml, int nsplit, int split_keys, int nh, int nkv, int ps,
                   float scale, hipStream_t stream) {
-  const int G = nh / nkv;
   dim3 grid(nsplit, nkv, num_items);
-  attention_decode_kernel<HD, NSETS><<<grid, 64, 0, stream>>>(
-      (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
-      positions, req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit,
-      split_keys, nh, nkv, ps, scale * 1.4426950408889634f);
+  const int G = nh / nkv;
+  // sixteen waves a block and one tile a wave in flight measured best at every batch size
+  // (four or eight waves with two tiles: 12 % slower at batch 64, 15 % at batch 8)
+  const size_t lds = (size_t)(kDecodeWaves * G * HD + 2 * kDecodeWaves * 16) * 4;
+  if (lds > 160 * 1024) return -2;
+  if (lds > 48 * 1024) {  // beyond the default limit of dynamic LDS (groups of 7 heads and more)
+    static bool raised = false;  // per template instance
+    if (!raised) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_kernel<HD, kDecodeWaves, 1>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) {
+        (void)hipGetLastError();
+        return -2;
+      }
+      raised = true;
+    }
+  }
+  attention_decode_kernel<HD, kDecodeWaves, 1><<<grid, kDecodeWaves * 64, lds, stream>>>(
+          (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages, positions,
+          req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps,
+          scale * 1.4426950408889634f);
   if (nsplit > 1) {
     dim3 mgrid(num_items, nh);
     attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token, nullptr,
@@ -569,11 +608,14 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
   return launch_status();
 }
 
-// mode 0: heads (every item is one decode token; item_count is ignored)
+// mode 0: heads (every item is one decode token; item_count is ignored; split_keys is a multiple of
+//         16 * tk_attention_decode_waves(), a tile for every wave of a block)
 // mode 1: tokens (item = up to 16 consecutive tokens of one request; with nsplit > 1 split_keys
 //         is a multiple of 64 and the partial buffers hold 16 rows per item)
 // mode 2: tokens, every tile over a long context (same results; the kernel built for four waves a SIMD)
 // Returns -2 if this shape is not instantiated (the caller uses the generic kernel).
+TK_API int tk_attention_decode_waves() { return kDecodeWaves; }
+
 TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const void* v_cache,
                              const int* block_tables, int max_pages, const int* positions,
                              const int* req_of_token, const int* item_token, const int* item_count,
@@ -590,8 +632,8 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
       num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream
   if (mode == 0) {
     if (G > 16) return -2;
-    if (hd == 128) return launch<128, 1>(TK_ARGS);
-    if (hd == 64) return launch<64, 1>(TK_ARGS);
+    if (hd == 128) return launch<128>(TK_ARGS);
+    if (hd == 64) return launch<64>(TK_ARGS);
     return -2;
   }
   // the keys of a tile may be split too: in whole stages of 64 keys, sixteen partial rows a tile

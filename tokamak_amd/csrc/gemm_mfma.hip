@@ -219,103 +219,121 @@ TK_API int tk_gemm_skinny(int out_dtype, const void* A, const void* W, void* C, 
 constexpr int SBK = 256;        // k per chunk
 constexpr int SLD = SBK + 8;    // LDS row stride in elements
 
-// GATED: W is [2N, K], gate rows then up rows; the block owns 32 output columns, waves
-// 0,1 their gate rows and waves 2,3 the matching up rows, and the result is
-// silu(gate) * up [M, N] (the SwiGLU feed-forward's first half in one kernel).
-template <int MT, typename TO, bool GATED>
-__global__ __launch_bounds__(256) void gemm_stream_kernel(
+// GATED: W is [2N, K], gate rows then up rows; the block owns 8*WAVES output columns, the
+// first half of its waves their gate rows and the second half the matching up rows, and
+// the result is silu(gate) * up [M, N] (the SwiGLU feed-forward's first half in one kernel).
+//
+// WAVES (4 or 8): waves a block; they share the activations' chunk, so 8 waves read it
+// once per 128 weight rows (what pays from 33 rows of activations on: +10 % at 64 rows).
+// A second chunk of weights in flight per wave was measured too and gained nothing: at 64
+// rows the kernel is held by LDS traffic (seven bytes through LDS per byte of weights),
+// at 16 rows and fewer by the launch and drain of blocks that live for a few microseconds.
+template <int MT, typename TO, bool GATED, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TO* __restrict__ C, int M, int N,
     int K, long lda, long ldw, long ldc, int chunks_per_split, long split_stride) {
-  __shared__ __attribute__((aligned(16))) bf16_t ws[4][16][SLD];
+  constexpr int THREADS = WAVES * 64;
+  constexpr int XP = 16 * MT * 32 / THREADS;  // 16-byte pieces of the activations a thread loads per chunk
+  static_assert(XP * THREADS == 16 * MT * 32, "the activations' chunk divides among the threads");
+  constexpr int HALF = WAVES / 2;
+  __shared__ __attribute__((aligned(16))) bf16_t ws[WAVES][16][SLD];
   __shared__ __attribute__((aligned(16))) bf16_t xs[16 * MT][SLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, kb = lane >> 4;
   const int row_block = blockIdx.x, split = blockIdx.y;
   // n_wave: first output column of this wave; w_first/w_limit: its weight rows
-  const int n_wave = GATED ? row_block * 32 + (wave & 1) * 16 : row_block * 64 + wave * 16;
-  const int w_first = (GATED && wave >= 2) ? N + n_wave : n_wave;
-  const int w_limit = (GATED && wave >= 2) ? 2 * N : N;
+  const bool up_wave = GATED && wave >= HALF;
+  const int n_wave = GATED ? row_block * (16 * HALF) + (wave % HALF) * 16 : row_block * (16 * WAVES) + wave * 16;
+  const int w_first = up_wave ? N + n_wave : n_wave;
+  const int w_limit = up_wave ? 2 * N : N;
   const int total_chunks = (K + SBK - 1) / SBK;
   const int c_begin = split * chunks_per_split;
   const int c_end = min(total_chunks, c_begin + chunks_per_split);
 
   // loader roles: W piece i of this lane = row 2i + lane/32, 16-byte column lane%32
   const int w_col = (lane & 31) * 8, w_row0 = lane >> 5;
-  // X pieces of this thread: piece p = i*256 + tid -> row p/32, column p%32
+  // X pieces of this thread: piece p = i*THREADS + tid -> row p/32, column p%32
   const int x_col = (tid & 31) * 8, x_row0 = tid >> 5;
 
   u32x4 wreg[8];
-  u32x4 xreg[2 * MT];
+  u32x4 xreg[XP];
   const u32x4 zero = {0u, 0u, 0u, 0u};
   // Rows are clamped into the matrices (rows past N or M are computed from a valid
-  // row and never stored); only a piece past K is zeroed, after an unconditional
-  // load from k = 0, so the loads of a chunk are all in flight together.
+  // row and never stored).  A piece past K is read at the row's last piece instead and
+  // meets zeros: the activations' pieces past K are zeroed on their way into LDS.
   const bf16_t* wrow[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) wrow[i] = W + (size_t)min(w_first + 2 * i + w_row0, w_limit - 1) * ldw;
-  const bf16_t* xrow[2 * MT];
+  const bf16_t* xrow[XP];
 #pragma unroll
-  for (int i = 0; i < 2 * MT; ++i) xrow[i] = A + (size_t)min(i * 8 + x_row0, M - 1) * lda;
-  auto fetch = [&](int c) {
-    const int k0 = c * SBK;
-    const bool kw = k0 + w_col < K, kx = k0 + x_col < K;
-    const int wo = kw ? k0 + w_col : 0, xo = kx ? k0 + x_col : 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i)  // weights are read once: streaming loads leave the caches to the activations
-      wreg[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[i] + wo));
-#pragma unroll
-    for (int i = 0; i < 2 * MT; ++i) xreg[i] = *reinterpret_cast<const u32x4*>(xrow[i] + xo);
-    if (k0 + SBK > K) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) wreg[i] = kw ? wreg[i] : zero;
-#pragma unroll
-      for (int i = 0; i < 2 * MT; ++i) xreg[i] = kx ? xreg[i] : zero;
-    }
-  };
+  for (int i = 0; i < XP; ++i) xrow[i] = A + (size_t)min(i * (THREADS / 32) + x_row0, M - 1) * lda;
 
   float4v acc[MT];
 #pragma unroll
   for (int j = 0; j < MT; ++j) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  if (c_begin < c_end) fetch(c_begin);
-  for (int c = c_begin; c < c_end; ++c) {
-    __syncthreads();  // the previous chunk's fragments have been read
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-      *reinterpret_cast<u32x4*>(&ws[wave][2 * i + w_row0][w_col]) = wreg[i];
-#pragma unroll
-    for (int i = 0; i < 2 * MT; ++i)
-      *reinterpret_cast<u32x4*>(&xs[i * 8 + x_row0][x_col]) = xreg[i];
-    __syncthreads();
-    if (c + 1 < c_end) fetch(c + 1);  // in flight while this chunk is multiplied
-#pragma unroll
-    for (int s = 0; s < SBK / 32; ++s) {
-      Frag8 wf;
-      wf.u = *reinterpret_cast<const uint4*>(&ws[wave][r][s * 32 + kb * 8]);
-#pragma unroll
-      for (int j = 0; j < MT; ++j) {
-        Frag8 xf;
-        xf.u = *reinterpret_cast<const uint4*>(&xs[j * 16 + r][s * 32 + kb * 8]);
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf.v, acc[j], 0, 0, 0);
-      }
-    }
+#define TK_FETCH_W(C_)                                                                              \
+  {                                                                                                 \
+    const int wo_ = min((C_) * SBK + w_col, K - 8);                                                 \
+    _Pragma("unroll") for (int i = 0; i < 8; ++i) /* weights are read once: streaming loads */      \
+        wreg[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[i] + wo_));        \
   }
+#define TK_FETCH_X(C_)                                                                              \
+  {                                                                                                 \
+    const int xo_ = min((C_) * SBK + x_col, K - 8);                                                 \
+    _Pragma("unroll") for (int i = 0; i < XP; ++i)                                                  \
+        xreg[i] = *reinterpret_cast<const u32x4*>(xrow[i] + xo_);                                   \
+  }
+  // One chunk: park the registers in LDS, start the next chunk's loads into them, multiply.
+#define TK_CHUNK(C_)                                                                                \
+  {                                                                                                 \
+    __syncthreads(); /* the previous chunk's fragments have been read */                            \
+    _Pragma("unroll") for (int i = 0; i < 8; ++i)                                                   \
+        *reinterpret_cast<u32x4*>(&ws[wave][2 * i + w_row0][w_col]) = wreg[i];                      \
+    {                                                                                               \
+      const bool inside_ = (C_) * SBK + x_col < K;                                                  \
+      _Pragma("unroll") for (int i = 0; i < XP; ++i)                                                \
+          *reinterpret_cast<u32x4*>(&xs[i * (THREADS / 32) + x_row0][x_col]) = inside_ ? xreg[i] : zero; \
+    }                                                                                               \
+    __syncthreads();                                                                                \
+    if ((C_) + 1 < c_end) TK_FETCH_W((C_) + 1)                                                      \
+    if ((C_) + 1 < c_end) TK_FETCH_X((C_) + 1)                                                      \
+    _Pragma("unroll") for (int s = 0; s < SBK / 32; ++s) {                                          \
+      Frag8 wf;                                                                                     \
+      wf.u = *reinterpret_cast<const uint4*>(&ws[wave][r][s * 32 + kb * 8]);                        \
+      _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                              \
+        Frag8 xf;                                                                                   \
+        xf.u = *reinterpret_cast<const uint4*>(&xs[j * 16 + r][s * 32 + kb * 8]);                   \
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf.v, acc[j], 0, 0, 0);              \
+      }                                                                                             \
+    }                                                                                               \
+  }
+
+  if (c_begin < c_end) {
+    TK_FETCH_W(c_begin)
+    TK_FETCH_X(c_begin)
+  }
+  for (int c = c_begin; c < c_end; ++c) TK_CHUNK(c)
+#undef TK_CHUNK
+#undef TK_FETCH_X
+#undef TK_FETCH_W
 
   // With several splits, split s writes its partial sums to C + s * split_stride; whoever
   // reads C next adds the splits (in split order, so the sum is deterministic).
   C += (size_t)split * split_stride;
 
   if (GATED) {
-    float* up = reinterpret_cast<float*>(&xs[0][0]);  // [2 up waves][MT][64 lanes][4]
-    __syncthreads();                                   // the last chunk's fragments have been read
-    if (wave >= 2) {
+    float* up = reinterpret_cast<float*>(&ws[0][0][0]);  // [HALF up waves][MT][64 lanes][4]
+    static_assert(sizeof(ws) >= sizeof(float) * HALF * MT * 64 * 4, "the exchange fits the weights' tiles");
+    __syncthreads();                                      // the last chunk's fragments have been read
+    if (wave >= HALF) {
 #pragma unroll
       for (int j = 0; j < MT; ++j)
-        *reinterpret_cast<float4*>(up + ((size_t)((wave - 2) * MT + j) * 64 + lane) * 4) =
+        *reinterpret_cast<float4*>(up + ((size_t)((wave - HALF) * MT + j) * 64 + lane) * 4) =
             make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
     }
     __syncthreads();
-    if (wave >= 2) return;
+    if (wave >= HALF) return;
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
       const float4 u = *reinterpret_cast<const float4*>(up + ((size_t)(wave * MT + j) * 64 + lane) * 4);
@@ -339,14 +357,15 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(
   }
 }
 
-template <typename TO, bool GATED>
-static int launch_stream(const void* A, const void* W, void* C, int M, int N, int K, long lda,
-                         long ldw, long ldc, int chunks_per_split, int KS, long split_stride,
-                         hipStream_t stream) {
-  dim3 grid(GATED ? (N + 31) / 32 : (N + 63) / 64, KS);
+template <typename TO, bool GATED, int WAVES>
+static int launch_stream_shape(const void* A, const void* W, void* C, int M, int N, int K, long lda,
+                               long ldw, long ldc, int chunks_per_split, int KS, long split_stride,
+                               hipStream_t stream) {
+  const int cols = GATED ? 8 * WAVES : 16 * WAVES;
+  dim3 grid((N + cols - 1) / cols, KS);
   const int mt = (M + 15) / 16;
 #define TK_STREAM(MT_)                                                                          \
-  gemm_stream_kernel<MT_, TO, GATED><<<grid, 256, 0, stream>>>(                                 \
+  gemm_stream_kernel<MT_, TO, GATED, WAVES><<<grid, WAVES * 64, 0, stream>>>(            \
       (const bf16_t*)A, (const bf16_t*)W, (TO*)C, M, N, K, lda, ldw, ldc, chunks_per_split,     \
       split_stride)
   if (mt == 1) TK_STREAM(1);
@@ -357,30 +376,39 @@ static int launch_stream(const void* A, const void* W, void* C, int M, int N, in
   return launch_status();
 }
 
+// waves: 4 or 8 a block.
+template <typename TO, bool GATED>
+static int launch_stream(int waves, const void* A, const void* W, void* C, int M, int N, int K,
+                         long lda, long ldw, long ldc, int cps, int KS, long split_stride, hipStream_t stream) {
+  if (waves >= 8)
+    return launch_stream_shape<TO, GATED, 8>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, stream);
+  return launch_stream_shape<TO, GATED, 4>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, stream);
+}
+
 // out_dtype: 0 float32, 1 bfloat16.  M <= 64; K a multiple of 8; rows 16-byte aligned.
-// splits: shares of K.  With splits > 1 the output must be float32 and C holds
+// waves: 4 or 8 waves a block.  splits: shares of K.  With splits > 1 the output must be float32 and C holds
 // `splits` partial results, split_stride elements apart, that the reader adds.
 // Returns the number of splits actually used (<= splits; no split is empty), or < 0.
 TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, int M, int N, int K,
-                          long lda, long ldw, long ldc, int splits, long split_stride,
+                          long lda, long ldw, long ldc, int splits, long split_stride, int waves,
                           hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535) return -1;
+  if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535) return -1;
   if (splits > 1 && out_dtype != 0) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
   const int cps = (total_chunks + splits - 1) / splits;
   const int ks = (total_chunks + cps - 1) / cps;
   int status = -1;
-  if (out_dtype == 0) status = launch_stream<float, false>(A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
-  if (out_dtype == 1) status = launch_stream<bf16_t, false>(A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
+  if (out_dtype == 0) status = launch_stream<float, false>(waves, A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
+  if (out_dtype == 1) status = launch_stream<bf16_t, false>(waves, A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
   return status == 0 ? ks : (status > 0 ? -status : status);
 }
 
 // C[M, N] = silu(A W_gate^T) * (A W_up^T) with W = [W_gate; W_up] of 2N rows; bfloat16 out.
 TK_API int tk_gemm_stream_swiglu(const void* A, const void* W, void* C, int M, int N, int K, long lda,
-                                 long ldw, long ldc, hipStream_t stream) {
+                                 long ldw, long ldc, int waves, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K <= 0 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
+  if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
-  return launch_stream<bf16_t, true>(A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0, stream);
+  return launch_stream<bf16_t, true>(waves, A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0, stream);
 }

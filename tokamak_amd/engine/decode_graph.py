@@ -26,6 +26,18 @@ def pow2_at_least(n: int, floor: int) -> int:
     return v
 
 
+def quarter_octave_at_least(n: int, floor: int) -> int:
+    """The smallest of floor, 1.25 floor, 1.5 floor, 1.75 floor, 2 floor, 2.5 floor, ...
+    that is >= n: four buckets an octave, so a bucket overshoots by a quarter at most."""
+    v = floor
+    while 2 * v < n:
+        v *= 2
+    if n <= v:
+        return v
+    step = v // 4
+    return v + -(-(n - v) // step) * step
+
+
 class DecodeGraph:
     """One recorded decode shape.
 

@@ -18,7 +18,7 @@ from tokamak_amd.cache.manager import CacheManager, OutOfSlotsError
 from tokamak_amd.cache.pages import OutOfPagesError
 from tokamak_amd.config.registry import load_model_description
 from tokamak_amd.engine.batch import StepBatch, StepSpan, batch_from_device, pack_batch
-from tokamak_amd.engine.decode_graph import DecodeGraph, pow2_at_least
+from tokamak_amd.engine.decode_graph import DecodeGraph, pow2_at_least, quarter_octave_at_least
 from tokamak_amd.engine.model import LayeredModel
 from tokamak_amd.engine.storage import CacheStorage
 from tokamak_amd.kernels import ops
@@ -223,7 +223,8 @@ class ModelRunner:
             s.want = [0]            # the captured step computes every row's logits
         widths = [pow2_at_least(max(len(s.tables[g]) for s in spans), 16) for g in range(self.num_groups)]
         packed = pack_batch(spans, self.num_groups, fixed_widths=widths)
-        packed.max_decode_len = pow2_at_least(packed.max_decode_len, 256)
+        # the longest context fixes how the attention kernel splits the keys: bucketed, four an octave
+        packed.max_decode_len = quarter_octave_at_least(packed.max_decode_len, 256)
         key = (len(spans), tuple(widths), packed.max_decode_len)
         graph = self._graphs.pop(key, None)
         if graph is None:

@@ -7,9 +7,8 @@ import torch
 from tokamak_amd.kernels import ops
 
 MFMA_HEAD_DIMS = (64, 128)
-SPLIT_KEYS = 256          # fewest keys a split of a decode token's context holds
+DECODE_WAVES = 16           # waves of a decode block (csrc/attention_mfma.hip: kDecodeWaves)
 TARGET_DECODE_WAVES = 4096  # waves wanted in flight; beyond that splits only cost a merge
-FEW_DECODE_WAVES = 512      # below this many waves the splits are halved again
 TILE_SPLIT_BELOW_BLOCKS = 256   # a portion with fewer blocks than this has its keys split ...
 TILE_SPLIT_MIN_KEYS = 512       # ... into pieces no shorter than this
 TARGET_TILE_BLOCKS = 1024
@@ -22,17 +21,16 @@ def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
 
 
 def decode_split(num_decode: int, num_kv_heads: int, max_len: int) -> tuple[int, int]:
-    """(keys per split, number of splits) for the decode tokens of a step: as few
-    splits as fill the GPU (one wave per request, kv head and split), never
-    shorter than SPLIT_KEYS; half that when even so the waves are few (one or two
-    requests: the walk over a split's keys is then pure latency, and shorter walks
-    win more than the larger merge costs)."""
-    heads = num_decode * num_kv_heads
-    keys = SPLIT_KEYS if heads * -(-max_len // SPLIT_KEYS) >= FEW_DECODE_WAVES else SPLIT_KEYS // 2
-    most = max(1, -(-max_len // keys))
-    nsplit = min(most, max(1, -(-TARGET_DECODE_WAVES // heads)))
-    split = -(-max_len // nsplit)
-    split = -(-split // 16) * 16
+    """(keys per split, number of splits) for the decode tokens of a step.  A block of
+    DECODE_WAVES waves walks one split of one request and kv head, every wave a share of
+    it; the splits of a token are merged by a second kernel.  As few splits as put
+    TARGET_DECODE_WAVES waves on the GPU: more only add to the merge, and with one split
+    there is no merge.  A split is a whole number of 16 keys for every wave."""
+    pairs = max(1, num_decode * num_kv_heads)
+    least = 16 * DECODE_WAVES
+    most = max(1, -(-max_len // least))
+    nsplit = min(most, max(1, -(-TARGET_DECODE_WAVES // (DECODE_WAVES * pairs))))
+    split = -(-(-(-max_len // nsplit)) // least) * least
     return split, max(1, -(-max_len // split))
 
 

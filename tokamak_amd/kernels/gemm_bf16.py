@@ -38,9 +38,9 @@ def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
     return row_tiles, waves
 
 
-def stream_splits(n: int, k: int) -> int:
+def stream_splits(n: int, k: int, m: int = 1) -> int:
     """Shares of K for the LDS-staged kernel so that enough blocks exist."""
-    blocks = -(-n // 64)
+    blocks = -(-n // (16 * ops.stream_waves(m)))
     chunks = -(-k // 256)
     return max(1, min(chunks // 2, -(-STREAM_TARGET_BLOCKS // blocks), 64))
 
@@ -61,7 +61,7 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype, allow_pa
     dev = x.device
     if skinny_fits(x, weight) and (m <= SKINNY_MAX_ROWS or out_dtype == torch.float32):
         if m <= SKINNY_MAX_ROWS and allow_partials:
-            splits = stream_splits(n, k)
+            splits = stream_splits(n, k, m)
             if splits > 1:
                 out = torch.empty((splits, m, n), dtype=torch.float32, device=dev)
                 used = ops.gemm_stream(x, weight, out, splits=splits)

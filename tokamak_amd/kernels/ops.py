@@ -92,9 +92,9 @@ _SIGS = {
     },
     "gemm_mfma": {
         "tk_gemm_stream": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
-                           c_long, c_int, c_long, c_void_p],
+                           c_long, c_int, c_long, c_int, c_void_p],
         "tk_gemm_stream_swiglu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long,
-                                  c_void_p],
+                                  c_int, c_void_p],
         "tk_gemm_skinny": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                            c_long, c_int, c_int, c_void_p],
     },
@@ -320,9 +320,16 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
                                               _stream()), "gemm_tiled")
 
 
-def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: int = 1) -> int:
+def stream_waves(rows: int) -> int:
+    """Waves a block of the streaming product: from 33 rows of activations on, eight waves
+    share a chunk of them (the block then owns 128 weight rows), else four."""
+    return 8 if rows > 32 else 4
+
+
+def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: int = 1, waves: int = 0) -> int:
     """out = a[M, K] @ w[N, K]^T for M <= 64 with the LDS-staged weight-streaming
-    MFMA kernel.  ``splits == 1``: out is [M, N], bfloat16 or float32.  More:
+    MFMA kernel (``waves``: 4 or 8 waves a block; 0 chooses by M).  ``splits == 1``: out is
+    [M, N], bfloat16 or float32.  More:
     out is float32 [splits, M, N] and receives partial sums; returns how many of
     them were written (the reader adds out[:returned])."""
     for t in (a, w):
@@ -331,7 +338,7 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
     n = w.shape[0]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "the streaming product takes bfloat16 inputs")
     _need(w.shape[1] == k, "gemm shapes disagree")
-    _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+    _need(0 < m <= 64 and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "streaming product needs M <= 64 and 16-byte aligned rows")
     _need(out.is_cuda and out.stride(-1) == 1, "output must be a GPU tensor with unit inner stride")
     if splits == 1:
@@ -343,13 +350,13 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
         ldc, stride = n, m * n
     _note(f"{m}x{n}x{k}", (n * k + m * k) * 2 + splits * m * n * out.element_size(), 2.0 * m * n * k)
     used = _fn("gemm_mfma", "tk_gemm_stream")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
-                                              w.stride(0), ldc, splits, stride, _stream())
+                                              w.stride(0), ldc, splits, stride, waves or stream_waves(m), _stream())
     if used < 1:
         raise KernelError(f"gemm_stream failed with status {used}")
     return used
 
 
-def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, waves: int = 0) -> None:
     """out[M, I] = silu(a @ w[:I]^T) * (a @ w[I:]^T) for M <= 64: the gate and up
     projections and the SiLU product in one weight-streaming kernel (bfloat16)."""
     for t in (a, w, out):
@@ -357,11 +364,11 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> N
     m, k = a.shape
     _need(w.shape[0] % 2 == 0 and w.shape[1] == k and out.shape == (m, w.shape[0] // 2), "gated product shapes disagree")
     _need(a.dtype == w.dtype == out.dtype == torch.bfloat16, "the gated product is bfloat16")
-    _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+    _need(0 < m <= 64 and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gated product needs M <= 64 and 16-byte aligned rows")
     _note(f"{m}x{w.shape[0]}x{k}", (w.shape[0] * k + m * k) * 2 + m * w.shape[0], 2.0 * m * w.shape[0] * k)
     _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
-                                                     w.stride(0), out.stride(0), _stream()), "gemm_stream_swiglu")
+                                                     w.stride(0), out.stride(0), waves or stream_waves(m), _stream()), "gemm_stream_swiglu")
 
 
 LT_WORKSPACE_BYTES = 128 << 20
@@ -420,7 +427,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, row_tile
     n = w.shape[0]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "the skinny product takes bfloat16 inputs")
     _need(w.shape[1] == k and out.shape == (m, n), "gemm shapes disagree")
-    _need(0 < m <= 64 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+    _need(0 < m <= 64 and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "skinny product needs M <= 64 and 16-byte aligned rows")
     _need(row_tiles in (1, 2, 4) and 1 <= waves <= 16, "row_tiles in (1, 2, 4), waves in 1..16")
     _note(f"{m}x{n}x{k}", (n * k + m * k) * 2 + m * n * out.element_size(), 2.0 * m * n * k)
@@ -463,7 +470,8 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     request ("tokens_dense": the same, with the kernel variant for tiles that all
     walk a long context).  With ``num_splits`` > 1 the keys of an item are cut into pieces of
     ``split_keys`` (a multiple of 16; of 64 in "tokens" mode), each its own block, and a
-    second kernel merges the pieces.  Returns False (nothing launched) if the shape
+    second kernel merges the pieces (in "heads" mode the sixteen waves of a block share a piece, so
+    ``split_keys`` is a multiple of 256).  Returns False (nothing launched) if the shape
     is not instantiated."""
     _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, item_token, item_count, out)
     n = positions.numel()
@@ -478,6 +486,7 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
           and item_token.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
     _need(item_token.numel() >= num_items and 0 < num_items <= 65535, "bad item list")
     _need(mode in ("heads", "tokens", "tokens_dense"), "mode is heads, tokens or tokens_dense")
+    _need(mode != "heads" or num_splits == 1 or split_keys % 256 == 0, "heads mode splits keys in multiples of 256")
     if mode != "heads":
         _need(item_count is not None and item_count.dtype == torch.int32 and item_count.numel() >= num_items,
               "tokens mode needs item counts")
