@@ -284,20 +284,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
     _Pragma("unroll") for (int i = 0; i < XP; ++i)                                                  \
         xreg[i] = *reinterpret_cast<const u32x4*>(xrow[i] + xo_);                                   \
   }
+  // Blocks walk their chunks of K in rotated order (block b starts b chunks in): all blocks
+  // start together, and in step they would all read the same 512-byte window of their rows,
+  // 8 KB apart, which lands on a few memory channels only.
+  const int nchunks = c_end - c_begin;
+  const int rot = nchunks > 0 ? (int)(blockIdx.x % (unsigned)nchunks) : 0;
+  auto chunk_at = [&](int i) {
+    const int j = i + rot;
+    return c_begin + (j >= nchunks ? j - nchunks : j);
+  };
   // One chunk: park the registers in LDS, start the next chunk's loads into them, multiply.
-#define TK_CHUNK(C_)                                                                                \
+#define TK_CHUNK(I_)                                                                                \
   {                                                                                                 \
+    const int cur_ = chunk_at(I_);                                                                  \
     __syncthreads(); /* the previous chunk's fragments have been read */                            \
     _Pragma("unroll") for (int i = 0; i < 8; ++i)                                                   \
         *reinterpret_cast<u32x4*>(&ws[wave][2 * i + w_row0][w_col]) = wreg[i];                      \
     {                                                                                               \
-      const bool inside_ = (C_) * SBK + x_col < K;                                                  \
+      const bool inside_ = cur_ * SBK + x_col < K;                                                  \
       _Pragma("unroll") for (int i = 0; i < XP; ++i)                                                \
           *reinterpret_cast<u32x4*>(&xs[i * (THREADS / 32) + x_row0][x_col]) = inside_ ? xreg[i] : zero; \
     }                                                                                               \
     __syncthreads();                                                                                \
-    if ((C_) + 1 < c_end) TK_FETCH_W((C_) + 1)                                                      \
-    if ((C_) + 1 < c_end) TK_FETCH_X((C_) + 1)                                                      \
+    if ((I_) + 1 < nchunks) {                                                                       \
+      const int next_ = chunk_at((I_) + 1);                                                         \
+      TK_FETCH_W(next_)                                                                             \
+      TK_FETCH_X(next_)                                                                             \
+    }                                                                                               \
     _Pragma("unroll") for (int s = 0; s < SBK / 32; ++s) {                                          \
       Frag8 wf;                                                                                     \
       wf.u = *reinterpret_cast<const uint4*>(&ws[wave][r][s * 32 + kb * 8]);                        \
@@ -309,11 +322,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
     }                                                                                               \
   }
 
-  if (c_begin < c_end) {
-    TK_FETCH_W(c_begin)
-    TK_FETCH_X(c_begin)
+  if (nchunks > 0) {
+    const int first_ = chunk_at(0);
+    TK_FETCH_W(first_)
+    TK_FETCH_X(first_)
   }
-  for (int c = c_begin; c < c_end; ++c) TK_CHUNK(c)
+  for (int i = 0; i < nchunks; ++i) TK_CHUNK(i)
 #undef TK_CHUNK
 #undef TK_FETCH_X
 #undef TK_FETCH_W

@@ -320,10 +320,12 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
                                               _stream()), "gemm_tiled")
 
 
-def stream_waves(rows: int) -> int:
-    """Waves a block of the streaming product: from 33 rows of activations on, eight waves
-    share a chunk of them (the block then owns 128 weight rows), else four."""
-    return 8 if rows > 32 else 4
+def stream_waves(rows: int, k: int, gated: bool = False) -> int:
+    """Waves a block of the streaming product.  Eight waves share a chunk of the
+    activations (the block then owns 128 weight rows), which pays when the chunk is large
+    (more than 32 rows) and the walk over K long (the gated product, whose halves meet in
+    one block, and K from 8192 on); else four."""
+    return 8 if rows > 32 and (gated or k >= 8192) else 4
 
 
 def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: int = 1, waves: int = 0) -> int:
@@ -350,7 +352,7 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
         ldc, stride = n, m * n
     _note(f"{m}x{n}x{k}", (n * k + m * k) * 2 + splits * m * n * out.element_size(), 2.0 * m * n * k)
     used = _fn("gemm_mfma", "tk_gemm_stream")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
-                                              w.stride(0), ldc, splits, stride, waves or stream_waves(m), _stream())
+                                              w.stride(0), ldc, splits, stride, waves or stream_waves(m, k), _stream())
     if used < 1:
         raise KernelError(f"gemm_stream failed with status {used}")
     return used
@@ -368,7 +370,7 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, w
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gated product needs M <= 64 and 16-byte aligned rows")
     _note(f"{m}x{w.shape[0]}x{k}", (w.shape[0] * k + m * k) * 2 + m * w.shape[0], 2.0 * m * w.shape[0] * k)
     _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
-                                                     w.stride(0), out.stride(0), waves or stream_waves(m), _stream()), "gemm_stream_swiglu")
+                                                     w.stride(0), out.stride(0), waves or stream_waves(m, k, True), _stream()), "gemm_stream_swiglu")
 
 
 LT_WORKSPACE_BYTES = 128 << 20
