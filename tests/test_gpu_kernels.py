@@ -144,6 +144,55 @@ def test_many_tiles_over_long_contexts_use_the_four_wave_kernel():
         torch.testing.assert_close(g, w, **TOL[torch.bfloat16])
 
 
+@pytest.mark.parametrize("nh, nkv, hd, ps", [(8, 2, 128, 16), (6, 3, 64, 32), (3, 1, 128, 16), (32, 8, 128, 16), (4, 4, 64, 64)])
+def test_wide_tiles_for_long_walks(nh, nkv, hd, ps, monkeypatch):
+    """Portions cut into tiles of 32 tokens, the 32x32 matrix-core form: taken (checked by
+    its conditions, here with the threshold on the context lowered) when tiles are mostly
+    full; portions that start at zero, in the middle of a page, end inside a tile, a
+    one-token tail tile, and a decode token beside them."""
+    from tokamak_amd.kernels import attention
+
+    monkeypatch.setattr(attention, "WIDE_FROM_KEYS", 64)
+    requests = [(0, 200), (37, 150), (900, 33), (5, 32), (300, 1)]
+    tiles = [q for _, q in requests if q > 1]
+    assert sum(tiles) >= attention.WIDE_FROM_TOKENS * sum(-(-q // 32) for q in tiles)
+    launched = []
+    real = attention.ops.attention_mfma
+    monkeypatch.setattr(attention.ops, "attention_mfma", lambda mode, *a, **k: (launched.append(mode), real(mode, *a, **k))[1])
+    got, want = run_attention(torch.bfloat16, nh, nkv, hd, ps, requests, seed=21)
+    assert launched == ["heads", "tokens_wide"]
+    for g, w in zip(got, want):
+        assert torch.isfinite(g).all(), "a page that the request does not own, or a slot past its end, was read"
+        torch.testing.assert_close(g, w, **TOL[torch.bfloat16])
+
+
+def test_wide_tiles_find_a_far_key_and_respect_the_causal_edge():
+    """The wide form on inputs made to show faults: one key far back dominates one query's
+    softmax (its value must come out), and the key right after a query's position is made
+    enormous (reading it would show)."""
+    from tokamak_amd.kernels import attention
+
+    hd, nh, nkv = 128, 8, 2
+    seen = {}
+
+    def boost(q, k, v, ctx, qlen):
+        direction = torch.nn.functional.normalize(torch.randn(hd, generator=torch.Generator().manual_seed(9)), dim=0)
+        k[7, :, :] = (direction * 16.0).to(k.dtype)                 # far back, first page
+        q[40, :, :] = (direction * 16.0).to(q.dtype)                # query at position ctx + 40
+        other = torch.nn.functional.normalize(torch.randn(hd, generator=torch.Generator().manual_seed(10)), dim=0)
+        q[10, :, :] = (other * 4.0).to(q.dtype)
+        k[ctx + 11, :, :] = (other * 50.0).to(k.dtype)              # the key right after query 10: hidden from it
+        v[ctx + 11, :, :] = 1000.0
+        seen["far"] = v[7].float().clone()
+
+    got, want = run_attention(torch.bfloat16, nh, nkv, hd, 16, [(4100, 96)], boost=boost, seed=5)
+    assert attention.WIDE_FROM_KEYS <= 4196
+    torch.testing.assert_close(got[0], want[0], **TOL[torch.bfloat16])
+    expected = seen["far"].repeat_interleave(nh // nkv, dim=0)
+    torch.testing.assert_close(got[0][40], expected, rtol=0, atol=2e-2)
+    assert got[0][10].abs().max() < 50           # nothing of the hidden key's value of 1000
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("far", [0, 3, 255, 256, 511, 777])
 def test_a_far_key_among_hundreds_is_found(dtype, far):

@@ -550,6 +550,223 @@ void attention_prefill_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Prompt portions, wide form: a tile is up to 32 consecutive tokens of one request, a
+// wave owns the tile's 32 queries of one query head, and the products are
+// v_mfma_f32_32x32x16_bf16 (twice the work of a 16x16x32 per operand read from LDS, and
+// the shape that reaches the matrix cores' full rate).  As in the narrow form above, the
+// block of four waves shares 64 keys at a time through LDS, wave w < HPB owns head w of
+// the block's group, and every page lookup is wave-uniform.
+//   S^T[key][query] = K[key][:] . Q[query][:]   A = K rows (32 keys x 16 dims), B = Q
+//   O^T[dim][query] += V^T[dim][key] P^T[key][query]
+// A lane holds, of a 32-key block of S^T, the keys 8i + 4g + j (g = lane / 32; i, j < 4)
+// of its query: exactly the B operand of the second product if that product's sixteen
+// keys are taken in the order (g: four keys of quad 4h+g, then four of quad 4h+2+g).
+// V goes into LDS in that order ([16-key group][g][dim][two quads]), so its A operand is
+// one 16-byte read, contiguous over the wave's 32 dims.  K keeps the page's piece order.
+// No key split here (the narrow form has it for few tiles over long contexts).
+// ---------------------------------------------------------------------------
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+template <int HD, int HPB>
+__global__ __launch_bounds__(kPrefillThreads) __attribute__((amdgpu_waves_per_eu(2)))
+void attention_prefill_wide_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
+    const int* __restrict__ positions, const int* __restrict__ req_of_token,
+    const int* __restrict__ item_token, const int* __restrict__ item_count,
+    bf16_t* __restrict__ out, int num_items, int nh, int nkv, int ps, float scale_log2) {
+  constexpr int KST = HD / 16;  // 16-wide steps over the head dim (QK^T)
+  constexpr int DB = HD / 32;   // 32-wide blocks of the head dim (PV outputs)
+  constexpr int DBL = HD / 16;  // 16-dim blocks of a V page
+  constexpr int THREADS = kPrefillThreads;
+  constexpr int GROUP_PIECES = 2 * HD;      // 16-byte pieces of K (and of V) per 16-key group
+  constexpr int PIECES = 4 * GROUP_PIECES;  // per stage of 64 keys
+  constexpr int PPT = PIECES / THREADS;     // pieces of K, and of V, per thread and stage
+  constexpr int NBUF = 1;
+  static_assert(GROUP_PIECES % 64 == 0, "a wave's pieces of one load lie in one 16-key group");
+  __shared__ __attribute__((aligned(16))) bf16_t ks[PIECES * 8];
+  __shared__ __attribute__((aligned(16))) bf16_t vs[PIECES * 8];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, g = lane >> 5;
+  const int G = nh / nkv;
+  const int groups_per_kv = G / HPB;
+  const int kvh = blockIdx.x / groups_per_kv;
+  const bool computes = wave < HPB;
+  const int head = kvh * G + (blockIdx.x % groups_per_kv) * HPB + (computes ? wave : 0);
+  const int item = num_items - 1 - blockIdx.y;  // later tiles have more keys: start them first
+
+  const int n0 = item_token[item];
+  const int count = item_count[item];
+  const int pos0 = positions[n0];
+  const int last_pos = pos0 + count - 1;
+  const int last_key = last_pos;
+  const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
+  const size_t page_elems = (size_t)nkv * HD * ps;
+  const size_t head_off = (size_t)kvh * HD * ps;
+  const int c_pos = pos0 + col;
+  const bool c_valid = col < count;
+
+  // Q as B operand: lane (query col, g) holds Q[col][16c + 8g .. +8]
+  bf16x8 qreg[KST];
+  {
+    const bf16_t* qp = q + ((size_t)(n0 + (c_valid ? col : 0)) * nh + head) * HD + g * 8;
+#pragma unroll
+    for (int c = 0; c < KST; ++c) {
+      Frag8 f;
+      f.u = *reinterpret_cast<const uint4*>(qp + c * 16);
+      if (!c_valid) f.u = make_uint4(0, 0, 0, 0);
+      qreg[c] = f.v;
+    }
+  }
+
+  float m_run = -INFINITY, l_run = 0.f;
+  float16v acc[DB];  // acc[db][4i + j] = O^T[dim 32 db + 8i + 4g + j][col]
+#pragma unroll
+  for (int d = 0; d < DB; ++d)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[d][e] = 0.f;
+
+  // Piece p = i * THREADS + tid of a stage, as the pages hold it.  K: (group j, dim chunk
+  // c8, key) = (p / GROUP_PIECES, (p / 16) % (HD/8), p % 16), kept in that order in LDS.
+  // V: (group j, dim block d, quad, dim pair) = (p / GROUP_PIECES, (p / 32) % DBL,
+  // (p % 32) / 8, p % 8): two dims x four keys.
+  u32x4 kpre[NBUF][PPT], vpre[NBUF][PPT];
+  const int ps_shift = __ffs(ps) - 1;  // page sizes are powers of two here
+  int grp[PPT];                        // wave-uniform
+  unsigned k_in[PPT], v_in[PPT];       // byte offset inside the page's head, for key 0 of a group
+  int v_quad[PPT];
+  unsigned v_lds[PPT][2];              // element offsets in vs of the piece's two dims
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    const int p = i * THREADS + tid;
+    grp[i] = __builtin_amdgcn_readfirstlane(p / GROUP_PIECES);
+    k_in[i] = (unsigned)((((p / 16) % (HD / 8)) * ps + (p % 16)) * 8) * 2u;
+    const int d = (p / 32) % DBL, quad = (p % 32) / 8, dp = p % 8;
+    v_in[i] = (unsigned)(d * (ps >> 2) * 64 + (p % 32) * 8) * 2u;
+    v_quad[i] = quad;
+    // vs: [group j][g = quad & 1][dim][quad >> 1][4 keys]
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+      v_lds[i][half] =
+          (unsigned)(((((p / GROUP_PIECES) * 2 + (quad & 1)) * HD + d * 16 + 2 * dp + half) * 2 + (quad >> 1)) * 4);
+  }
+  int page_next[PPT];
+
+  TK_PAGES(0)
+  TK_FETCH(0, 0)
+  for (int s0 = 0; s0 <= last_key; s0 += 64) {
+    constexpr int buf = 0;
+    __syncthreads();  // every wave has read the previous stage
+    if (s0 + 63 > last_pos) {
+      // keys past the request's end may hold anything (their probability is zero, but
+      // 0 * NaN is NaN): zero their values on the way into LDS
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) {
+        const int k0 = s0 + grp[i] * 16 + v_quad[i] * 4;
+        const unsigned m01 = (k0 + 0 > last_pos ? 0u : 0x0000ffffu) | (k0 + 1 > last_pos ? 0u : 0xffff0000u);
+        const unsigned m23 = (k0 + 2 > last_pos ? 0u : 0x0000ffffu) | (k0 + 3 > last_pos ? 0u : 0xffff0000u);
+        vpre[buf][i] &= u32x4{m01, m23, m01, m23};
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      *reinterpret_cast<u32x4*>(ks + (size_t)(i * THREADS + tid) * 8) = kpre[buf][i];
+      *reinterpret_cast<uint2*>(vs + v_lds[i][0]) = make_uint2(vpre[buf][i][0], vpre[buf][i][1]);
+      *reinterpret_cast<uint2*>(vs + v_lds[i][1]) = make_uint2(vpre[buf][i][2], vpre[buf][i][3]);
+    }
+    __syncthreads();
+    if (s0 + 64 <= last_key) TK_FETCH(s0 + 64, buf)
+    if (!computes) continue;
+
+    // S^T for two blocks of 32 keys: sc[kb][4i + j] = score of key s0 + 32 kb + 8i + 4g + j
+    float16v sc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sc[kb][e] = 0.f;
+#pragma unroll
+      for (int c = 0; c < KST; ++c) {
+        Frag8 kf;  // K[key 32 kb + col][16c + 8g .. +8]: piece (group 2kb + col/16, chunk 2c + g, key col%16)
+        kf.u = *reinterpret_cast<const uint4*>(
+            ks + ((size_t)((2 * kb + (col >> 4)) * (HD / 8) + 2 * c + g) * 16 + (col & 15)) * 8);
+        sc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qreg[c], sc[kb], 0, 0, 0);
+      }
+    }
+    if (s0 + 63 > pos0) {  // some key of this stage is hidden from some query, or is past the end
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = s0 + 32 * kb + 8 * (e >> 2) + 4 * g + (e & 3);
+          if (key > c_pos || key > last_pos) sc[kb][e] = -INFINITY;
+        }
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) tmax = fmaxf(tmax, sc[kb][e]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    // the running maximum is kept in units of log2: m = max(score) * scale * log2(e)
+    const float m_new = fmaxf(m_run, tmax * scale_log2);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);
+    m_run = m_new;
+    float psum = 0.f;
+    Frag8 pb[2][2];  // pb[kb][h]: the sixteen keys 32 kb + 16 h .. of this lane's half
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        float pr[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pr[e] = fast_exp2(fmaf(sc[kb][8 * h + e], scale_log2, -m_safe));
+          psum += pr[e];
+        }
+        pb[kb][h].u = make_uint4(pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3]), pack_bf16x2(pr[4], pr[5]),
+                                 pack_bf16x2(pr[6], pr[7]));
+      }
+    l_run = l_run * alpha + psum;
+    // the accumulators need rescaling only when some query's maximum moved
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+      for (int d = 0; d < DB; ++d) acc[d] *= alpha;
+    }
+#pragma unroll
+    for (int d = 0; d < DB; ++d) {
+      float16v a = acc[d];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          Frag8 vf;  // V^T[dim 32 d + col][the lane half's eight keys of group 2 kb + h]
+          vf.u = *reinterpret_cast<const uint4*>(vs + ((size_t)((2 * kb + h) * 2 + g) * HD + 32 * d + col) * 8);
+          a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pb[kb][h].v, a, 0, 0, 0);
+        }
+      acc[d] = a;
+    }
+  }
+
+  float l = l_run;
+  l += __shfl_xor(l, 32, kWave);
+  if (c_valid && computes) {
+    const float inv = 1.f / l;
+    bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * HD + g * 4;
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint2 o;
+        o.x = pack_bf16x2(acc[d][4 * i] * inv, acc[d][4 * i + 1] * inv);
+        o.y = pack_bf16x2(acc[d][4 * i + 2] * inv, acc[d][4 * i + 3] * inv);
+        *reinterpret_cast<uint2*>(op + 32 * d + 8 * i) = o;
+      }
+  }
+}
+
 #undef TK_FETCH
 #undef TK_PAGES
 
@@ -570,6 +787,21 @@ static int launch_prefill(const void* q, const void* k_cache, const void* v_cach
     attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token, item_count,
                                                          (bf16_t*)out, nsplit, split_keys, nh);
   }
+  return launch_status();
+}
+
+template <int HD, int HPB>
+static int launch_prefill_wide(const void* q, const void* k_cache, const void* v_cache,
+                               const int* block_tables, int max_pages, const int* positions,
+                               const int* req_of_token, const int* item_token, const int* item_count,
+                               int num_items, void* out, int nh, int nkv, int ps, float scale,
+                               hipStream_t stream) {
+  const int G = nh / nkv;
+  dim3 grid(nkv * (G / HPB), num_items);
+  attention_prefill_wide_kernel<HD, HPB><<<grid, kPrefillThreads, 0, stream>>>(
+      (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
+      positions, req_of_token, item_token, item_count, (bf16_t*)out, num_items, nh, nkv, ps,
+      scale * 1.4426950408889634f);
   return launch_status();
 }
 
@@ -613,6 +845,7 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
 // mode 1: tokens (item = up to 16 consecutive tokens of one request; with nsplit > 1 split_keys
 //         is a multiple of 64 and the partial buffers hold 16 rows per item)
 // mode 2: tokens, every tile over a long context (same results; the kernel built for four waves a SIMD)
+// mode 3: tokens, wide form (item = up to 32 consecutive tokens of one request; nsplit must be 1)
 // Returns -2 if this shape is not instantiated (the caller uses the generic kernel).
 TK_API int tk_attention_decode_waves() { return kDecodeWaves; }
 
@@ -623,7 +856,7 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
                              int split_keys, int nh, int nkv, int hd, int ps, float scale,
                              hipStream_t stream) {
   if (num_items <= 0) return 0;
-  if (mode < 0 || mode > 2) return -1;
+  if (mode < 0 || mode > 3) return -1;
   if (nkv <= 0 || nh % nkv != 0 || ps < 16 || (ps & (ps - 1)) != 0 || split_keys % 16 != 0 || nsplit < 1) return -1;
   if (num_items > 65535 || nh > 65535) return -1;
   const int G = nh / nkv;
@@ -636,9 +869,27 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
     if (hd == 64) return launch<64>(TK_ARGS);
     return -2;
   }
+  const int hpb = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
+  if (mode == 3) {
+    if (nsplit != 1) return -1;
+#define TK_WARGS                                                                                  \
+  q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
+      num_items, out, nh, nkv, ps, scale, stream
+    if (hd == 128) {
+      if (hpb == 4) return launch_prefill_wide<128, 4>(TK_WARGS);
+      if (hpb == 2) return launch_prefill_wide<128, 2>(TK_WARGS);
+      return launch_prefill_wide<128, 1>(TK_WARGS);
+    }
+    if (hd == 64) {
+      if (hpb == 4) return launch_prefill_wide<64, 4>(TK_WARGS);
+      if (hpb == 2) return launch_prefill_wide<64, 2>(TK_WARGS);
+      return launch_prefill_wide<64, 1>(TK_WARGS);
+    }
+#undef TK_WARGS
+    return -2;
+  }
   // the keys of a tile may be split too: in whole stages of 64 keys, sixteen partial rows a tile
   if (nsplit > 1 && (split_keys % 64 != 0 || (long)num_items * 16 > 65535)) return -1;
-  const int hpb = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
 #define TK_PARGS                                                                                  \
   q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
       num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream

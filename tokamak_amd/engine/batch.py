@@ -42,12 +42,16 @@ class StepBatch:
     logit_rows: torch.Tensor     # [M] int32, token rows whose logits are wanted
     block_tables: list[torch.Tensor]  # per cache group [R, max_pages] int32
     # work lists for the attention kernels: single (decode) tokens, and tiles of up to
-    # 16 consecutive tokens of the longer spans
+    # 16, and of up to 32, consecutive tokens of the longer spans
     decode_tokens: torch.Tensor | None = None   # [num_decode] int32 token rows
     tile_first: torch.Tensor | None = None      # [num_tiles] int32 first token row
     tile_count: torch.Tensor | None = None      # [num_tiles] int32 tokens in the tile
+    wide_first: torch.Tensor | None = None      # [num_wide] int32 first token row of a 32-token tile
+    wide_count: torch.Tensor | None = None      # [num_wide] int32 tokens in it
     num_decode: int = 0
     num_tiles: int = 0
+    num_wide: int = 0
+    num_tile_tokens: int = 0                    # tokens of the spans that are cut into tiles
     max_decode_len: int = 0                     # longest context among the decode tokens
     max_tile_len: int = 0                       # longest context (with the portion) among the tiled spans
     min_tile_ctx: int = 0                       # shortest cached context among the tiled spans
@@ -60,7 +64,8 @@ class StepBatch:
 
 
 TILE_TOKENS = 16   # tokens per attention tile of a prompt portion
-NUM_FIXED = 10     # arrays in the packed buffer before the block tables
+WIDE_TOKENS = 32   # and per tile of the wide attention kernel
+NUM_FIXED = 12     # arrays in the packed buffer before the block tables
 
 
 @dataclass
@@ -76,6 +81,7 @@ class PackedBatch:
     num_logit_rows: int
     num_decode: int
     num_tiles: int
+    num_wide: int
     q_lens: list[int]
     ctx_lens: list[int]
     max_decode_len: int
@@ -98,7 +104,7 @@ def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] |
                           None if fixed_widths is None else fixed_widths[g])
               for g in range(num_groups)]
     m = sum(len(s.want) for s in spans)
-    decode_rows, tiles = [], []
+    decode_rows, tiles, wide = [], [], []
     at = 0
     for s in spans:
         q = len(s.tokens)
@@ -106,20 +112,23 @@ def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] |
             decode_rows.append(at)
         else:
             tiles.extend((at + t, min(TILE_TOKENS, q - t)) for t in range(0, q, TILE_TOKENS))
+            wide.extend((at + t, min(WIDE_TOKENS, q - t)) for t in range(0, q, WIDE_TOKENS))
         at += q
-    nd, nt = len(decode_rows), len(tiles)
-    sizes = [n, n, n, r + 1, r, r, m, nd, nt, nt] + [r * w for w in widths]
+    nd, nt, nw = len(decode_rows), len(tiles), len(wide)
+    sizes = [n, n, n, r + 1, r, r, m, nd, nt, nt, nw, nw] + [r * w for w in widths]
     offsets = [0]
     for size in sizes:
         offsets.append(offsets[-1] + size)
     buf = np.zeros(offsets[-1], dtype=np.int32)
-    tok, pos, req, qs, ctx, slots, rows, dec, tfirst, tcount = (
+    tok, pos, req, qs, ctx, slots, rows, dec, tfirst, tcount, wfirst, wcount = (
         buf[offsets[i]:offsets[i + 1]] for i in range(NUM_FIXED))
     tabs = [buf[offsets[NUM_FIXED + g]:offsets[NUM_FIXED + 1 + g]].reshape(r, widths[g])
             for g in range(num_groups)]
     dec[:] = decode_rows
     tfirst[:] = [t[0] for t in tiles]
     tcount[:] = [t[1] for t in tiles]
+    wfirst[:] = [t[0] for t in wide]
+    wcount[:] = [t[1] for t in wide]
     at = 0
     mi = 0
     for i, s in enumerate(spans):
@@ -143,7 +152,7 @@ def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] |
     qs[r] = at
     return PackedBatch(
         buf=buf, offsets=offsets, widths=widths, num_tokens=n, num_requests=r, num_logit_rows=m,
-        num_decode=nd, num_tiles=nt, q_lens=[len(s.tokens) for s in spans],
+        num_decode=nd, num_tiles=nt, num_wide=nw, q_lens=[len(s.tokens) for s in spans],
         ctx_lens=[s.ctx_len for s in spans],
         max_decode_len=max((s.ctx_len + 1 for s in spans if len(s.tokens) == 1), default=0),
         max_tile_len=max((s.ctx_len + len(s.tokens) for s in spans if len(s.tokens) > 1), default=0),
@@ -160,7 +169,9 @@ def batch_from_device(packed: PackedBatch, dev: torch.Tensor) -> StepBatch:
         ctx_len=parts[4], state_slots=parts[5], logit_rows=parts[6],
         block_tables=[parts[NUM_FIXED + g].view(r, widths[g]) for g in range(len(widths))],
         decode_tokens=parts[7], tile_first=parts[8], tile_count=parts[9],
-        num_decode=packed.num_decode, num_tiles=packed.num_tiles,
+        wide_first=parts[10], wide_count=parts[11],
+        num_decode=packed.num_decode, num_tiles=packed.num_tiles, num_wide=packed.num_wide,
+        num_tile_tokens=sum(q for q in packed.q_lens if q > 1),
         max_decode_len=packed.max_decode_len, max_tile_len=packed.max_tile_len,
         min_tile_ctx=packed.min_tile_ctx,
         q_lens=packed.q_lens, ctx_lens=packed.ctx_lens,

@@ -13,6 +13,9 @@ TILE_SPLIT_BELOW_BLOCKS = 256   # a portion with fewer blocks than this has its 
 TILE_SPLIT_MIN_KEYS = 512       # ... into pieces no shorter than this
 TARGET_TILE_BLOCKS = 1024
 DENSE_TILES_FROM = 2048         # every tiled span starts at least this deep: the four-wave kernel
+WIDE_FROM_KEYS = 4096           # longest context from which the 32-token tiles of the wide kernel pay (+15-20 %;
+                                # for shorter walks the narrow one's smaller tiles balance better)
+WIDE_FROM_TOKENS = 20           # ... if a 32-token tile holds at least this many tokens on average
 
 
 def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
@@ -82,6 +85,15 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
             group = num_heads // num_kv_heads
             per_tile = num_kv_heads * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
             split, nsplit = tile_split(batch.num_tiles, per_tile, batch.max_tile_len)
+            if (nsplit == 1 and batch.max_tile_len >= WIDE_FROM_KEYS
+                    and batch.num_tile_tokens >= WIDE_FROM_TOKENS * batch.num_wide):
+                # long walks over the keys, tiles of 32 tokens mostly full: the wide kernel
+                if profiling:
+                    ops._note(f"portions {batch.num_wide} wide tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
+                ops.attention_mfma("tokens_wide", q, k_cache, v_cache, block_tables, batch.positions,
+                                   batch.req_of_token, batch.wide_first, batch.wide_count, batch.num_wide,
+                                   out, **common)
+                return
             dense = nsplit == 1 and batch.min_tile_ctx >= DENSE_TILES_FROM
             if profiling:
                 ops._note(f"portions {batch.num_tiles} tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
