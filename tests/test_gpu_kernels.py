@@ -487,3 +487,72 @@ def test_fused_gate_up_silu_product(M, I, K):
     g = x.double() @ w[:I].double().T
     u = x.double() @ w[I:].double().T
     torch.testing.assert_close(out.cpu().double(), g / (1 + torch.exp(-g)) * u, rtol=2e-2, atol=1e-2)
+
+
+# ---------------------------------------------------------------------------
+# decode tokens in one kernel: q/k norm, rotation, cache write and attention
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("nh, nkv, hd, ps", [(32, 8, 128, 16), (6, 3, 64, 32), (14, 1, 128, 16), (3, 3, 128, 64)])
+@pytest.mark.parametrize("form", ["partial sums", "bfloat16", "no norm", "no rotation", "reads only"])
+def test_fused_decode_equals_the_two_kernels(nh, nkv, hd, ps, form):
+    """The one-kernel form of a decode-only step against the q/k norm kernel followed by
+    the attention kernel, on the same inputs: attention output, and every page of the cache
+    afterwards (the token's key and value land in their slots, nothing else is touched).
+    Contexts end at a tile's first and last key, at a page's edge, at position zero and
+    deep enough for several splits; unowned pages are NaN."""
+    from tokamak_amd.kernels import ops
+    from tokamak_amd.kernels.attention import decode_attention_fused, fused_decode_fits, paged_attention
+
+    g = torch.Generator().manual_seed(nh * 7 + hd)
+    ctxs = [0, 15, 16, 31, 255, 256, 700, 2300, 47]
+    stores = form != "reads only"
+    width = (nh + (2 * nkv if stores else 0)) * hd
+    n = len(ctxs)
+    total_pages = sum(-(-(c + 1) // ps) for c in ctxs) + 4
+    order = torch.randperm(total_pages, generator=g).tolist()
+    k_cache = torch.full((total_pages, nkv * hd * ps), float("nan"), dtype=torch.bfloat16)
+    v_cache = torch.full((total_pages, nkv * hd * ps), float("nan"), dtype=torch.bfloat16)
+    spans = []
+    for c in ctxs:
+        npages = -(-(c + 1) // ps)
+        table, order = order[:npages], order[npages:]
+        keys = c + (0 if stores else 1)            # a reading call finds the token's own key in the cache
+        if keys:
+            pack_pages(k_cache, v_cache, torch.randn(keys, nkv, hd, generator=g), torch.randn(keys, nkv, hd, generator=g), table, ps)
+        spans.append((1, c, table))
+    batch = make_batch(spans)
+    parts = 3 if form == "partial sums" else 1
+    if form == "bfloat16":
+        qkv = (torch.randn(n, width, generator=g) * 0.7).bfloat16().to(DEV)
+    else:
+        qkv = (torch.randn(parts, n, width, generator=g) * 0.5).to(DEV)
+        qkv = qkv if parts > 1 else qkv[0]
+    q_w = k_w = None
+    if form != "no norm":
+        q_w, k_w = (1 + 0.2 * torch.randn(hd, generator=g)).to(DEV), (1 + 0.2 * torch.randn(hd, generator=g)).to(DEV)
+    rot = 0 if form == "no rotation" else hd
+    cos = sin = None
+    if rot:
+        angle = torch.rand(n, hd // 2, generator=g) * 6.28
+        cos, sin = angle.cos().to(DEV), angle.sin().to(DEV)
+    common = dict(num_heads=nh, num_kv_heads=nkv, head_dim=hd, page_size=ps)
+    assert fused_decode_fits(torch.bfloat16, hd, ps, nh // nkv, None, rot, batch)
+
+    kc1, vc1 = k_cache.to(DEV), v_cache.to(DEV)
+    q = torch.empty(n, nh * hd, dtype=torch.bfloat16, device=DEV)
+    ops.qknorm_rope_store(qkv, q_w, k_w, cos, sin, batch.positions, batch.req_of_token, batch.block_tables[0], q,
+                          kc1, vc1, rotary_dim=rot, eps=1e-5, store=stores, **common)
+    want = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    paged_attention(q, kc1, vc1, batch.block_tables[0], batch, want, scale=hd ** -0.5, **common)
+
+    kc2, vc2 = k_cache.to(DEV), v_cache.to(DEV)
+    got = torch.full((n, nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert decode_attention_fused(qkv, q_w, k_w, cos, sin, kc2, vc2, batch.block_tables[0], batch, got,
+                                  rotary_dim=rot, eps=1e-5, scale=hd ** -0.5, store=stores, **common)
+    assert torch.isfinite(got).all()
+    torch.testing.assert_close(got.float().cpu(), want.float().cpu(), rtol=2e-2, atol=1e-2)
+    # the caches agree bit for bit where they hold numbers, and NaN stays where it was
+    for a, b in ((kc1, kc2), (vc1, vc2)):
+        a, b = a.cpu(), b.cpu()
+        assert torch.equal(torch.isnan(a), torch.isnan(b))
+        assert torch.equal(torch.nan_to_num(a.float()), torch.nan_to_num(b.float()))

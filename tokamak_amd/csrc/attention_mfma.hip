@@ -43,16 +43,77 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 constexpr int kDecodeWaves = 16;
 
+// What the fused form of the decode kernel takes instead of finished queries: the q/k/v
+// projection's output as it left the product (`parts` float32 partial sums of a split-K
+// product, part_stride elements apart, or one bfloat16 matrix), rows of (nh + 2 nkv_in)
+// heads; the per-head norm weights (or null), the rotary tables [N, HD/2] (rot == HD) or
+// none (rot == 0).  nkv_in == 0: the call only reads the cache (queries alone are made).
+struct DecodeInputs {
+  const void* qkv;
+  int in_f32, parts;
+  long part_stride;
+  const float *q_weight, *k_weight, *cos_t, *sin_t;
+  int rot, nkv_in;
+  float eps;
+};
+
+// One head's vector from the projection's output: partial sums added, per-head RMSNorm,
+// half-split rotation; lane l ends up with dims 2l and 2l + 1 (HD / 2 lanes take part).
+// What the separate kernel of elementwise.hip computes, for one token and head.
+template <int HD>
+__device__ __forceinline__ void decode_head_vector(const DecodeInputs& in, size_t row_offset, int head_col,
+                                                   const float* weight, bool rotate, int token, int lane,
+                                                   float& x0, float& x1) {
+  const bool active = lane < HD / 2;
+  const int d = 2 * (active ? lane : 0);
+  x0 = x1 = 0.f;
+  if (in.in_f32) {
+    const float* src = static_cast<const float*>(in.qkv) + row_offset + (size_t)head_col * HD + d;
+    for (int p = 0; p < in.parts; ++p) {
+      const float2 v = *reinterpret_cast<const float2*>(src + (size_t)p * in.part_stride);
+      x0 += v.x;
+      x1 += v.y;
+    }
+  } else {
+    const uint32_t v = *reinterpret_cast<const uint32_t*>(static_cast<const bf16_t*>(in.qkv) + row_offset +
+                                                          (size_t)head_col * HD + d);
+    x0 = __uint_as_float(v << 16);
+    x1 = __uint_as_float(v & 0xffff0000u);
+  }
+  if (!active) x0 = x1 = 0.f;
+  if (weight != nullptr) {
+    const float ss = wave_sum(x0 * x0 + x1 * x1);
+    const float rstd = rsqrtf(ss / (float)HD + in.eps);
+    x0 = x0 * rstd * weight[d];
+    x1 = x1 * rstd * weight[d + 1];
+  }
+  if (rotate) {
+    // out[j] = x[j] cos_j - x[j + HD/2] sin_j ; out[j + HD/2] = x[j + HD/2] cos_j + x[j] sin_j
+    const float p0 = __shfl_xor(x0, HD / 4, kWave), p1 = __shfl_xor(x1, HD / 4, kWave);
+    const int j = d % (HD / 2);
+    const float2 c = *reinterpret_cast<const float2*>(in.cos_t + (size_t)token * (HD / 2) + j);
+    const float2 sn = *reinterpret_cast<const float2*>(in.sin_t + (size_t)token * (HD / 2) + j);
+    const float sign = (d < HD / 2) ? -1.f : 1.f;
+    x0 = x0 * c.x + sign * p0 * sn.x;
+    x1 = x1 * c.y + sign * p1 * sn.y;
+  }
+}
+
 // WAVES: waves of a block (they share a split's keys and merge through LDS); D: tiles of
-// 16 keys a wave keeps in flight.
-template <int HD, int WAVES, int D>
+// 16 keys a wave keeps in flight.  FUSED: the block first makes its queries (and, if the
+// call stores, the token's own key and value, which the block of the last split writes to
+// the page and every wave that meets the token's position takes from LDS) from the
+// projection's output: one kernel less a layer than with the separate q/k norm kernel.
+template <int HD, int WAVES, int D, bool FUSED>
 __global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
-    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache_in,
+    const bf16_t* __restrict__ v_cache_in, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ item_token, const int* __restrict__ item_count,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int nsplit,
-    int split_keys, int nh, int nkv, int ps, float scale_log2) {
+    int split_keys, int nh, int nkv, int ps, float scale_log2, DecodeInputs in) {
+  const bf16_t* __restrict__ k_cache = k_cache_in;
+  const bf16_t* __restrict__ v_cache = v_cache_in;
   constexpr int KCH = HD / 32;  // 32-wide chunks of the head dim (QK^T steps)
   constexpr int DBL = HD / 16;  // 16-wide blocks of the head dim (PV outputs)
   // LDS: the waves' accumulators of the group's heads [WAVES][G][HD], then their (m, l) [WAVES][16] each
@@ -82,7 +143,43 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
 
   // Q as B operand: lane (col, kb) holds Q[col][c*32 + kb*8 .. +8]
   bf16x8 qreg[KCH];
-  {
+  bool stores = false;    // FUSED: this call stores the token's key and value
+  bf16_t* s_new = nullptr;  // FUSED: [G + 2][HD] in LDS: the group's queries, then the new key and value
+  if constexpr (FUSED) {
+    s_new = reinterpret_cast<bf16_t*>(s_dyn + (size_t)WAVES * G * HD + 2 * WAVES * 16);
+    stores = in.nkv_in > 0;
+    const int heads_in = nh + 2 * in.nkv_in;
+    const size_t row_offset = (size_t)n0 * heads_in * HD;
+    if (wave < G + (stores ? 2 : 0)) {
+      float x0, x1;
+      if (wave < G)
+        decode_head_vector<HD>(in, row_offset, kvh * G + wave, in.q_weight, in.rot != 0, n0, lane, x0, x1);
+      else if (wave == G)
+        decode_head_vector<HD>(in, row_offset, nh + kvh, in.k_weight, in.rot != 0, n0, lane, x0, x1);
+      else
+        decode_head_vector<HD>(in, row_offset, nh + in.nkv_in + kvh, nullptr, false, n0, lane, x0, x1);
+      if (lane < HD / 2)
+        *reinterpret_cast<uint32_t*>(s_new + (size_t)wave * HD + 2 * lane) = pack_bf16x2(x0, x1);
+    }
+    __syncthreads();
+    // the block that holds the token's position writes its key and value to the page
+    if (stores && wave == 0 && lane < HD / 2 && k_begin <= pos0 && pos0 < k_begin + split_keys) {
+      const int page = table[pos0 / ps], off = pos0 % ps, d = 2 * lane;
+      bf16_t* kp = const_cast<bf16_t*>(k_cache_in) + (size_t)page * page_elems + head_off;
+      bf16_t* vp = const_cast<bf16_t*>(v_cache_in) + (size_t)page * page_elems + head_off;
+      *reinterpret_cast<uint32_t*>(kp + ((size_t)(d >> 3) * ps + off) * 8 + (d & 7)) =
+          *reinterpret_cast<const uint32_t*>(s_new + (size_t)G * HD + d);
+      const bf16_t* vn = s_new + (size_t)(G + 1) * HD + d;
+      vp[((size_t)(d >> 4) * (ps >> 2) + (off >> 2)) * 64 + (d & 15) * 4 + (off & 3)] = vn[0];
+      vp[((size_t)((d + 1) >> 4) * (ps >> 2) + (off >> 2)) * 64 + ((d + 1) & 15) * 4 + (off & 3)] = vn[1];
+    }
+#pragma unroll
+    for (int c = 0; c < KCH; ++c) {
+      Frag8 f;
+      f.u = c_valid ? *reinterpret_cast<const uint4*>(s_new + (size_t)col * HD + c * 32 + kb * 8) : make_uint4(0, 0, 0, 0);
+      qreg[c] = f.v;
+    }
+  } else {
     const bf16_t* qp = q + ((size_t)n0 * nh + c_head) * HD + kb * 8;
 #pragma unroll
     for (int c = 0; c < KCH; ++c) {
@@ -135,6 +232,24 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
       if (t >= t_end) break;  // the same for every lane of the wave
       const int c0 = k_begin + t * 16;
       const bool edge = c0 + 15 > pos0;  // some key of this tile lies past the token's position
+      if constexpr (FUSED) {
+        // the token's own key and value come from LDS (the page's slot is being written, or was not yet)
+        if (stores && c0 <= pos0 && pos0 - c0 < 16) {
+          if (col == pos0 - c0) {
+#pragma unroll
+            for (int c = 0; c < KCH; ++c)
+              kreg[i][c].u = *reinterpret_cast<const uint4*>(s_new + (size_t)G * HD + c * 32 + kb * 8);
+          }
+          if (kb == ((pos0 - c0) >> 2)) {
+#pragma unroll
+            for (int d = 0; d < DBL; ++d) {
+              short4v tv = vreg[i][d].v;
+              tv[(pos0 - c0) & 3] = (short)s_new[(size_t)(G + 1) * HD + d * 16 + col];
+              vreg[i][d].v = tv;
+            }
+          }
+        }
+      }
       float4v sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < KCH; ++c) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[i][c].v, qreg[c], sc, 0, 0, 0);
@@ -805,22 +920,22 @@ static int launch_prefill_wide(const void* q, const void* k_cache, const void* v
   return launch_status();
 }
 
-template <int HD>
+template <int HD, bool FUSED>
 static int launch(const void* q, const void* k_cache, const void* v_cache, const int* block_tables,
                   int max_pages, const int* positions, const int* req_of_token,
                   const int* item_token, const int* item_count, int num_items, void* out,
                   float* part_o, float* part_ml, int nsplit, int split_keys, int nh, int nkv, int ps,
-                  float scale, hipStream_t stream) {
+                  float scale, hipStream_t stream, DecodeInputs in = DecodeInputs{}) {
   dim3 grid(nsplit, nkv, num_items);
   const int G = nh / nkv;
   // sixteen waves a block and one tile a wave in flight measured best at every batch size
   // (four or eight waves with two tiles: 12 % slower at batch 64, 15 % at batch 8)
-  const size_t lds = (size_t)(kDecodeWaves * G * HD + 2 * kDecodeWaves * 16) * 4;
+  const size_t lds = (size_t)(kDecodeWaves * G * HD + 2 * kDecodeWaves * 16) * 4 + (FUSED ? (size_t)(G + 2) * HD * 2 : 0);
   if (lds > 160 * 1024) return -2;
   if (lds > 48 * 1024) {  // beyond the default limit of dynamic LDS (groups of 7 heads and more)
     static bool raised = false;  // per template instance
     if (!raised) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_kernel<HD, kDecodeWaves, 1>),
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_kernel<HD, kDecodeWaves, 1, FUSED>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) {
         (void)hipGetLastError();
         return -2;
@@ -828,10 +943,10 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
       raised = true;
     }
   }
-  attention_decode_kernel<HD, kDecodeWaves, 1><<<grid, kDecodeWaves * 64, lds, stream>>>(
-          (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages, positions,
-          req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps,
-          scale * 1.4426950408889634f);
+  attention_decode_kernel<HD, kDecodeWaves, 1, FUSED><<<grid, kDecodeWaves * 64, lds, stream>>>(
+      (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages, positions,
+      req_of_token, item_token, item_count, (bf16_t*)out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps,
+      scale * 1.4426950408889634f, in);
   if (nsplit > 1) {
     dim3 mgrid(num_items, nh);
     attention_merge_kernel<HD><<<mgrid, 64, 0, stream>>>(part_o, part_ml, positions, item_token, nullptr,
@@ -865,8 +980,8 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
       num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream
   if (mode == 0) {
     if (G > 16) return -2;
-    if (hd == 128) return launch<128>(TK_ARGS);
-    if (hd == 64) return launch<64>(TK_ARGS);
+    if (hd == 128) return launch<128, false>(TK_ARGS);
+    if (hd == 64) return launch<64, false>(TK_ARGS);
     return -2;
   }
   const int hpb = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
@@ -906,5 +1021,38 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
   }
 #undef TK_PARGS
 #undef TK_ARGS
+  return -2;
+}
+
+// Decode tokens straight from the q/k/v projection's output: what tk_qknorm_rope_store
+// (elementwise.hip) followed by tk_attention_mfma in mode 0 computes, in one kernel (and a
+// merge if nsplit > 1).  qkv: rows of (nh + 2 nkv_in) heads of hd, bfloat16 (parts == 1,
+// in_f32 == 0) or `parts` float32 partial sums part_stride elements apart; nkv_in is nkv
+// (the token's key and value are made and stored) or 0 (the call only reads the cache).
+// q_weight/k_weight: per-head norm weights [hd] or null; rot: hd (tables cos_t/sin_t
+// [N, hd/2]) or 0.  Groups of up to 14 query heads.  Returns -2 if not instantiated.
+TK_API int tk_attention_decode_fused(const void* qkv, int in_f32, int parts, long part_stride,
+                                     const float* q_weight, const float* k_weight, const float* cos_t,
+                                     const float* sin_t, int rot, float eps, int nkv_in, void* k_cache,
+                                     void* v_cache, const int* block_tables, int max_pages,
+                                     const int* positions, const int* req_of_token, const int* item_token,
+                                     int num_items, void* out, float* part_o, float* part_ml, int nsplit,
+                                     int split_keys, int nh, int nkv, int hd, int ps, float scale,
+                                     hipStream_t stream) {
+  if (num_items <= 0) return 0;
+  if (nkv <= 0 || nh % nkv != 0 || ps < 16 || (ps & (ps - 1)) != 0 || split_keys % (16 * kDecodeWaves) != 0 || nsplit < 1)
+    return -1;
+  if (num_items > 65535 || nh > 65535 || parts < 1 || (parts > 1 && !in_f32)) return -1;
+  if ((nkv_in != 0 && nkv_in != nkv) || (rot != 0 && rot != hd) || (rot != 0 && (!cos_t || !sin_t))) return -1;
+  if ((q_weight != nullptr) != (k_weight != nullptr) && nkv_in != 0) return -1;
+  const int G = nh / nkv;
+  if (G + 2 > kDecodeWaves) return -2;
+  DecodeInputs in{qkv, in_f32, parts, part_stride, q_weight, k_weight, cos_t, sin_t, rot, nkv_in, eps};
+#define TK_FARGS                                                                                       \
+  nullptr, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, nullptr,  \
+      num_items, out, part_o, part_ml, nsplit, split_keys, nh, nkv, ps, scale, stream, in
+  if (hd == 128) return launch<128, true>(TK_FARGS);
+  if (hd == 64) return launch<64, true>(TK_FARGS);
+#undef TK_FARGS
   return -2;
 }

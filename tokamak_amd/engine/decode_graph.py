@@ -54,17 +54,20 @@ class DecodeGraph:
         self._turn = 0
         self.dev = torch.empty(self.size, dtype=torch.int32, device=device)
         self.batch = batch_from_device(packed, self.dev)
-        before = torch.cuda.memory_allocated(device)
         self._load(packed)
         # this step itself, eagerly: code objects are loaded and the allocator is warm
         # before the recording starts; the recording executes nothing
         self.first_logits = model.forward(self.batch, storage)
         torch.cuda.synchronize(device)
         self.batch.memo.clear()
+        # what the recording holds: the most that is live at once while it is recorded (its
+        # private pool keeps that much), measured from here on
+        torch.cuda.reset_peak_memory_stats(device)
+        before = torch.cuda.memory_allocated(device)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
             self.logits = model.forward(self.batch, storage)
-        self.bytes = max(0, torch.cuda.memory_allocated(device) - before)
+        self.bytes = max(0, torch.cuda.max_memory_allocated(device) - before) + self.size * 4
         self.replays = 0
 
     def _load(self, packed: PackedBatch) -> None:

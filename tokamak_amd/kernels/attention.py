@@ -53,6 +53,29 @@ def tile_split(num_tiles: int, blocks_per_tile: int, max_len: int) -> tuple[int,
     return split, -(-max_len // split)
 
 
+def fused_decode_fits(dtype, head_dim, page_size, group, window, rotary_dim, batch) -> bool:
+    """A step of decode tokens only, at shapes the one-kernel form takes."""
+    return (batch.num_tiles == 0 and batch.num_decode == batch.num_tokens and batch.num_decode > 0
+            and mfma_fits(dtype, head_dim, page_size, group, window) and group <= ops.FUSED_DECODE_MAX_GROUP
+            and rotary_dim in (0, head_dim))
+
+
+def decode_attention_fused(qkv, q_weight, k_weight, cos, sin, k_cache, v_cache, block_tables, batch, out, *,
+                           num_heads, num_kv_heads, head_dim, rotary_dim, page_size, eps, scale, store) -> bool:
+    """q/k norm, rotation, cache write and attention of a decode-only step in one kernel
+    (plus the merge of the splits, if a token's keys are split)."""
+    split, nsplit = decode_split(batch.num_decode, num_kv_heads, batch.max_decode_len)
+    if ops._profile is not None:
+        keys = sum(c + 1 for c in batch.ctx_lens)
+        ops._note(f"decode {batch.num_decode} tokens, fused", keys * 2 * num_kv_heads * head_dim * 2,
+                  keys * 4.0 * num_heads * head_dim)
+    return ops.attention_decode_fused(
+        qkv, q_weight, k_weight, cos, sin, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token,
+        batch.decode_tokens, batch.num_decode, out, num_heads=num_heads, num_kv_heads=num_kv_heads,
+        head_dim=head_dim, rotary_dim=rotary_dim, page_size=page_size, eps=eps, scale=scale, store=store,
+        split_keys=split, num_splits=nsplit)
+
+
 def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads, num_kv_heads,
                     head_dim, page_size, scale, window=None) -> None:
     """out[n] = softmax(q[n] . K[0..pos_n] * scale) V, per head, over the pages

@@ -112,6 +112,12 @@ _SIGS = {
                               c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
                               c_int, c_int, c_int, c_int, c_float, c_void_p],
     },
+    "attention_fused": {
+        "tk_attention_decode_fused": [c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                      c_float, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                      c_int, c_int, c_float, c_void_p],
+    },
     "sampling": {
         "tk_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
         "tk_argmax_segments": [],
@@ -119,6 +125,7 @@ _SIGS = {
                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     },
 }
+_LIBRARY_FILE = {"attention_fused": "attention_mfma"}   # signature group -> library that holds it
 _fns: dict[str, ctypes._CFuncPtr] = {}
 _profile: "KernelProfile | None" = None
 
@@ -181,7 +188,7 @@ def _fn(library: str, name: str):
     if fn is None:
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: tokamak_amd runs on an MI355X only")
-        lib = load_library(library)
+        lib = load_library(_LIBRARY_FILE.get(library, library))
         fn = getattr(lib, name)
         fn.argtypes = _SIGS[library][name]
         fn.restype = c_int
@@ -508,6 +515,62 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     if status == NOT_INSTANTIATED:
         return False
     _check(status, "attention_mfma")
+    return True
+
+
+FUSED_DECODE_MAX_GROUP = 14   # query heads per kv head the fused decode kernel takes (two waves make the key and value)
+
+
+def attention_decode_fused(qkv: torch.Tensor, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None,
+                           cos: torch.Tensor | None, sin: torch.Tensor | None, k_cache: torch.Tensor,
+                           v_cache: torch.Tensor, block_tables: torch.Tensor, positions: torch.Tensor,
+                           req_of_token: torch.Tensor, item_token: torch.Tensor, num_items: int,
+                           out: torch.Tensor, *, num_heads: int, num_kv_heads: int, head_dim: int,
+                           rotary_dim: int, page_size: int, eps: float, scale: float, store: bool,
+                           split_keys: int, num_splits: int) -> bool:
+    """Decode tokens from the q/k/v projection's output in one kernel: per-head norm and
+    rotation of the queries (and, with ``store``, of the token's key, which is written to
+    its page with the value), then attention over the pages as ``attention_mfma("heads")``.
+    ``qkv``: [N, (nh + 2 nkv) hd] bfloat16, or float32 partial sums [P, N, ...] (without
+    ``store`` the rows hold queries only).  Returns False (nothing launched) if the shape is
+    not instantiated; the caller then runs the two kernels."""
+    _gpu(qkv, q_weight, k_weight, cos, sin, k_cache, v_cache, block_tables, positions, req_of_token, item_token, out)
+    n = positions.numel()
+    nkv_in = num_kv_heads if store else 0
+    width = (num_heads + 2 * nkv_in) * head_dim
+    in_f32, parts, stride = _partials(qkv, n, width, out.dtype, "qkv")
+    _need(qkv.shape[-2] == n, "the fused kernel reads qkv rows by token: one row per token")
+    _need(out.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16,
+          "the fused decode kernel is bfloat16")
+    _need(out.numel() >= n * num_heads * head_dim, "out too small")
+    _need(num_heads % num_kv_heads == 0 and page_size >= 16 and page_size & (page_size - 1) == 0,
+          "bad head counts or page size (a power of two >= 16)")
+    _need(rotary_dim in (0, head_dim), "the fused decode kernel rotates whole heads or not at all")
+    _need(rotary_dim == 0 or (cos is not None and sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32
+                              and cos.numel() >= n * (head_dim // 2) and sin.numel() >= n * (head_dim // 2)
+                              and cos.data_ptr() % 8 == 0 and sin.data_ptr() % 8 == 0), "rotary tables missing or too small")
+    for w in (q_weight, k_weight):
+        _need(w is None or (w.dtype == torch.float32 and w.numel() == head_dim), "q/k norm weights are float32 [head_dim]")
+    _need((q_weight is None) == (k_weight is None), "q and k are normed together or not at all")
+    page_elems = num_kv_heads * head_dim * page_size
+    _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
+    _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32 and block_tables.dtype == torch.int32
+          and item_token.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
+    _need(item_token.numel() >= num_items and 0 < num_items <= 65535, "bad item list")
+    _need(split_keys % 256 == 0 and num_splits >= 1, "splits are multiples of 256 keys")
+    part_o = part_ml = None
+    if num_splits > 1:
+        rows = num_items * num_heads * num_splits
+        part_o = torch.empty((rows, head_dim), dtype=torch.float32, device=out.device)
+        part_ml = torch.empty((rows, 2), dtype=torch.float32, device=out.device)
+    status = _fn("attention_fused", "tk_attention_decode_fused")(
+        _p(qkv), in_f32, parts, stride, _p(q_weight), _p(k_weight), _p(cos), _p(sin), rotary_dim, float(eps), nkv_in,
+        _p(k_cache), _p(v_cache), _p(block_tables), block_tables.shape[1], _p(positions), _p(req_of_token),
+        _p(item_token), num_items, _p(out), _p(part_o), _p(part_ml), num_splits, split_keys, num_heads, num_kv_heads,
+        head_dim, page_size, float(scale), _stream())
+    if status == NOT_INSTANTIATED:
+        return False
+    _check(status, "attention_decode_fused")
     return True
 
 

@@ -6,7 +6,7 @@ import torch
 
 from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels import ops
-from tokamak_amd.kernels.attention import paged_attention
+from tokamak_amd.kernels.attention import decode_attention_fused, fused_decode_fits, paged_attention
 from tokamak_amd.kernels.linear import linear
 from tokamak_amd.parts.base import CacheRequest, Fetch, Mixer, PositionData
 from tokamak_amd.weights.spec import TensorSpec
@@ -82,13 +82,21 @@ class GQAAttention(Mixer):
                                       "it takes rotary tables or no position data")
             cos, sin, rotary_dim = position.cos, position.sin, position.rotary_dim
         tables = batch.block_tables[store.group]
+        attended = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
+        if fused_decode_fits(h.dtype, hd, store.page_size, nh // nkv, self.window, rotary_dim, batch):
+            # a step of decode tokens only: norm, rotation, cache write and attention in one kernel
+            if decode_attention_fused(
+                    qkv, self.q_norm, self.k_norm, cos, sin, store.arrays["k"], store.arrays["v"], tables, batch,
+                    attended, num_heads=nh, num_kv_heads=nkv, head_dim=hd, rotary_dim=rotary_dim,
+                    page_size=store.page_size, eps=self.qk_norm_eps or 0.0, scale=self.softmax_scale,
+                    store=writes_cache):
+                return linear(attended, self.o, allow_partials=True)
         q = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
         ops.qknorm_rope_store(
             qkv, self.q_norm, self.k_norm, cos, sin, batch.positions, batch.req_of_token, tables, q,
             store.arrays["k"], store.arrays["v"], num_heads=nh, num_kv_heads=nkv, head_dim=hd,
             rotary_dim=rotary_dim, page_size=store.page_size,
             eps=self.qk_norm_eps or 0.0, store=writes_cache)
-        attended = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
         paged_attention(q, store.arrays["k"], store.arrays["v"], tables, batch, attended,
                         num_heads=nh, num_kv_heads=nkv, head_dim=hd, page_size=store.page_size,
                         scale=self.softmax_scale, window=self.window)
