@@ -490,6 +490,101 @@ def test_fused_gate_up_silu_product(M, I, K):
 
 
 # ---------------------------------------------------------------------------
+# few rows: the product that adds into the residual stream, and the row scale applied late
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("M, N, K", [(1, 4096, 4096), (8, 4096, 12288), (16, 1000, 264), (5, 100, 72), (3, 64, 2048), (7, 20, 8)])
+@pytest.mark.parametrize("waves", [4, 8, 16])
+def test_whole_k_product_adds_into_the_stream(M, N, K, waves):
+    """resid += x W^T in the product's own kernel, with bf16(resid * gamma) and the rows' sums
+    of squares per slab of 16 columns beside it; rows and columns past the ends (NaN around
+    the operands) are never touched."""
+    from tokamak_amd.kernels import ops
+
+    x = rand(M, K, seed=1).to(torch.bfloat16)
+    w = rand(N, K, seed=2, scale=K ** -0.5).to(torch.bfloat16)
+    stream = rand(M, N, seed=3)
+    gamma = 1 + 0.3 * rand(N, seed=4)
+    want = stream.double() + x.double() @ w.double().T
+    wide = torch.full((M + 2, N + 8), float("nan"), device=DEV)     # the stream as rows of a wider array
+    resid = wide[1:M + 1, 4:N + 4]
+    resid.copy_(stream)
+    sumsq, scaled = ops.gemm_wholek_add(x.to(DEV), w.to(DEV), resid, gamma.to(DEV), waves=waves)
+    torch.testing.assert_close(resid.cpu().double(), want, rtol=1e-3, atol=1e-3)
+    assert torch.isnan(wide[0]).all() and torch.isnan(wide[M + 1]).all() and torch.isnan(wide[:, :4]).all() and torch.isnan(wide[:, N + 4:]).all()
+    torch.testing.assert_close(scaled.cpu().double(), want * gamma.double(), rtol=1e-2, atol=1e-2)
+    assert sumsq.shape == (-(-N // 16), M)
+    torch.testing.assert_close(sumsq.sum(0).cpu().double(), (want ** 2).sum(1), rtol=1e-4, atol=1e-4)
+    slab3 = (want[:, 48:64] ** 2).sum(1) if N >= 64 else None
+    if slab3 is not None:
+        torch.testing.assert_close(sumsq[3].cpu().double(), slab3, rtol=1e-4, atol=1e-4)
+    # without a norm weight: the stream and the sums only
+    resid.copy_(stream)
+    sumsq2, none = ops.gemm_wholek_add(x.to(DEV), w.to(DEV), resid, None, waves=waves)
+    assert none is None and torch.equal(sumsq2, sumsq)
+    # the same call twice gives the same bits (the waves' sums are added in a fixed order)
+    resid.copy_(stream)
+    again, _ = ops.gemm_wholek_add(x.to(DEV), w.to(DEV), resid, gamma.to(DEV), waves=waves)
+    assert torch.equal(again, sumsq)
+
+
+@pytest.mark.parametrize("M, N, K", [(1, 6144, 4096), (8, 4096, 4096), (16, 1000, 264), (5, 100, 72), (3, 2048, 200)])
+def test_products_apply_a_pending_row_scale(M, N, K):
+    """RMSNorm = row scale x column scale; given bf16(x * gamma) and the rows' sums of squares
+    in slabs, the streaming products (plain, split over K, gated) and the whole-K product
+    give what they give on the finished norm.  x is far from unit scale and eps is large
+    enough to matter, so a scale taken without eps, or from K of the wrong matrix, shows."""
+    from tokamak_amd.kernels import ops
+
+    eps = 1e-2
+    x = rand(M, K, seed=1) * 0.05
+    gamma = 1 + 0.3 * rand(K, seed=2)
+    w = rand(N, K, seed=3, scale=K ** -0.5).to(torch.bfloat16)
+    slabs = -(-K // 16)
+    padded = torch.zeros(M, slabs * 16, dtype=torch.float64)
+    padded[:, :K] = x.double()
+    sumsq = (padded.view(M, slabs, 16) ** 2).sum(2).T.contiguous().float()
+    scaled = (x * gamma).to(torch.bfloat16)
+    rstd = torch.rsqrt((x.double() ** 2).mean(1) + eps)
+    want = (scaled.double() * rstd[:, None]) @ w.double().T
+    tol = dict(rtol=2e-3, atol=2e-3 * want.abs().max().item())
+    args = (scaled.to(DEV), w.to(DEV))
+    out = torch.full((M, N), float("nan"), device=DEV)
+    ops.gemm_stream(*args, out, sumsq=sumsq.to(DEV), eps=eps)
+    torch.testing.assert_close(out.cpu().double(), want, **tol)
+    parts = torch.full((3, M, N), float("nan"), device=DEV)
+    used = ops.gemm_stream(*args, parts, splits=3, sumsq=sumsq.to(DEV), eps=eps)
+    torch.testing.assert_close(parts[:used].sum(0).cpu().double(), want, **tol)
+    out = torch.full((M, N), float("nan"), device=DEV)
+    ops.gemm_wholek(*args, out, sumsq=sumsq.to(DEV), eps=eps)
+    torch.testing.assert_close(out.cpu().double(), want, **tol)
+    if N % 2 == 0:
+        half = N // 2
+        g, u = want[:, :half], want[:, half:]
+        gated = g / (1 + torch.exp(-g)) * u
+        gtol = dict(rtol=2e-2, atol=1e-2 * gated.abs().max().item())
+        for fn in (ops.gemm_stream_swiglu, lambda a, b, c, **kw: ops.gemm_wholek(a, b, c, gated=True, **kw)):
+            out = torch.full((M, half), float("nan"), dtype=torch.bfloat16, device=DEV)
+            fn(*args, out, sumsq=sumsq.to(DEV), eps=eps)
+            torch.testing.assert_close(out.cpu().double(), gated, **gtol)
+
+
+def test_fused_forms_refuse_what_they_cannot_take():
+    from tokamak_amd.kernels import ops
+
+    x = torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
+    resid = torch.zeros(17, 64, device=DEV)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_wholek_add(x, w, resid)                      # more than sixteen rows
+    with pytest.raises(ops.KernelError):
+        ops.gemm_wholek_add(x[:4], w[:63], resid[:4, :63])    # N not a multiple of 4
+    with pytest.raises(ops.KernelError):
+        ops.gemm_stream(x, w, torch.zeros(17, 64, device=DEV), sumsq=torch.zeros(4, 17, device=DEV))
+    with pytest.raises(ops.KernelError):
+        ops.gemm_stream(x[:4], w, torch.zeros(4, 64, device=DEV), sumsq=torch.zeros(4, 5, device=DEV))  # sums of other rows
+
+
+# ---------------------------------------------------------------------------
 # decode tokens in one kernel: q/k norm, rotation, cache write and attention
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("nh, nkv, hd, ps", [(32, 8, 128, 16), (6, 3, 64, 32), (14, 1, 128, 16), (3, 3, 128, 64)])

@@ -223,3 +223,49 @@ def test_32b_width_default_pool_leaves_room_for_steps_and_graphs():
     out = runner.step([StepEntry("long", long, [2047])])
     assert torch.isfinite(out).all()
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("use_graphs", [False, True], ids=["eager", "replayed"])
+def test_decode_steps_of_few_requests_over_deep_contexts_at_8b_width(use_graphs, monkeypatch):
+    """bfloat16 decode steps of three requests that hold 40, 700 and 2,300 tokens, at
+    Qwen3-8B's width: the steps in which the o projection adds into the residual stream
+    itself, the gate/up product finishes the norm after it, and the attention kernel makes
+    its own queries and keys.  Eight steps, eager and replayed from a recorded step; every
+    row of logits against the plain implementation."""
+    from tokamak_amd.engine.runner import ModelRunner, StepEntry
+    from tokamak_amd.kernels import ops
+
+    cfg, cfg_json, plan, source, w = shaped("qwen3-8b", on_gpu=True, num_layers=2, vocab_size=4096,
+                                            max_position_embeddings=4096)
+    lengths = [40, 700, 2300]
+    steps = 8
+    calls = {"added": 0, "scaled": 0}
+    add, gated = ops.gemm_wholek_add, ops.gemm_stream_swiglu
+
+    def watched_add(*args, **kwargs):
+        calls["added"] += 1
+        return add(*args, **kwargs)
+
+    def watched_gated(*args, **kwargs):
+        calls["scaled"] += kwargs.get("sumsq") is not None
+        return gated(*args, **kwargs)
+
+    monkeypatch.setattr(ops, "gemm_wholek_add", watched_add)
+    monkeypatch.setattr(ops, "gemm_stream_swiglu", watched_gated)
+    runner = ModelRunner(plan, source, dtype="bfloat16", page_size=16, kv_pool_tokens=3200, max_requests=3,
+                         use_graphs=use_graphs)
+    ids = [random_ids(cfg.vocab_size, t + steps, 40 + i) for i, t in enumerate(lengths)]
+    for r, t in enumerate(lengths):
+        for at in range(0, t, 2048):
+            runner.step([StepEntry(r, ids[r][at:min(t, at + 2048)], [])])
+    assert calls == {"added": 0, "scaled": 0}, "portions of prompts take the kernels for many rows"
+    want = [plain.logits(x, cfg_json, w) for x in ids]
+    for i in range(steps):
+        got = runner.step([StepEntry(r, [ids[r][t + i]], [0]) for r, t in enumerate(lengths)]).cpu()
+        for r, t in enumerate(lengths):
+            err = float((got[r] - want[r][t + i]).abs().max())
+            assert err <= tolerance("bfloat16", want[r][t + i]), f"step {i}, request {r}: {err}"
+    assert bool(runner._graphs) == use_graphs
+    assert calls["added"] >= cfg.num_layers and calls["scaled"] == calls["added"], \
+        "the decode steps did not take the products that add into the stream"
+    runner.manager.check()

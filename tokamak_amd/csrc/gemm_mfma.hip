@@ -228,10 +228,23 @@ constexpr int SLD = SBK + 8;    // LDS row stride in elements
 // A second chunk of weights in flight per wave was measured too and gained nothing: at 64
 // rows the kernel is held by LDS traffic (seven bytes through LDS per byte of weights),
 // at 16 rows and fewer by the launch and drain of blocks that live for a few microseconds.
+//
+// RowScale (up to 16 rows): the activations may be given as bf16(x * gamma) of an RMSNorm whose
+// row statistics are not applied yet (what the product that adds into the residual stream
+// leaves, gemm_wholek.hip); the product is linear in a row's scale, so the block multiplies
+// row m of its sums by rstd[m] = rsqrt(sum_s sumsq[s][m] / K + eps) before it stores them
+// (partial sums of a split too: their sum is scaled alike) or gates them.
+constexpr int kRowScaleLoads = 32;  // slab sums a thread of a four-wave block holds: slabs <= 16 * this
+struct RowScale {
+  const float* sumsq;  // [slabs][M]: sums of squares of the rows over slabs of columns; nullptr: no scaling
+  int slabs;
+  float eps;
+};
+
 template <int MT, typename TO, bool GATED, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TO* __restrict__ C, int M, int N,
-    int K, long lda, long ldw, long ldc, int chunks_per_split, long split_stride) {
+    int K, long lda, long ldw, long ldc, int chunks_per_split, long split_stride, RowScale scale) {
   constexpr int THREADS = WAVES * 64;
   constexpr int XP = 16 * MT * 32 / THREADS;  // 16-byte pieces of the activations a thread loads per chunk
   static_assert(XP * THREADS == 16 * MT * 32, "the activations' chunk divides among the threads");
@@ -271,6 +284,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
   float4v acc[MT];
 #pragma unroll
   for (int j = 0; j < MT; ++j) acc[j] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  // RowScale: thread (row tid % 16, group tid / 16) adds its share of the row's slab sums;
+  // they meet in LDS behind the walk's barriers and are added in group order at the end.
+  __shared__ float s_stat[MT == 1 ? THREADS : 1];
+  const bool scaled = MT == 1 && scale.sumsq != nullptr;
 
 #define TK_FETCH_W(C_)                                                                              \
   {                                                                                                 \
@@ -327,6 +345,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
     TK_FETCH_W(first_)
     TK_FETCH_X(first_)
   }
+  // RowScale: the slab sums are asked for now and first looked at after the walk over K (a
+  // block that waited for them here would start its walk a memory round trip late).
+  constexpr int STAT_STEP = THREADS / 16;
+  float stat[MT == 1 ? kRowScaleLoads : 1];
+  if constexpr (MT == 1) {
+#pragma unroll
+    for (int u = 0; u < kRowScaleLoads; ++u) stat[u] = 0.f;
+    if (scaled && (tid & 15) < M) {
+#pragma unroll
+      for (int u = 0; u < kRowScaleLoads; ++u) {
+        const int sl = (tid >> 4) + u * STAT_STEP;
+        if (sl < scale.slabs) stat[u] = scale.sumsq[(size_t)sl * M + (tid & 15)];
+      }
+    }
+  }
   for (int i = 0; i < nchunks; ++i) TK_CHUNK(i)
 #undef TK_CHUNK
 #undef TK_FETCH_X
@@ -335,6 +368,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
   // With several splits, split s writes its partial sums to C + s * split_stride; whoever
   // reads C next adds the splits (in split order, so the sum is deterministic).
   C += (size_t)split * split_stride;
+
+  if constexpr (MT == 1) {
+    if (scaled) {
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < kRowScaleLoads; ++u) ss += stat[u];
+      s_stat[tid] = ss;
+      __syncthreads();
+      float total = 0.f;
+#pragma unroll
+      for (int grp = 0; grp < THREADS / 16; ++grp) total += s_stat[grp * 16 + r];
+      acc[0] *= rsqrtf(total / (float)K + scale.eps);
+    }
+  }
 
   if (GATED) {
     float* up = reinterpret_cast<float*>(&ws[0][0][0]);  // [HALF up waves][MT][64 lanes][4]
@@ -374,14 +421,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
 template <typename TO, bool GATED, int WAVES>
 static int launch_stream_shape(const void* A, const void* W, void* C, int M, int N, int K, long lda,
                                long ldw, long ldc, int chunks_per_split, int KS, long split_stride,
-                               hipStream_t stream) {
+                               RowScale scale, hipStream_t stream) {
   const int cols = GATED ? 8 * WAVES : 16 * WAVES;
   dim3 grid((N + cols - 1) / cols, KS);
   const int mt = (M + 15) / 16;
 #define TK_STREAM(MT_)                                                                          \
   gemm_stream_kernel<MT_, TO, GATED, WAVES><<<grid, WAVES * 64, 0, stream>>>(            \
       (const bf16_t*)A, (const bf16_t*)W, (TO*)C, M, N, K, lda, ldw, ldc, chunks_per_split,     \
-      split_stride)
+      split_stride, scale)
   if (mt == 1) TK_STREAM(1);
   else if (mt == 2) TK_STREAM(2);
   else if (mt == 3) TK_STREAM(3);
@@ -393,36 +440,43 @@ static int launch_stream_shape(const void* A, const void* W, void* C, int M, int
 // waves: 4 or 8 a block.
 template <typename TO, bool GATED>
 static int launch_stream(int waves, const void* A, const void* W, void* C, int M, int N, int K,
-                         long lda, long ldw, long ldc, int cps, int KS, long split_stride, hipStream_t stream) {
+                         long lda, long ldw, long ldc, int cps, int KS, long split_stride, RowScale scale,
+                         hipStream_t stream) {
   if (waves >= 8)
-    return launch_stream_shape<TO, GATED, 8>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, stream);
-  return launch_stream_shape<TO, GATED, 4>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, stream);
+    return launch_stream_shape<TO, GATED, 8>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, scale, stream);
+  return launch_stream_shape<TO, GATED, 4>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, scale, stream);
 }
 
 // out_dtype: 0 float32, 1 bfloat16.  M <= 64; K a multiple of 8; rows 16-byte aligned.
 // waves: 4 or 8 waves a block.  splits: shares of K.  With splits > 1 the output must be float32 and C holds
 // `splits` partial results, split_stride elements apart, that the reader adds.
+// sumsq (may be null), slabs, eps: the rows' scale, see RowScale; then M <= 16.
 // Returns the number of splits actually used (<= splits; no split is empty), or < 0.
 TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, int M, int N, int K,
                           long lda, long ldw, long ldc, int splits, long split_stride, int waves,
-                          hipStream_t stream) {
+                          const float* sumsq, int slabs, float eps, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535) return -1;
+  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > 16 * kRowScaleLoads || waves >= 8)) return -1;
+  const RowScale scale{sumsq, slabs, eps};
   if (splits > 1 && out_dtype != 0) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
   const int cps = (total_chunks + splits - 1) / splits;
   const int ks = (total_chunks + cps - 1) / cps;
   int status = -1;
-  if (out_dtype == 0) status = launch_stream<float, false>(waves, A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
-  if (out_dtype == 1) status = launch_stream<bf16_t, false>(waves, A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, stream);
+  if (out_dtype == 0) status = launch_stream<float, false>(waves, A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, scale, stream);
+  if (out_dtype == 1) status = launch_stream<bf16_t, false>(waves, A, W, C, M, N, K, lda, ldw, ldc, cps, ks, split_stride, scale, stream);
   return status == 0 ? ks : (status > 0 ? -status : status);
 }
 
 // C[M, N] = silu(A W_gate^T) * (A W_up^T) with W = [W_gate; W_up] of 2N rows; bfloat16 out.
 TK_API int tk_gemm_stream_swiglu(const void* A, const void* W, void* C, int M, int N, int K, long lda,
-                                 long ldw, long ldc, int waves, hipStream_t stream) {
+                                 long ldw, long ldc, int waves, const float* sumsq, int slabs, float eps,
+                                 hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
+  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > 16 * kRowScaleLoads || waves >= 8)) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
-  return launch_stream<bf16_t, true>(waves, A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0, stream);
+  return launch_stream<bf16_t, true>(waves, A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0,
+                                     RowScale{sumsq, slabs, eps}, stream);
 }

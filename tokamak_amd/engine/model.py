@@ -9,6 +9,7 @@ import torch
 from tokamak_amd.cache.pages import CacheGroupSpec
 from tokamak_amd.config.model_config import ModelPlan, PartSpec
 from tokamak_amd.config.registry import get_part
+from tokamak_amd.kernels.linear import Added
 from tokamak_amd.parts.base import Block, CacheRequest, Part, StateArray
 from tokamak_amd.weights.spec import TensorSpec
 
@@ -138,10 +139,20 @@ class LayeredModel:
     def forward(self, batch, storage) -> torch.Tensor:
         resid = self.embedding.forward(batch)
         pending = None
-        for call in self.plan.order:
-            pending = self.blocks[call.layer].forward(
-                resid, pending, batch, storage.slot(call.cache), call.writes_cache)
+        order = self.plan.order
+        for at, call in enumerate(order):
+            block = self.blocks[call.layer]
+            if block.fuses_residual:
+                # the norm that reads the stream after this block: its last product may prepare for it
+                then = self.blocks[order[at + 1].layer].entry_norm if at + 1 < len(order) else self.final_norm
+                pending = block.forward(resid, pending, batch, storage.slot(call.cache), call.writes_cache, then=then)
+            else:
+                if isinstance(pending, Added):
+                    pending = None      # the sum is in the stream already
+                pending = block.forward(resid, pending, batch, storage.slot(call.cache), call.writes_cache)
         if batch.num_logit_rows == 0:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
+        if isinstance(pending, Added) and not self.final_norm.fuses_residual:
+            pending = None
         h = self.final_norm.forward(resid, pending, rows=batch.logit_rows, write_resid=False)
         return self.head.forward(h)

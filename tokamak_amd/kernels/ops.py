@@ -92,11 +92,18 @@ _SIGS = {
     },
     "gemm_mfma": {
         "tk_gemm_stream": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
-                           c_long, c_int, c_long, c_int, c_void_p],
+                           c_long, c_int, c_long, c_int, c_void_p, c_int, c_float, c_void_p],
         "tk_gemm_stream_swiglu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long,
-                                  c_int, c_void_p],
+                                  c_int, c_void_p, c_int, c_float, c_void_p],
         "tk_gemm_skinny": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
                            c_long, c_int, c_int, c_void_p],
+    },
+    "gemm_wholek": {
+        "tk_gemm_wholek": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long,
+                           c_void_p, c_int, c_float, c_int, c_void_p],
+        "tk_gemm_wholek_slabs": [c_int],
+        "tk_gemm_wholek_add": [c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_void_p, c_long, c_void_p,
+                               c_void_p, c_long, c_void_p, c_int, c_void_p],
     },
     "blas_lt": {
         "tk_lt_gemm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p,
@@ -335,12 +342,26 @@ def stream_waves(rows: int, k: int, gated: bool = False) -> int:
     return 8 if rows > 32 and (gated or k >= 8192) else 4
 
 
-def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: int = 1, waves: int = 0) -> int:
+def _row_scale(sumsq: torch.Tensor | None, m: int, what: str) -> int:
+    """Checks the rows' sums of squares [slabs, M] that a product scales its result by; slabs."""
+    if sumsq is None:
+        return 0
+    _gpu(sumsq)
+    _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.shape[0] >= 1
+          and m <= ROW_SCALE_MAX_ROWS, f"{what}: the rows' sums of squares are float32 [slabs, M], M <= {ROW_SCALE_MAX_ROWS}")
+    return sumsq.shape[0]
+
+
+def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: int = 1, waves: int = 0,
+                sumsq: torch.Tensor | None = None, eps: float = 0.0) -> int:
     """out = a[M, K] @ w[N, K]^T for M <= 64 with the LDS-staged weight-streaming
     MFMA kernel (``waves``: 4 or 8 waves a block; 0 chooses by M).  ``splits == 1``: out is
     [M, N], bfloat16 or float32.  More:
     out is float32 [splits, M, N] and receives partial sums; returns how many of
-    them were written (the reader adds out[:returned])."""
+    them were written (the reader adds out[:returned]).  ``sumsq`` [slabs, M] (M <= 16): row m
+    of the result is multiplied by rsqrt(sum_s sumsq[s, m] / K + eps): ``a`` is then
+    bf16(x * gamma) of an RMSNorm and ``sumsq`` the sums of squares of x's rows over slabs of
+    columns (``gemm_wholek_add`` leaves both)."""
     for t in (a, w):
         _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
     m, k = a.shape
@@ -357,17 +378,21 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
         _need(1 < splits <= 64 and out.dtype == torch.float32 and out.shape == (splits, m, n) and out.is_contiguous(),
               "with splits the output is contiguous float32 [splits, M, N]")
         ldc, stride = n, m * n
+    slabs = _row_scale(sumsq, m, "gemm_stream")
     _note(f"{m}x{n}x{k}", (n * k + m * k) * 2 + splits * m * n * out.element_size(), 2.0 * m * n * k)
     used = _fn("gemm_mfma", "tk_gemm_stream")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
-                                              w.stride(0), ldc, splits, stride, waves or stream_waves(m, k), _stream())
+                                              w.stride(0), ldc, splits, stride, waves or stream_waves(m, k),
+                                              _p(sumsq), slabs, float(eps), _stream())
     if used < 1:
         raise KernelError(f"gemm_stream failed with status {used}")
     return used
 
 
-def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, waves: int = 0) -> None:
+def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, waves: int = 0,
+                       sumsq: torch.Tensor | None = None, eps: float = 0.0) -> None:
     """out[M, I] = silu(a @ w[:I]^T) * (a @ w[I:]^T) for M <= 64: the gate and up
-    projections and the SiLU product in one weight-streaming kernel (bfloat16)."""
+    projections and the SiLU product in one weight-streaming kernel (bfloat16).  ``sumsq``,
+    ``eps``: the rows' scale, applied to both products before the gate, as in ``gemm_stream``."""
     for t in (a, w, out):
         _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
     m, k = a.shape
@@ -375,9 +400,81 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, w
     _need(a.dtype == w.dtype == out.dtype == torch.bfloat16, "the gated product is bfloat16")
     _need(0 < m <= 64 and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gated product needs M <= 64 and 16-byte aligned rows")
+    slabs = _row_scale(sumsq, m, "gemm_stream_swiglu")
     _note(f"{m}x{w.shape[0]}x{k}", (w.shape[0] * k + m * k) * 2 + m * w.shape[0], 2.0 * m * w.shape[0] * k)
     _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
-                                                     w.stride(0), out.stride(0), waves or stream_waves(m, k, True), _stream()), "gemm_stream_swiglu")
+                                                     w.stride(0), out.stride(0), waves or stream_waves(m, k, True),
+                                                     _p(sumsq), slabs, float(eps), _stream()), "gemm_stream_swiglu")
+
+
+WHOLEK_MAX_ROWS = 16    # rows of activations that the whole-K product takes
+ROW_SCALE_MAX_ROWS = 16  # rows up to which the streaming product applies a pending row scale
+
+
+def wholek_waves(n: int, k: int, gated: bool = False) -> int:
+    """Waves a block of the whole-K product: they split K in chunks of 256."""
+    chunks = -(-k // 256)
+    if gated:
+        return 4 if chunks <= 16 else 8
+    return 16 if chunks >= 16 else 8 if chunks >= 8 else 4
+
+
+def _wholek_operands(a, w, what):
+    for t in (a, w):
+        _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1 and t.dtype == torch.bfloat16,
+              f"{what}: operands are 2-D bfloat16 GPU tensors with unit inner stride")
+    m, k = a.shape
+    _need(w.shape[1] == k, f"{what}: shapes disagree")
+    _need(0 < m <= WHOLEK_MAX_ROWS and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+          and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0,
+          f"{what} needs M <= {WHOLEK_MAX_ROWS}, K a multiple of 8 and 16-byte aligned rows")
+    return m, k
+
+
+def gemm_wholek(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, sumsq: torch.Tensor | None = None,
+                eps: float = 0.0, gated: bool = False, waves: int = 0) -> None:
+    """out[M, N] = (a[M, K] @ w[N, K]^T) * rstd for M <= 16, every block holding the whole of K
+    for its 16 columns (no partial sums).  ``sumsq`` [slabs, M] float32: sums of squares of the
+    rows of the stream that ``a`` was made from, over slabs of its columns; then
+    rstd[m] = rsqrt(sum_s sumsq[s, m] / K + eps) (an RMSNorm whose weight is already in ``a``);
+    without it rstd = 1.  ``gated``: w = [gate; up] of 2N rows and out = silu(.) * (.), bfloat16."""
+    m, k = _wholek_operands(a, w, "gemm_wholek")
+    n = w.shape[0] // 2 if gated else w.shape[0]
+    _need(not gated or (w.shape[0] % 2 == 0 and out.dtype == torch.bfloat16), "the gated product has 2N weight rows and a bfloat16 result")
+    _need(out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and out.shape == (m, n), "output must be [M, N] on the GPU")
+    if sumsq is not None:
+        _gpu(sumsq)
+        _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.shape[0] >= 1,
+              "the rows' sums of squares are float32 [slabs, M]")
+    _note(f"{m}x{w.shape[0]}x{k}", (w.shape[0] * k + m * k) * 2 + m * n * out.element_size(), 2.0 * m * w.shape[0] * k)
+    _check(_fn("gemm_wholek", "tk_gemm_wholek")(
+        _code(out.dtype), int(gated), _p(a), _p(w), _p(out), m, n, k, a.stride(0), w.stride(0), out.stride(0),
+        _p(sumsq), 0 if sumsq is None else sumsq.shape[0], float(eps), waves or wholek_waves(n, k, gated), _stream()),
+        "gemm_wholek")
+
+
+def gemm_wholek_add(a: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gamma: torch.Tensor | None = None,
+                    *, waves: int = 0) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """resid[M, N] += a[M, K] @ w[N, K]^T (float32 stream, M <= 16) in the product's own kernel.
+    Returns (sumsq, scaled): sumsq float32 [N/16, M], the sums of squares of every row of the new
+    stream over slabs of 16 columns, and, given ``gamma`` [N] (the weight of the norm that reads
+    the stream next), scaled = bf16(resid * gamma) [M, N]: what ``gemm_wholek`` takes."""
+    m, k = _wholek_operands(a, w, "gemm_wholek_add")
+    n = w.shape[0]
+    _need(resid.is_cuda and resid.dtype == torch.float32 and resid.shape == (m, n) and resid.stride(1) == 1
+          and n % 4 == 0 and resid.stride(0) % 4 == 0 and resid.data_ptr() % 16 == 0,
+          "the stream is float32 [M, N], N a multiple of 4, rows 16-byte aligned")
+    scaled = None
+    if gamma is not None:
+        _gpu(gamma)
+        _need(gamma.dtype == torch.float32 and gamma.numel() == n and gamma.data_ptr() % 16 == 0, "the norm weight is float32 [N]")
+        scaled = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    sumsq = torch.empty((-(-n // 16), m), dtype=torch.float32, device=a.device)
+    _note(f"{m}x{n}x{k}", (n * k + m * k) * 2 + m * n * 10, 2.0 * m * n * k)
+    _check(_fn("gemm_wholek", "tk_gemm_wholek_add")(
+        _p(a), _p(w), m, n, k, a.stride(0), w.stride(0), _p(resid), resid.stride(0), _p(gamma), _p(scaled),
+        0 if scaled is None else scaled.stride(0), _p(sumsq), waves or wholek_waves(n, k), _stream()), "gemm_wholek_add")
+    return sumsq, scaled
 
 
 LT_WORKSPACE_BYTES = 128 << 20

@@ -25,6 +25,7 @@ class GQAAttention(Mixer):
     """
 
     capturable = True
+    fuses_residual = True
 
     def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qk_norm_eps: float | None, softmax_scale: float, window: int | None,
@@ -68,8 +69,8 @@ class GQAAttention(Mixer):
         width = self.num_kv_heads * self.head_dim
         return CacheRequest.of(window=self.window, k=width, v=width)
 
-    def forward(self, h: torch.Tensor, batch, store, writes_cache: bool = True,
-                position: PositionData | None = None) -> torch.Tensor:
+    def forward(self, h, batch, store, writes_cache: bool = True,
+                position: PositionData | None = None, add_into=None):
         nh, nkv, hd = self.num_heads, self.num_kv_heads, self.head_dim
         n = h.shape[0]
         weight = self.qkv if writes_cache else self.qkv[: nh * hd]
@@ -90,7 +91,7 @@ class GQAAttention(Mixer):
                     attended, num_heads=nh, num_kv_heads=nkv, head_dim=hd, rotary_dim=rotary_dim,
                     page_size=store.page_size, eps=self.qk_norm_eps or 0.0, scale=self.softmax_scale,
                     store=writes_cache):
-                return linear(attended, self.o, allow_partials=True)
+                return linear(attended, self.o, allow_partials=True, add_into=add_into)
         q = torch.empty((n, nh * hd), dtype=h.dtype, device=h.device)
         ops.qknorm_rope_store(
             qkv, self.q_norm, self.k_norm, cos, sin, batch.positions, batch.req_of_token, tables, q,
@@ -100,7 +101,7 @@ class GQAAttention(Mixer):
         paged_attention(q, store.arrays["k"], store.arrays["v"], tables, batch, attended,
                         num_heads=nh, num_kv_heads=nkv, head_dim=hd, page_size=store.page_size,
                         scale=self.softmax_scale, window=self.window)
-        return linear(attended, self.o, allow_partials=True)
+        return linear(attended, self.o, allow_partials=True, add_into=add_into)
 
 
 register_part("mixer", "gqa_attention", GQAAttention)

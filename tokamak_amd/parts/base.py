@@ -46,6 +46,17 @@ class Part:
     """
 
     capturable = False
+    # Whether the part takes part in the fusion of the residual add and the norm into the
+    # products around them (kernels/linear.py).  A norm that says so takes ``Added`` as its
+    # ``delta`` (the sum is already in the stream) and a keyword ``defer`` (it may then
+    # return a ``DeferredNorm`` instead of a tensor), and offers ``sink(resid)``.  A mixer or
+    # feed-forward that says so takes a ``DeferredNorm`` as its input ``h`` (it hands it to
+    # ``linear`` / ``gated_linear`` only, before the stream is written again) and a keyword
+    # ``add_into``: a ``StreamSink`` for its last product, whose ``Added`` it returns.  A
+    # block that says so takes ``Added`` as ``pending``, a keyword ``then`` (the norm that
+    # reads the stream after the block, or None) and names its first norm ``entry_norm``.
+    # Parts that do not say so never meet these types.
+    fuses_residual = False
 
     def __init__(self, *, dtype: torch.dtype, device: torch.device | str) -> None:
         self.dtype = dtype
@@ -169,6 +180,8 @@ class Block:
 
     roles: tuple[str, ...] = ()
     optional: tuple[str, ...] = ()
+    fuses_residual = False      # see Part.fuses_residual
+    entry_norm: "Norm | None" = None   # the norm that reads the stream first, if the block fuses
 
     def __init__(self, parts: dict[str, Part]) -> None:
         missing = [r for r in self.roles if r not in parts]

@@ -19,6 +19,7 @@ class SwiGLU(FeedForward):
     """
 
     capturable = True
+    fuses_residual = True
 
     def __init__(self, *, hidden_size: int, intermediate_size: int, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)
@@ -39,8 +40,8 @@ class SwiGLU(FeedForward):
         self.gate_up = torch.cat([fetch(prefix + "gate_proj.weight"), fetch(prefix + "up_proj.weight")], dim=0).contiguous()
         self.down = fetch(prefix + "down_proj.weight")
 
-    def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
-        return linear(gated_linear(h, self.gate_up), self.down, allow_partials=True)
+    def forward(self, h, batch, add_into=None):
+        return linear(gated_linear(h, self.gate_up), self.down, allow_partials=True, add_into=add_into)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

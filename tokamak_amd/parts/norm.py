@@ -6,6 +6,7 @@ import torch
 
 from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels import ops
+from tokamak_amd.kernels.linear import Added, DeferredNorm, StreamSink
 from tokamak_amd.parts.base import Fetch, Norm
 from tokamak_amd.weights.spec import TensorSpec
 
@@ -19,6 +20,7 @@ class RMSNorm(Norm):
     """
 
     capturable = True
+    fuses_residual = True
 
     def __init__(self, *, dim: int, eps: float, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)
@@ -32,7 +34,16 @@ class RMSNorm(Norm):
     def bind(self, prefix: str, fetch: Fetch) -> None:
         self.weight = fetch(prefix + "weight")
 
-    def forward(self, resid, delta, *, rows=None, write_resid=True):
+    def sink(self, resid: torch.Tensor) -> StreamSink:
+        return StreamSink(resid, self.weight)
+
+    def forward(self, resid, delta, *, rows=None, write_resid=True, defer=False):
+        if isinstance(delta, Added):
+            # the product before has added into the stream; if it has left the stream times
+            # this norm's weight, the product after may finish the norm
+            if defer and rows is None and delta.scaled is not None and delta.gamma is self.weight:
+                return DeferredNorm(resid, self.weight, self.eps, self.dtype, delta.scaled, delta.sumsq)
+            delta = None
         m = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((m, self.dim), dtype=self.dtype, device=resid.device)
         ops.add_rmsnorm(resid, delta, self.weight, self.eps, out, rows=rows, write_resid=write_resid)
