@@ -69,10 +69,19 @@ __device__ __forceinline__ void decode_head_vector(const DecodeInputs& in, size_
   x0 = x1 = 0.f;
   if (in.in_f32) {
     const float* src = static_cast<const float*>(in.qkv) + row_offset + (size_t)head_col * HD + d;
-    for (int p = 0; p < in.parts; ++p) {
-      const float2 v = *reinterpret_cast<const float2*>(src + (size_t)p * in.part_stride);
-      x0 += v.x;
-      x1 += v.y;
+    // four partial sums in flight at a time (a chain of dependent loads would cost a memory
+    // round trip each); added in split order
+    for (int p = 0; p < in.parts; p += 4) {
+      float2 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        v[u] = p + u < in.parts ? *reinterpret_cast<const float2*>(src + (size_t)(p + u) * in.part_stride)
+                                : make_float2(0.f, 0.f);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        x0 += v[u].x;
+        x1 += v[u].y;
+      }
     }
   } else {
     const uint32_t v = *reinterpret_cast<const uint32_t*>(static_cast<const bf16_t*>(in.qkv) + row_offset +
@@ -141,6 +150,40 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
   const int c_head = kvh * G + col;
   const bool c_valid = col < G;
 
+  // The wave's first tiles are asked for before anything else: they depend on the block
+  // table only, and the queries (which the fused form first has to make) are needed when
+  // they arrive.
+  Frag8 kreg[D][KCH];
+  Frag4 vreg[D][DBL];
+#define TK_TILE_ADDR(T_)                                                  \
+    const int c0_ = k_begin + (T_) * 16;                                    \
+    const int page_ = table[c0_ / ps];                                      \
+    const int off_ = c0_ % ps;
+#define TK_LOAD_K(SLOT_, T_)                                                                          \
+  {                                                                                                   \
+    TK_TILE_ADDR(T_)                                                                                  \
+    const bf16_t* kp_ = k_cache + (size_t)page_ * page_elems + head_off + (size_t)(off_ + col) * 8;   \
+    _Pragma("unroll") for (int c = 0; c < KCH; ++c) kreg[SLOT_][c].w = __builtin_nontemporal_load(    \
+        reinterpret_cast<const u32x4*>(kp_ + (size_t)(c * 4 + kb) * ps * 8));                         \
+  }
+  // V page [hd/16][ps/4][16][4]: lane (dim col, quad kb) of block d reads 8 bytes, the wave 512
+  // contiguous bytes
+#define TK_LOAD_V(SLOT_, T_)                                                                          \
+  {                                                                                                   \
+    TK_TILE_ADDR(T_)                                                                                  \
+    const bf16_t* vp_ =                                                                               \
+        v_cache + (size_t)page_ * page_elems + head_off + (size_t)((off_ >> 2) + kb) * 64 + col * 4;  \
+    _Pragma("unroll") for (int d = 0; d < DBL; ++d) vreg[SLOT_][d].w = __builtin_nontemporal_load(    \
+        reinterpret_cast<const u32x2*>(vp_ + (size_t)d * (ps >> 2) * 64));                            \
+  }
+
+#pragma unroll
+  for (int i = 0; i < D; ++i)
+    if (t_begin + i < t_end) {
+      TK_LOAD_K(i, t_begin + i)
+      TK_LOAD_V(i, t_begin + i)
+    }
+
   // Q as B operand: lane (col, kb) holds Q[col][c*32 + kb*8 .. +8]
   bf16x8 qreg[KCH];
   bool stores = false;    // FUSED: this call stores the token's key and value
@@ -193,37 +236,6 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
   float4v acc[DBL];
 #pragma unroll
   for (int d = 0; d < DBL; ++d) acc[d] = float4v{0.f, 0.f, 0.f, 0.f};
-
-  Frag8 kreg[D][KCH];
-  Frag4 vreg[D][DBL];
-#define TK_TILE_ADDR(T_)                                                  \
-    const int c0_ = k_begin + (T_) * 16;                                    \
-    const int page_ = table[c0_ / ps];                                      \
-    const int off_ = c0_ % ps;
-#define TK_LOAD_K(SLOT_, T_)                                                                          \
-  {                                                                                                   \
-    TK_TILE_ADDR(T_)                                                                                  \
-    const bf16_t* kp_ = k_cache + (size_t)page_ * page_elems + head_off + (size_t)(off_ + col) * 8;   \
-    _Pragma("unroll") for (int c = 0; c < KCH; ++c) kreg[SLOT_][c].w = __builtin_nontemporal_load(    \
-        reinterpret_cast<const u32x4*>(kp_ + (size_t)(c * 4 + kb) * ps * 8));                         \
-  }
-  // V page [hd/16][ps/4][16][4]: lane (dim col, quad kb) of block d reads 8 bytes, the wave 512
-  // contiguous bytes
-#define TK_LOAD_V(SLOT_, T_)                                                                          \
-  {                                                                                                   \
-    TK_TILE_ADDR(T_)                                                                                  \
-    const bf16_t* vp_ =                                                                               \
-        v_cache + (size_t)page_ * page_elems + head_off + (size_t)((off_ >> 2) + kb) * 64 + col * 4;  \
-    _Pragma("unroll") for (int d = 0; d < DBL; ++d) vreg[SLOT_][d].w = __builtin_nontemporal_load(    \
-        reinterpret_cast<const u32x2*>(vp_ + (size_t)d * (ps >> 2) * 64));                            \
-  }
-
-#pragma unroll
-  for (int i = 0; i < D; ++i)
-    if (t_begin + i < t_end) {
-      TK_LOAD_K(i, t_begin + i)
-      TK_LOAD_V(i, t_begin + i)
-    }
 
   for (int t0 = t_begin; t0 < t_end; t0 += D) {
 #pragma unroll
