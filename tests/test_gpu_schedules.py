@@ -269,3 +269,54 @@ def test_decode_steps_of_few_requests_over_deep_contexts_at_8b_width(use_graphs,
     assert calls["added"] >= cfg.num_layers and calls["scaled"] == calls["added"], \
         "the decode steps did not take the products that add into the stream"
     runner.manager.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_launched_from_a_recorded_layer_give_the_same_bits(dtype):
+    """Steps that are not replayed from a graph record the launches of one layer of a kind
+    and launch the others from the list.  Against the same steps with every layer run as
+    written: equal bits of every logit, step after step (portions of two requests beside a
+    decode token, a whole prompt, decode steps of few rows with their fused products, a
+    step of 70 tokens), and the same cache afterwards; and the list was in fact used."""
+    from tokamak_amd.engine import layer_replay
+    from tokamak_amd.engine.runner import ModelRunner, StepEntry
+
+    cfg, cfg_json, plan, source, w = shaped("qwen3-0.6b", on_gpu=True, num_layers=5, vocab_size=2048,
+                                            max_position_embeddings=1024)
+    ids = [random_ids(cfg.vocab_size, 400, 70 + i) for i in range(4)]
+    launched = []
+    launch = layer_replay.LayerRecording.launch
+
+    def run(replay):
+        runner = ModelRunner(plan, source, dtype=dtype, page_size=16, kv_pool_tokens=2048, max_requests=4, use_graphs=False)
+        runner.model.replay_layers = replay
+        out = []
+        out.append(runner.step([StepEntry(0, ids[0][:150], [149])]))
+        out.append(runner.step([StepEntry(1, ids[1][:90], [0, 89]), StepEntry(0, ids[0][150:151], [0]),
+                                StepEntry(2, ids[2][:37], [])]))
+        out.append(runner.step([StepEntry(r, ids[r][n:n + 1], [0]) for r, n in ((0, 151), (1, 90), (2, 37))]))
+        out.append(runner.step([StepEntry(3, ids[3][:70], [69])]))
+        out.append(runner.step([StepEntry(2, ids[2][38:40], [1]), StepEntry(3, ids[3][70:73], [2])]))
+        torch.cuda.synchronize()
+        cache = [a.clone() for slot in sorted(runner.storage._slots) for a in runner.storage.slot(slot).arrays.values()]
+        return [o.cpu() for o in out], cache
+
+    def counted(self, tensors, then):
+        launched.append(len(self.calls))
+        return launch(self, tensors, then)
+
+    plainly, cache_plain = run(False)
+    try:
+        layer_replay.LayerRecording.launch = counted
+        replayed, cache_replayed = run(True)
+    finally:
+        layer_replay.LayerRecording.launch = launch
+    assert len(launched) == 5 * (cfg.num_layers - 2), "three of five layers of every step are launched from the list"
+    assert min(launched) >= 5
+    for step, (a, b) in enumerate(zip(plainly, replayed)):
+        assert torch.equal(a, b), f"step {step}: {float((a - b).abs().max())}"
+    for a, b in zip(cache_plain, cache_replayed):
+        assert torch.equal(a, b)
+    want = plain.logits(ids[0][:152], cfg_json, w)
+    err = float((replayed[2][0] - want[151]).abs().max())
+    assert err <= tolerance(dtype, want[151]), err

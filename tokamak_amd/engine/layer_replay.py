@@ -1,0 +1,119 @@
+"""Layers of one kind launch the same kernels in a step: record one, replay the others.
+
+A step that is not replayed from a HIP graph (prompt portions, more requests than the
+recorded shapes take) pays for every kernel launch in Python: checks of shapes and dtypes,
+the choice of a kernel, allocations.  Within a step all of that is the same for every
+layer of one kind; only the addresses of the layer's own tensors differ.  So the first
+layer of a kind that meets a given kind of input runs as written while its launches are
+listed (``kernels.ops.recording``), and every later layer of that kind launches from the
+list, with the addresses of its own weights, cache arrays, incoming sub-layer output and
+following norm in place of the recorded layer's.  Everything else the recorded layer
+allocated is kept until the step ends and used again: layers run one after the other on
+one stream, so a buffer a layer has finished with is free for the next.
+
+A block takes part only if it says ``replayable``: its parts launch all their work through
+``kernels.ops`` and decide nothing from values that differ between layers of a kind.
+"""
+
+from __future__ import annotations
+
+import bisect
+import dataclasses
+from ctypes import c_void_p
+from dataclasses import dataclass
+
+import torch
+
+from tokamak_amd.kernels import ops
+from tokamak_amd.kernels.linear import Added
+
+
+def _span_bytes(t: torch.Tensor) -> int:
+    if t.numel() == 0:
+        return 0
+    return (sum((size - 1) * stride for size, stride in zip(t.shape, t.stride())) + 1) * t.element_size()
+
+
+def _fields(obj) -> list[tuple[str, torch.Tensor]]:
+    """The GPU tensors an object holds as attributes."""
+    return [(name, value) for name, value in vars(obj).items() if isinstance(value, torch.Tensor) and value.is_cuda]
+
+
+def pending_tensors(pending) -> list[tuple[str, torch.Tensor]]:
+    if pending is None:
+        return []
+    if isinstance(pending, torch.Tensor):
+        return [("", pending)]
+    return _fields(pending)
+
+
+def pending_kind(pending) -> tuple:
+    """What must agree between the recorded layer's incoming sub-layer output and another's."""
+    return (type(pending).__name__, tuple((name, tuple(t.shape), t.dtype, t.stride()) for name, t in pending_tensors(pending)))
+
+
+def own_tensors(block, store) -> dict[tuple, torch.Tensor]:
+    """The tensors that belong to one layer call: its parts' and its cache slot's."""
+    out: dict[tuple, torch.Tensor] = {}
+    for role, part in block.parts.items():
+        for name, t in _fields(part):
+            out[("part", role, name)] = t
+    for name, t in store.arrays.items():
+        out[("cache", name)] = t
+    for name, t in store.state.items():
+        out[("state", name)] = t
+    return out
+
+
+def call_tensors(own: dict, pending, then) -> dict[tuple, torch.Tensor]:
+    out = dict(own)
+    for name, t in pending_tensors(pending):
+        out[("pending", name)] = t
+    if then is not None:
+        for name, t in _fields(then):
+            out[("then", name)] = t
+    return out
+
+
+@dataclass
+class LayerRecording:
+    calls: list[tuple]          # (function, arguments, ((argument index, tensor key, byte offset), ...), status)
+    keep: list[torch.Tensor]
+    result: object
+
+    def launch(self, tensors: dict[tuple, torch.Tensor], then):
+        for fn, args, patches, status in self.calls:
+            if patches:
+                args = list(args)
+                for index, key, offset in patches:
+                    args[index] = c_void_p(tensors[key].data_ptr() + offset)
+            got = fn(*args)
+            if got != status:
+                raise ops.KernelError(f"a replayed launch returned {got}, the recorded one {status}")
+        result = self.result
+        if isinstance(result, Added) and result.gamma is not None:
+            # the stream times the weight of the norm that follows THIS layer
+            result = dataclasses.replace(result, gamma=then.sink(None).gamma)
+        return result
+
+
+def record(run, tensors: dict[tuple, torch.Tensor]):
+    """Run ``run()`` while its launches are listed.  Returns (its result, a LayerRecording or
+    None if what ran cannot be replayed)."""
+    with ops.recording() as recorder:
+        result = run()
+    if not recorder.valid:
+        return result, None
+    spans = sorted((t.data_ptr(), t.data_ptr() + _span_bytes(t), key) for key, t in tensors.items() if t.numel())
+    starts = [s[0] for s in spans]
+    calls = []
+    for fn, args, status in recorder.calls:
+        patches = []
+        for index, arg in enumerate(args):
+            if not isinstance(arg, c_void_p) or not arg.value:
+                continue
+            at = bisect.bisect_right(starts, arg.value) - 1     # (the spans of different tensors do not overlap)
+            if at >= 0 and spans[at][0] <= arg.value < spans[at][1]:
+                patches.append((index, spans[at][2], arg.value - spans[at][0]))
+        calls.append((fn, args, tuple(patches), status))
+    return result, LayerRecording(calls, recorder.keep, result)

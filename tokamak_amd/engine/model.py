@@ -9,6 +9,8 @@ import torch
 from tokamak_amd.cache.pages import CacheGroupSpec
 from tokamak_amd.config.model_config import ModelPlan, PartSpec
 from tokamak_amd.config.registry import get_part
+from tokamak_amd.engine import layer_replay
+from tokamak_amd.kernels import ops
 from tokamak_amd.kernels.linear import Added
 from tokamak_amd.parts.base import Block, CacheRequest, Part, StateArray
 from tokamak_amd.weights.spec import TensorSpec
@@ -43,6 +45,15 @@ class LayeredModel:
             self.blocks.append(get_part("block", spec.block.kind)(parts, **spec.block.as_dict()))
         self.final_norm = self._build("norm", plan.final_norm)
         self.head = self._build("head", plan.head)
+        # Layers of one kind (equal parts, block and arguments; only their tensors differ) launch
+        # the same kernels in a step: one is recorded, the others replayed (engine/layer_replay.py).
+        self.replay_layers = True
+        kinds: dict[tuple, int] = {}
+        self._layer_kind = [
+            kinds.setdefault((spec.block, tuple((role, sub.family, sub.spec, sub.shared) for role, sub in spec.parts)), i)
+            for i, spec in enumerate(plan.layers)
+        ]
+        self._own_tensors: dict[tuple[int, int], tuple] = {}
 
     def _build(self, family: str, spec: PartSpec, shared: bool = False) -> Part:
         if shared and (family, spec) in self._shared:
@@ -87,6 +98,7 @@ class LayeredModel:
     def bind(self, fetch) -> None:
         for prefix, part in self._named_parts():
             part.bind(prefix, fetch)
+        self._own_tensors.clear()
         if self.plan.tie_word_embeddings:
             self.head.tie(self.embedding)
 
@@ -140,16 +152,36 @@ class LayeredModel:
         resid = self.embedding.forward(batch)
         pending = None
         order = self.plan.order
+        replay = self.replay_layers and ops.can_record()
+        recordings: dict[tuple, layer_replay.LayerRecording | None] = {}
         for at, call in enumerate(order):
             block = self.blocks[call.layer]
+            store = storage.slot(call.cache)
+            kwargs = {}
             if block.fuses_residual:
                 # the norm that reads the stream after this block: its last product may prepare for it
-                then = self.blocks[order[at + 1].layer].entry_norm if at + 1 < len(order) else self.final_norm
-                pending = block.forward(resid, pending, batch, storage.slot(call.cache), call.writes_cache, then=then)
-            else:
-                if isinstance(pending, Added):
-                    pending = None      # the sum is in the stream already
-                pending = block.forward(resid, pending, batch, storage.slot(call.cache), call.writes_cache)
+                kwargs["then"] = self.blocks[order[at + 1].layer].entry_norm if at + 1 < len(order) else self.final_norm
+            elif isinstance(pending, Added):
+                pending = None      # the sum is in the stream already
+            if not (replay and block.replayable):
+                pending = block.forward(resid, pending, batch, store, call.writes_cache, **kwargs)
+                continue
+            then = kwargs.get("then")
+            held = self._own_tensors.get((call.layer, call.cache))
+            if held is None or held[0] is not store:      # (another cache storage: its arrays lie elsewhere)
+                held = self._own_tensors[(call.layer, call.cache)] = (store, layer_replay.own_tensors(block, store))
+            own = held[1]
+            tensors = layer_replay.call_tensors(own, pending, then)
+            key = (self._layer_kind[call.layer], call.writes_cache, store.group, type(then), layer_replay.pending_kind(pending))
+            if key in recordings:
+                recorded = recordings[key]
+                if recorded is not None:
+                    pending = recorded.launch(tensors, then)
+                else:
+                    pending = block.forward(resid, pending, batch, store, call.writes_cache, **kwargs)
+                continue
+            pending, recordings[key] = layer_replay.record(
+                lambda: block.forward(resid, pending, batch, store, call.writes_cache, **kwargs), tensors)
         if batch.num_logit_rows == 0:
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=self.device)
         if isinstance(pending, Added) and not self.final_norm.fuses_residual:

@@ -83,6 +83,7 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype, allow_pa
         # hipBLASLt with kept plans and measured algorithms; shapes it has nothing for
         # (rows that are not 16-byte aligned, say) go through torch's binding of it
         if not (skinny_fits(x, weight) and ops.gemm_library(x, weight, out)):
+            ops.not_replayable()
             torch.matmul(x, weight.t(), out=out)
     else:
         ops.gemm_tiled(x, weight, out)

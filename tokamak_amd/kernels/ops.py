@@ -30,7 +30,59 @@ def _code(dtype: torch.dtype) -> int:
 
 
 def _p(t: torch.Tensor | None) -> c_void_p:
-    return c_void_p(0 if t is None else t.data_ptr())
+    if t is None:
+        return c_void_p(0)
+    if _recorder is not None:
+        _recorder.keep.append(t)    # a replay launches on this memory again
+    return c_void_p(t.data_ptr())
+
+
+class LaunchRecorder:
+    """The kernel launches of a stretch of host code: (library function, arguments, returned
+    status) of every call that went through this module while the recorder was current, and
+    the tensors whose addresses were passed.  The engine records one layer of a step and
+    launches the layers of the same kind from the list, with their own weights and cache
+    arrays in place of the recorded ones (engine/layer_replay.py): the checks, the choice of
+    kernels and the allocations of the recorded layer hold for them too."""
+
+    def __init__(self) -> None:
+        self.calls: list[tuple] = []
+        self.keep: list[torch.Tensor] = []
+        self.valid = True
+
+    def call(self, fn, args: tuple) -> int:
+        status = fn(*args)
+        self.calls.append((fn, args, status))
+        return status
+
+
+_recorder: LaunchRecorder | None = None
+
+
+class recording:
+    """``with recording() as rec``: launches inside the block are also listed in ``rec``."""
+
+    def __enter__(self) -> LaunchRecorder:
+        global _recorder
+        self._before = _recorder
+        _recorder = LaunchRecorder()
+        return _recorder
+
+    def __exit__(self, *exc):
+        global _recorder
+        _recorder = self._before
+        return False
+
+
+def not_replayable() -> None:
+    """Called where work is launched past this module (a library routine of torch): a
+    recording that is being made does not hold it and must not be replayed."""
+    if _recorder is not None:
+        _recorder.valid = False
+
+
+def can_record() -> bool:
+    return _recorder is None and _profile is None
 
 
 _pinned_stream: c_void_p | None = None
@@ -203,6 +255,9 @@ def _fn(library: str, name: str):
     if _profile is not None and name not in ("tk_argmax_segments",):
         profile = _profile
         return lambda *args: profile.timed(name, fn, args)
+    if _recorder is not None:
+        recorder = _recorder
+        return lambda *args: recorder.call(fn, args)
     return fn
 
 

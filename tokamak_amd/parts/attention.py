@@ -26,6 +26,7 @@ class GQAAttention(Mixer):
 
     capturable = True
     fuses_residual = True
+    replayable = True
 
     def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qk_norm_eps: float | None, softmax_scale: float, window: int | None,

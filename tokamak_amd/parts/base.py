@@ -46,6 +46,11 @@ class Part:
     """
 
     capturable = False
+    # ``replayable``: besides, the part launches all its work through ``kernels.ops`` (no
+    # routine of torch's computes for it) and decides nothing from what differs between two
+    # layers with equal parameters, so the launches of one layer, with another layer's
+    # tensors put in, are that layer's (engine/layer_replay.py).
+    replayable = False
     # Whether the part takes part in the fusion of the residual add and the norm into the
     # products around them (kernels/linear.py).  A norm that says so takes ``Added`` as its
     # ``delta`` (the sum is already in the stream) and a keyword ``defer`` (it may then
@@ -181,6 +186,7 @@ class Block:
     roles: tuple[str, ...] = ()
     optional: tuple[str, ...] = ()
     fuses_residual = False      # see Part.fuses_residual
+    replays_parts = False       # the block's own forward is replayable, see Part.replayable
     entry_norm: "Norm | None" = None   # the norm that reads the stream first, if the block fuses
 
     def __init__(self, parts: dict[str, Part]) -> None:
@@ -194,6 +200,8 @@ class Block:
             raise ValueError(f"{type(self).__name__}: a layer has one cache slot, so at most one mixer")
         self.parts = dict(parts)
         self.mixer: Mixer | None = mixers[0] if mixers else None
+        # a block's launches are replayed only if the block itself says so and all its parts do
+        self.replayable = bool(type(self).replays_parts) and all(p.replayable for p in parts.values())
 
     def forward(self, resid: torch.Tensor, pending: torch.Tensor | None, batch, store,
                 writes_cache: bool) -> torch.Tensor | None:

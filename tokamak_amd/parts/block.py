@@ -23,6 +23,7 @@ class PreNormBlock(Block):
     roles = ("mixer_norm", "mixer", "feed_forward_norm", "feed_forward")
     optional = ("position",)
     fuses_residual = True
+    replays_parts = True
 
     def __init__(self, parts) -> None:
         super().__init__(parts)

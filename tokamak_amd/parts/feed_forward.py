@@ -20,6 +20,7 @@ class SwiGLU(FeedForward):
 
     capturable = True
     fuses_residual = True
+    replayable = True
 
     def __init__(self, *, hidden_size: int, intermediate_size: int, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)

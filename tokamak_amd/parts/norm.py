@@ -21,6 +21,7 @@ class RMSNorm(Norm):
 
     capturable = True
     fuses_residual = True
+    replayable = True
 
     def __init__(self, *, dim: int, eps: float, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)

@@ -20,6 +20,7 @@ class RotaryHalf(PositionEncoding):
     """
 
     capturable = True
+    replayable = True
 
     def __init__(self, *, rotary_dim: int, theta: float, dtype, device) -> None:
         super().__init__(dtype=dtype, device=device)
