@@ -41,11 +41,13 @@ def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
 def stream_splits(n: int, k: int, m: int = 1) -> int:
     """Shares of K for the LDS-staged kernel so that enough blocks exist: about 512 for up
     to 32 rows; half as many beyond, where every split writes (and the next kernel reads)
-    float32 partial sums of 64 rows."""
+    float32 partial sums of 64 rows.  Down to one chunk of 256 a share: a small matrix
+    (the projections of a 0.6B-shaped model) is read in one memory round trip then, and
+    its time is round trips, not bytes."""
     blocks = -(-n // (16 * ops.stream_waves(m, k)))
     chunks = -(-k // 256)
     target = STREAM_TARGET_BLOCKS if m <= 32 else STREAM_TARGET_BLOCKS // 2
-    return max(1, min(chunks // 2, -(-target // blocks), 64))
+    return max(1, min(chunks, -(-target // blocks), 64))
 
 
 def gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype, allow_partials: bool = False) -> torch.Tensor:

@@ -389,11 +389,14 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
                                               _stream()), "gemm_tiled")
 
 
-def stream_waves(rows: int, k: int, gated: bool = False) -> int:
+def stream_waves(rows: int, k: int, gated: bool = False, n: int = 0) -> int:
     """Waves a block of the streaming product.  Eight waves share a chunk of the
     activations (the block then owns 128 weight rows), which pays when the chunk is large
     (more than 32 rows) and the walk over K long (the gated product, whose halves meet in
-    one block, and K from 8192 on); else four."""
+    one block, and K from 8192 on), and the gated product has columns (``n``) for at least
+    128 such blocks: a small one is spread over more blocks of four."""
+    if gated and 0 < n < 128 * 64:
+        return 4
     return 8 if rows > 32 and (gated or k >= 8192) else 4
 
 
@@ -458,7 +461,7 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, w
     slabs = _row_scale(sumsq, m, "gemm_stream_swiglu")
     _note(f"{m}x{w.shape[0]}x{k}", (w.shape[0] * k + m * k) * 2 + m * w.shape[0], 2.0 * m * w.shape[0] * k)
     _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
-                                                     w.stride(0), out.stride(0), waves or stream_waves(m, k, True),
+                                                     w.stride(0), out.stride(0), waves or stream_waves(m, k, True, w.shape[0] // 2),
                                                      _p(sumsq), slabs, float(eps), _stream()), "gemm_stream_swiglu")
 
 
