@@ -303,6 +303,74 @@ def test_qknorm_rope_store(dtype, nh, nkv, hd, ps, rot):
         at += n
 
 
+@pytest.mark.parametrize("form", ["float32", "bfloat16", "partial sums", "no norm", "queries only"])
+@pytest.mark.parametrize("nh, nkv, hd, ps", [(8, 2, 128, 16), (3, 3, 64, 32), (14, 1, 128, 64), (5, 5, 64, 16)])
+def test_qknorm_rope_store_of_long_portions(form, nh, nkv, hd, ps):
+    """Portions of 300 and 41 tokens that start inside a page, beside a decode token, with a
+    number of heads that is no multiple of a wave's share; pages scattered; partial sums as
+    input; what is not written stays as it was."""
+    from tokamak_amd.kernels import ops
+
+    dtype = torch.float32 if form == "float32" else torch.bfloat16
+    eps, theta = 1e-5, 50000.0
+    g = torch.Generator().manual_seed(nh + hd)
+    lengths = [(300, 11), (1, 77), (41, 0)]
+    need = [-(-(n + ctx) // ps) for n, ctx in lengths]
+    order = torch.randperm(sum(need) + 3, generator=g).tolist()
+    spans, at = [], 0
+    for (n, ctx), pages in zip(lengths, need):
+        spans.append((n, ctx, order[at:at + pages]))
+        at += pages
+    batch = make_batch(spans)
+    N = batch.num_tokens
+    stores = form != "queries only"
+    width = (nh + (2 * nkv if stores else 0)) * hd
+    qkv = rand(N, width, seed=1)
+    qw, kw = 1 + 0.3 * rand(hd, seed=2), 1 + 0.3 * rand(hd, seed=3)
+    cos = torch.empty(N, hd // 2, device=DEV)
+    sin = torch.empty(N, hd // 2, device=DEV)
+    inv_freq = 1.0 / (theta ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))
+    ops.rope_tables(batch.positions, inv_freq.to(DEV), cos, sin)
+    want_cos, want_sin = plain.rope_tables(batch.positions.cpu(), hd, theta)
+    if form == "partial sums":
+        pieces = rand(3, N, width, seed=5)
+        pieces[2] = qkv - pieces[0] - pieces[1]
+        given, qkv = pieces.to(DEV), pieces.sum(0)
+    else:
+        qkv = qkv.to(dtype).float()
+        given = qkv.to(dtype).to(DEV)
+    k_cache = torch.full((len(order), nkv * hd * ps), 7.0, dtype=dtype, device=DEV)
+    v_cache = torch.full((len(order), nkv * hd * ps), 7.0, dtype=dtype, device=DEV)
+    q_out = torch.empty(N, nh * hd, dtype=dtype, device=DEV)
+    normed = form != "no norm"
+    ops.qknorm_rope_store(given, qw.to(DEV) if normed else None, kw.to(DEV) if normed else None, cos, sin,
+                          batch.positions, batch.req_of_token, batch.block_tables[0], q_out,
+                          k_cache if stores else None, v_cache if stores else None, num_heads=nh, num_kv_heads=nkv,
+                          head_dim=hd, rotary_dim=hd, page_size=ps, eps=eps, store=stores)
+    x = qkv.view(N, -1, hd)
+
+    def expect(t, w, rows=slice(None)):
+        if normed:
+            t = plain.rmsnorm(t, w, eps)
+        return plain.apply_rope(t, want_cos[rows], want_sin[rows])
+
+    tol = TOL[dtype]
+    torch.testing.assert_close(q_out.cpu().float().view(N, nh, hd), expect(x[:, :nh], qw), **tol)
+    if not stores:
+        assert (k_cache == 7.0).all() and (v_cache == 7.0).all()
+        return
+    k, v = x[:, nh:nh + nkv], x[:, nh + nkv:]
+    at = 0
+    for n, ctx, table in spans:
+        kk, vv = unpack_pages(k_cache.cpu(), v_cache.cpu(), table, len(table) * ps, nkv, hd, ps)
+        torch.testing.assert_close(kk[ctx:ctx + n].float(), expect(k[at:at + n], kw, slice(at, at + n)), **tol)
+        torch.testing.assert_close(vv[ctx:ctx + n].float(), v[at:at + n].to(dtype).float(), **tol)
+        assert (kk[:ctx] == 7.0).all() and (vv[:ctx] == 7.0).all() and (kk[ctx + n:] == 7.0).all() and (vv[ctx + n:] == 7.0).all()
+        at += n
+    untouched = [p for p in range(len(order)) if all(p not in t for _, _, t in spans)]
+    assert (k_cache[untouched] == 7.0).all() and (v_cache[untouched] == 7.0).all()
+
+
 # ---------------------------------------------------------------------------
 # norms, activation, embedding, matrix product
 # ---------------------------------------------------------------------------
