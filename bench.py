@@ -205,13 +205,31 @@ def decode_pass(runner, vocab, batch, prompt_tokens, steps, seed):
     for r in range(batch):
         logits = fill(runner, r, random_prompt(vocab, prompt_tokens, seed * 1000 + r))
         last.append(int(greedy_tokens(logits).item()))
+    # The generation loop of LLM.generate: every step is launched before the tokens of the
+    # step before it are read (it takes them from the sampler's output on the GPU), and the
+    # host reads every step's tokens, one step late.
+    pinned = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+    copied = [torch.cuda.Event(), torch.cuda.Event()]
+    generated = []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        logits = runner.step([StepEntry(r, [last[r]], [0]) for r in range(batch)])
-        last = greedy_tokens(logits).tolist()
+    for i in range(steps):
+        if i == 0:
+            entries = [StepEntry(r, [last[r]], [0]) for r in range(batch)]
+        else:
+            entries = [StepEntry(r, [0], [0], feed=r) for r in range(batch)]
+        logits = runner.step(entries)
+        drawn = greedy_tokens(logits, out=runner.sampled)
+        pinned[i % 2].copy_(drawn, non_blocking=True)
+        copied[i % 2].record()
+        if i > 0:
+            copied[(i - 1) % 2].synchronize()
+            generated.append(pinned[(i - 1) % 2].tolist())
+    copied[(steps - 1) % 2].synchronize()
+    generated.append(pinned[(steps - 1) % 2].tolist())
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    assert len(generated) == steps and all(len(g) == batch for g in generated)
     for r in range(batch):
         runner.end(r)
     return elapsed

@@ -301,3 +301,92 @@ def test_captured_decode_steps_queued_without_a_host_sync(folders, dtype):
                 pages_g = graphed.manager.block_table(r)
                 pages_e = eager.manager.block_table(r)
                 assert torch.equal(ga[pages_g], ea[pages_e])
+
+
+@pytest.mark.parametrize("use_graphs", [False, True], ids=["eager", "replayed"])
+def test_a_step_takes_tokens_that_are_still_on_the_gpu(folders, use_graphs):
+    """``StepEntry.feed``: a decode token named by its row in the sampler's output instead
+    of by its value gives the logits of the same step with the value given, in steps that
+    are replayed from a recording and in steps that are not, beside entries whose tokens
+    the host gives; and what it refuses."""
+    from tokamak_amd.engine.runner import ModelRunner, StepEntry
+
+    folder = folders["E"] if "E" in folders else folders["A"]
+    cfg, _ = plain.read_folder(folder)
+    prompts = [random_ids(cfg["vocab_size"], n, 60 + i) for i, n in enumerate([9, 21, 5])]
+    nxt = [random_ids(cfg["vocab_size"], 6, 80 + i) for i in range(3)]
+
+    def run(fed):
+        runner = ModelRunner.from_folder(folder, dtype="bfloat16", page_size=16, kv_pool_tokens=256, max_requests=4,
+                                         use_graphs=use_graphs)
+        for r, p in enumerate(prompts):
+            runner.step([StepEntry(r, p, [])])
+        out = []
+        for i in range(6):
+            if fed:
+                # rows in another order than the entries, as a sampler might leave them
+                runner.sampled[:4].copy_(torch.tensor([nxt[2][i], 0, nxt[0][i], nxt[1][i]], dtype=torch.int32))
+                entries = [StepEntry(0, [0], [0], feed=2), StepEntry(1, [nxt[1][i]], [0]), StepEntry(2, [0], [0], feed=0)]
+            else:
+                entries = [StepEntry(r, [nxt[r][i]], [0]) for r in range(3)]
+            if i == 3:      # a prompt portion beside them: a step that is not replayed
+                entries.append(StepEntry(3, random_ids(cfg["vocab_size"], 7, 99), [6]))
+            out.append(runner.step(entries).cpu())
+        assert bool(runner._graphs) == use_graphs
+        return runner, out
+
+    _, want = run(False)
+    runner, got = run(True)
+    for i, (a, b) in enumerate(zip(want, got)):
+        assert torch.equal(a, b), f"step {i}"
+    with pytest.raises(ValueError):
+        runner.step([StepEntry(0, [1, 2], [0], feed=0)])
+    with pytest.raises(ValueError):
+        runner.step([StepEntry(0, [1], [0], feed=4)])
+    runner.manager.check()
+
+
+@pytest.mark.parametrize("which", ["A", "D"])
+def test_running_one_step_ahead_changes_no_token(tmp_path, which):
+    """The step loop launches a step before it has read the tokens of the step before.
+    Random workloads (greedy and sampled, stops on EOS ids that do occur and on length,
+    tight pools with preemption, small budgets): tokens and finish reasons equal those of
+    a loop that reads every step's tokens before it plans the next."""
+    import json
+    import random
+
+    from tokamak_amd import LLM, SamplingParams
+
+    folder = make_folder(tmp_path, which)
+    cfg = TINIES[which]["config"]
+    page, longest = TINIES[which]["page_size"], min(cfg.max_position_embeddings, 256)
+    # ids that greedy runs of this model do produce, so that some requests stop on them
+    probe = LLM(folder, dtype="float32", max_seq_len=longest, block_size=page, kv_pool_tokens=4 * longest, max_batch_size=4)
+    seen = probe.generate(prompt_token_ids=[[3, 1, 4], [1, 5, 9, 2, 6]],
+                          sampling_params=SamplingParams(temperature=0.0, max_new_tokens=30, ignore_eos=True))
+    eos = sorted({o.output_token_ids[7] for o in seen} | {o.output_token_ids[20] for o in seen})
+    (folder / "generation_config.json").write_text(json.dumps({"eos_token_id": eos}))
+    stops = preemptions = 0
+    for seed in range(6):
+        rng = random.Random(100 + seed)
+        count = rng.randint(2, 8)
+        prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(1, longest // 2))] for _ in range(count)]
+        prompts[0] = [3, 1, 4]
+        params = [SamplingParams(temperature=rng.choice([0.0, 0.0, 0.8, 1.2]), top_k=rng.choice([0, 5, 40]),
+                                 top_p=rng.choice([1.0, 0.9]), max_new_tokens=rng.randint(1, longest // 3),
+                                 seed=rng.randrange(1 << 30), ignore_eos=rng.random() < 0.3) for _ in range(count)]
+        params[0] = SamplingParams(temperature=0.0, max_new_tokens=30)
+        kwargs = dict(dtype="float32", max_seq_len=longest, block_size=page, kv_pool_tokens=longest + rng.randint(0, longest),
+                      max_batch_size=rng.randint(1, 6), max_num_batched_tokens=rng.choice([8, 16, 64, 2048]),
+                      prefill_chunk=rng.choice([None, 2, 7, 16, 100]))
+        ahead = LLM(folder, steps_ahead=True, **kwargs)
+        in_turn = LLM(folder, steps_ahead=False, **kwargs)
+        got = ahead.generate(prompt_token_ids=prompts, sampling_params=params)
+        want = in_turn.generate(prompt_token_ids=prompts, sampling_params=params)
+        assert [(o.output_token_ids, o.finish_reason) for o in got] == [(o.output_token_ids, o.finish_reason) for o in want]
+        for llm in (ahead, in_turn):
+            llm.runner.manager.check()
+            assert llm.runner.manager.num_free_pages() == llm.runner.manager.num_pages()
+        stops += sum(o.finish_reason.value == "stop" for o in got)
+        preemptions += ahead.num_preemptions
+    assert stops > 0 and preemptions > 0

@@ -208,3 +208,106 @@ def test_random_workloads_finish_with_every_page_back(seed):
         assert steps < 2000
     assert all(s.finished for s in seqs)
     assert manager.num_free_pages() == 12 and manager.slots.num_free == 3
+
+
+# ---------------------------------------------------------------------------
+# one step ahead: plans made before the tokens of the step before are read
+# ---------------------------------------------------------------------------
+def launch(step):
+    """What the step loop does when it launches a step: caches advance, sampled tokens
+    are on their way (rows in the order of the sampling spans)."""
+    row = 0
+    for span in step.spans:
+        assert span.start == span.request.cached
+        span.request.advance(span.length)
+    for span in step.spans:
+        if span.samples:
+            span.request.unknown += 1
+            span.request.feed_row = row
+            row += 1
+
+
+def read(step, token=0, eos=()):
+    """... and when it reads them."""
+    for span in step.spans:
+        if span.samples and not span.request.finished:
+            span.request.accept(token, eos_token_ids=tuple(eos), context_limit=10 ** 6)
+
+
+def test_a_decode_span_may_be_a_token_that_is_still_on_the_gpu():
+    sched, _ = make(budget=16)
+    a, b = make_seq(0, prompt_len=4, max_new=3), make_seq(1, prompt_len=6, max_new=8)
+    sched.submit(a)
+    sched.submit(b)
+    first = sched.plan()
+    launch(first)
+    assert a.unknown == b.unknown == 1 and a.length == 5 and a.decoding and not a.closing
+    second = sched.plan()                       # planned before the first step's tokens are read
+    assert [(s.request.rid, s.start, s.length, s.samples, s.feed) for s in second.spans] == [
+        (0, 4, 1, True, 0), (1, 6, 1, True, 1)]
+    assert a.span(1) == [0]                     # a placeholder: the step takes the token from the sampler's output
+    launch(second)
+    read(first, token=7)
+    assert a.tokens[-1] == 7 and a.unknown == 1 and a.num_drawn == 2
+    third = sched.plan()
+    launch(third)
+    read(second, token=8)
+    # a has drawn three tokens of three: it is certain to end, and is planned no further
+    assert a.unknown == 1 and a.closing and not a.decoding
+    fourth = sched.plan()
+    assert [s.request.rid for s in fourth.spans] == [1]
+    launch(fourth)
+    read(third, token=9)
+    assert a.finished and a.finish_reason == FinishReason.LENGTH and a.generated == [7, 8, 9]
+
+
+def test_a_plan_may_be_empty_while_the_last_tokens_are_on_their_way():
+    sched, manager = make()
+    a = make_seq(0, prompt_len=3, max_new=1)
+    sched.submit(a)
+    first = sched.plan()
+    launch(first)
+    assert a.closing and sched.busy
+    waiting = sched.plan()
+    assert waiting is not None and waiting.spans == []      # not "nothing left", and nobody is evicted for it
+    read(first, token=5)
+    assert a.finished
+    manager.free(a.rid)
+    assert sched.plan() is None
+
+
+def test_an_end_that_is_read_late_costs_one_token_and_nothing_else():
+    sched, manager = make()
+    a, b = make_seq(0, prompt_len=3, max_new=8), make_seq(1, prompt_len=3, max_new=8)
+    sched.submit(a)
+    sched.submit(b)
+    first = sched.plan()
+    launch(first)
+    second = sched.plan()
+    launch(second)
+    read(first, token=2, eos=(2,))              # both stop on the token of the first step ...
+    assert a.finished and b.finished and a.finish_reason == FinishReason.STOP
+    read(second, token=3)                       # ... and the second step's tokens are dropped
+    assert a.generated == [2] and b.generated == [2]
+    for r in (a, b):
+        manager.free(r.rid)
+    assert sched.plan() is None
+    manager.check()
+    assert manager.num_free_pages() == manager.num_pages()
+
+
+def test_a_request_evicted_with_a_token_on_its_way_waits_until_it_is_read():
+    sched, manager = make(num_pages=4, page_size=4, max_batch=2, budget=16)
+    a, b = make_seq(0, prompt_len=8, max_new=8), make_seq(1, prompt_len=8, max_new=8)
+    sched.submit(a)
+    sched.submit(b)
+    first = sched.plan()
+    launch(first)                               # 2 pages each: the pool is full, both tokens on their way
+    second = sched.plan()                       # a's next token needs a third page: b, the newest, goes
+    assert [r.rid for r in second.evicted] == [1] and [s.request.rid for s in second.spans] == [0]
+    assert b.cached == 0 and b.unknown == 1 and sched.waiting[0] is b
+    launch(second)
+    read(first, token=4)
+    assert b.tokens[-1] == 4 and b.unknown == 0 and len(b.tokens) == 9
+    third = sched.plan()
+    assert all(s.request is not b or s.feed is None for s in third.spans)

@@ -34,6 +34,24 @@ TK_API int tk_embed_gather(int dtype, const void* table, const int* ids, float* 
 }
 
 // ---------------------------------------------------------------------------
+// Token ids that are still on the GPU: ids[slots[i]] = sampled[rows[i]].  A step may be
+// launched before the host has read the tokens that the step before it sampled; its
+// descriptor then names, for such a token, the row of the sampler's output to take it from.
+// ---------------------------------------------------------------------------
+__global__ void feed_tokens_kernel(int* __restrict__ ids, const int* __restrict__ sampled,
+                                   const int* __restrict__ slots, const int* __restrict__ rows, int count) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) ids[slots[i]] = sampled[rows[i]];
+}
+
+TK_API int tk_feed_tokens(int* ids, const int* sampled, const int* slots, const int* rows, int count,
+                          hipStream_t stream) {
+  if (count <= 0) return 0;
+  feed_tokens_kernel<<<(count + 255) / 256, 256, 0, stream>>>(ids, sampled, slots, rows, count);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
 // residual add + RMSNorm over rows of width H.
 //   x = resid[row] (+ delta[row]);  if write_resid: resid[row] = x
 //   out[m] = x * rsqrt(mean(x^2) + eps) * weight

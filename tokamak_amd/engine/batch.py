@@ -26,6 +26,7 @@ class StepSpan:
     state_slot: int
     tables: list[list[int]]      # block table per cache group
     want: list[int] = field(default_factory=list)  # offsets within ``tokens`` whose logits are wanted
+    feed: int | None = None      # the span's one token is row ``feed`` of the sampler's last output, still on the GPU
 
 
 @dataclass
@@ -48,6 +49,9 @@ class StepBatch:
     tile_count: torch.Tensor | None = None      # [num_tiles] int32 tokens in the tile
     wide_first: torch.Tensor | None = None      # [num_wide] int32 first token row of a 32-token tile
     wide_count: torch.Tensor | None = None      # [num_wide] int32 tokens in it
+    feed_slots: torch.Tensor | None = None      # [N] int32: the first num_feed name token rows whose id ...
+    feed_rows: torch.Tensor | None = None       # [N] int32: ... is that row of the sampler's last output
+    num_feed: int = 0
     num_decode: int = 0
     num_tiles: int = 0
     num_wide: int = 0
@@ -65,7 +69,7 @@ class StepBatch:
 
 TILE_TOKENS = 16   # tokens per attention tile of a prompt portion
 WIDE_TOKENS = 32   # and per tile of the wide attention kernel
-NUM_FIXED = 12     # arrays in the packed buffer before the block tables
+NUM_FIXED = 14     # arrays in the packed buffer before the block tables
 
 
 @dataclass
@@ -87,6 +91,8 @@ class PackedBatch:
     max_decode_len: int
     max_tile_len: int = 0
     min_tile_ctx: int = 0
+    num_feed: int = 0
+    max_feed_row: int = -1
 
 
 def table_width(longest: int, fixed: int | None = None) -> int:
@@ -115,12 +121,12 @@ def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] |
             wide.extend((at + t, min(WIDE_TOKENS, q - t)) for t in range(0, q, WIDE_TOKENS))
         at += q
     nd, nt, nw = len(decode_rows), len(tiles), len(wide)
-    sizes = [n, n, n, r + 1, r, r, m, nd, nt, nt, nw, nw] + [r * w for w in widths]
+    sizes = [n, n, n, r + 1, r, r, m, nd, nt, nt, nw, nw, n, n] + [r * w for w in widths]
     offsets = [0]
     for size in sizes:
         offsets.append(offsets[-1] + size)
     buf = np.zeros(offsets[-1], dtype=np.int32)
-    tok, pos, req, qs, ctx, slots, rows, dec, tfirst, tcount, wfirst, wcount = (
+    tok, pos, req, qs, ctx, slots, rows, dec, tfirst, tcount, wfirst, wcount, fslots, frows = (
         buf[offsets[i]:offsets[i + 1]] for i in range(NUM_FIXED))
     tabs = [buf[offsets[NUM_FIXED + g]:offsets[NUM_FIXED + 1 + g]].reshape(r, widths[g])
             for g in range(num_groups)]
@@ -131,8 +137,14 @@ def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] |
     wcount[:] = [t[1] for t in wide]
     at = 0
     mi = 0
+    fed = 0
     for i, s in enumerate(spans):
         q = len(s.tokens)
+        if s.feed is not None:
+            if q != 1 or s.feed < 0:
+                raise ValueError("only a span of one token can take its token from the sampler's output")
+            fslots[fed], frows[fed] = at, s.feed
+            fed += 1
         tok[at:at + q] = s.tokens
         pos[at:at + q] = np.arange(s.ctx_len, s.ctx_len + q, dtype=np.int32)
         req[at:at + q] = i
@@ -156,7 +168,8 @@ def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] |
         ctx_lens=[s.ctx_len for s in spans],
         max_decode_len=max((s.ctx_len + 1 for s in spans if len(s.tokens) == 1), default=0),
         max_tile_len=max((s.ctx_len + len(s.tokens) for s in spans if len(s.tokens) > 1), default=0),
-        min_tile_ctx=min((s.ctx_len for s in spans if len(s.tokens) > 1), default=0))
+        min_tile_ctx=min((s.ctx_len for s in spans if len(s.tokens) > 1), default=0),
+        num_feed=fed, max_feed_row=max((s.feed for s in spans if s.feed is not None), default=-1))
 
 
 def batch_from_device(packed: PackedBatch, dev: torch.Tensor) -> StepBatch:
@@ -169,8 +182,8 @@ def batch_from_device(packed: PackedBatch, dev: torch.Tensor) -> StepBatch:
         ctx_len=parts[4], state_slots=parts[5], logit_rows=parts[6],
         block_tables=[parts[NUM_FIXED + g].view(r, widths[g]) for g in range(len(widths))],
         decode_tokens=parts[7], tile_first=parts[8], tile_count=parts[9],
-        wide_first=parts[10], wide_count=parts[11],
-        num_decode=packed.num_decode, num_tiles=packed.num_tiles, num_wide=packed.num_wide,
+        wide_first=parts[10], wide_count=parts[11], feed_slots=parts[12], feed_rows=parts[13],
+        num_feed=packed.num_feed, num_decode=packed.num_decode, num_tiles=packed.num_tiles, num_wide=packed.num_wide,
         num_tile_tokens=sum(q for q in packed.q_lens if q > 1),
         max_decode_len=packed.max_decode_len, max_tile_len=packed.max_tile_len,
         min_tile_ctx=packed.min_tile_ctx,

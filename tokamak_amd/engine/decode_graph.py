@@ -47,14 +47,14 @@ class DecodeGraph:
     whose copy has not run yet.
     """
 
-    def __init__(self, model, storage, packed: PackedBatch, device) -> None:
+    def __init__(self, model, storage, packed: PackedBatch, device, feed=None) -> None:
         self.size = int(packed.buf.size)
         self._host = [torch.empty(self.size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self._copied = [torch.cuda.Event(), torch.cuda.Event()]
         self._turn = 0
         self.dev = torch.empty(self.size, dtype=torch.int32, device=device)
         self.batch = batch_from_device(packed, self.dev)
-        self._load(packed)
+        self._load(packed, feed)
         # this step itself, eagerly: code objects are loaded and the allocator is warm
         # before the recording starts; the recording executes nothing
         self.first_logits = model.forward(self.batch, storage)
@@ -70,7 +70,9 @@ class DecodeGraph:
         self.bytes = max(0, torch.cuda.max_memory_allocated(device) - before) + self.size * 4
         self.replays = 0
 
-    def _load(self, packed: PackedBatch) -> None:
+    def _load(self, packed: PackedBatch, feed=None) -> None:
+        """The descriptor to the device; then ``feed(batch)`` puts in the token ids that are
+        still on the GPU (outside the recording: how many there are changes from step to step)."""
         if packed.buf.size != self.size:
             raise ValueError("descriptor does not have the shape this graph was captured for")
         turn = self._turn
@@ -79,11 +81,14 @@ class DecodeGraph:
         self._host[turn].numpy()[:] = packed.buf
         self.dev.copy_(self._host[turn], non_blocking=True)
         self._copied[turn].record()
+        self.batch.num_feed = packed.num_feed
+        if feed is not None:
+            feed(self.batch)
 
-    def run(self, packed: PackedBatch) -> torch.Tensor:
+    def run(self, packed: PackedBatch, feed=None) -> torch.Tensor:
         """Replay with a new descriptor; the returned logits live in the graph's
         own memory and are overwritten by the next replay."""
-        self._load(packed)
+        self._load(packed, feed)
         self.graph.replay()
         self.replays += 1
         return self.logits

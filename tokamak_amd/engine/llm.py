@@ -11,6 +11,7 @@ import json
 import random
 import time
 from collections.abc import Sequence as AbcSequence
+from dataclasses import dataclass
 from pathlib import Path
 
 import torch
@@ -25,6 +26,15 @@ from tokamak_amd.sampling.params import SamplingParams
 from tokamak_amd.sampling.sampler import sample_tokens
 from tokamak_amd.weights.random_init import expected_tensors_of
 from tokamak_amd.weights.sources import RandomSource, SafetensorsSource
+
+
+@dataclass
+class _InFlight:
+    """A launched step whose sampled tokens the host has not read yet."""
+
+    requests: list[Request]         # in the order of the sampler's rows
+    tokens: torch.Tensor            # pinned host copy of those rows ...
+    copied: torch.cuda.Event        # ... complete after this
 
 
 class LLM:
@@ -51,6 +61,9 @@ class LLM:
             default: the library's first choice is taken, so that two runs of the same
             input compute the same bits).
         prefill_chunk: longest prompt portion in one step (new; default the budget).
+        steps_ahead: launch every step before the tokens of the step before are read
+            (new; default on: the host's work between two steps is hidden behind the GPU's;
+            the tokens generated are the same either way).
         device: ``"auto"`` or a cuda device; there is no CPU path.
         kv_backend, scheduling, attention_backend, attention_policy, draft_model: the
             reference's further options; this engine has one choice for each
@@ -68,7 +81,8 @@ class LLM:
                  device: str | torch.device = "auto", kv_backend: str = "paged",
                  scheduling: str = "continuous", attention_backend: str = "auto",
                  attention_policy: str = "full", draft_model=None, seed: int = 0,
-                 random_weights_on_gpu: bool = False, tune_library_products: bool = False) -> None:
+                 random_weights_on_gpu: bool = False, tune_library_products: bool = False,
+                 steps_ahead: bool = True) -> None:
         given = {"kv_backend": kv_backend, "scheduling": scheduling, "attention_backend": attention_backend,
                  "attention_policy": attention_policy, "draft_model": draft_model}
         for name, value in given.items():
@@ -124,6 +138,11 @@ class LLM:
         self.tokenizer = self._load_tokenizer(folder) if folder is not None else None
         self.num_steps = 0
         self.num_preemptions = 0
+        # the step loop runs one step ahead of the tokens it has read (see generate)
+        self.steps_ahead = steps_ahead
+        self._host_tokens = [torch.empty(max_batch_size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._copied = [torch.cuda.Event(), torch.cuda.Event()]
+        self._turn = 0
 
     @staticmethod
     def _load_tokenizer(folder: Path):
@@ -193,12 +212,24 @@ class LLM:
                               self.prefill_chunk)
         for request in requests:
             scheduler.submit(request)
+        for request in requests:
+            request.context_limit = self._context_limit(request)
         try:
-            while scheduler.busy:
-                plan = scheduler.plan()
-                if plan is None:
+            # One step ahead: a step is planned and launched while the one before it runs; the
+            # tokens that one sampled are read (and stop rules applied) meanwhile.  A decoding
+            # request's next step takes its token from the sampler's output on the GPU.
+            in_flight = None
+            while scheduler.busy or in_flight is not None:
+                plan = scheduler.plan() if scheduler.busy else None
+                launched = self._launch(plan) if plan is not None else None
+                if in_flight is not None:
+                    self._read(in_flight)
+                elif plan is None or not plan.spans:
                     raise RuntimeError("the scheduler has unfinished requests but plans no step")
-                self._run(plan)
+                in_flight = launched
+                if in_flight is not None and not self.steps_ahead:
+                    self._read(in_flight)
+                    in_flight = None
         finally:
             # also what the scheduler reserved for requests that never reached a step
             self.runner.end_all()
@@ -206,17 +237,22 @@ class LLM:
                 self.runner.manager.free(request.rid)
         return [self._output(request, text) for request, text in zip(requests, texts)]
 
-    def _run(self, plan: StepPlan) -> None:
+    def _launch(self, plan: StepPlan) -> _InFlight | None:
+        """Run the plan's step and draw its tokens, all without waiting for the GPU; None
+        if the step samples nothing (or the plan is empty)."""
         for victim in plan.evicted:
             self.runner.forget(victim.rid)      # the scheduler has already freed its pages
             self.num_preemptions += 1
+        if not plan.spans:
+            return None
         entries, sampling = [], []
         for span in plan.spans:
             request = span.request
             held = self.runner.cached_tokens(request.rid)
             if span.start != held or span.start != request.cached:
                 raise RuntimeError(f"request {request.rid}: span starts at {span.start}, the cache holds {held}")
-            entries.append(StepEntry(request.rid, request.span(span.length), [span.length - 1] if span.samples else []))
+            entries.append(StepEntry(request.rid, request.span(span.length), [span.length - 1] if span.samples else [],
+                                     span.feed))
             if span.samples:
                 sampling.append(request)
         logits = self.runner.step(entries)
@@ -224,14 +260,29 @@ class LLM:
         for span in plan.spans:
             span.request.advance(span.length)
         if not sampling:
-            return
-        chosen = sample_tokens(logits, [r.params for r in sampling], [r.seed for r in sampling],
-                               [r.num_generated for r in sampling]).tolist()
+            return None
+        drawn = sample_tokens(logits, [r.params for r in sampling], [r.seed for r in sampling],
+                              [r.num_drawn for r in sampling], out=self.runner.sampled)
+        for row, request in enumerate(sampling):
+            request.unknown += 1
+            request.feed_row = row
+        turn = self._turn
+        self._turn = 1 - turn
+        host = self._host_tokens[turn][:len(sampling)]
+        host.copy_(drawn, non_blocking=True)
+        self._copied[turn].record()
+        return _InFlight(sampling, host, self._copied[turn])
+
+    def _read(self, step: _InFlight) -> None:
+        """Wait for a launched step's tokens and give them to their requests."""
+        step.copied.synchronize()
         stamp = time.perf_counter()
-        for request, token in zip(sampling, chosen):
+        for request, token in zip(step.requests, step.tokens.tolist()):
+            if request.finished:
+                continue    # it ended with an earlier token while this step already ran: one token for nothing
             if request.first_token_at is None:
                 request.first_token_at = stamp
-            if request.accept(token, eos_token_ids=self.eos_token_ids, context_limit=self._context_limit(request)):
+            if request.accept(token, eos_token_ids=self.eos_token_ids, context_limit=request.context_limit):
                 request.finished_at = stamp
                 self.runner.end(request.rid)
 

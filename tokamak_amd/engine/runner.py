@@ -42,11 +42,17 @@ def resolve_dtype(dtype) -> torch.dtype:
 
 @dataclass
 class StepEntry:
-    """A request's next tokens, and the offsets among them whose logits are wanted."""
+    """A request's next tokens, and the offsets among them whose logits are wanted.
+
+    ``feed``: the entry brings one token that the host does not know yet: row ``feed`` of
+    ``ModelRunner.sampled``, where the sampler of the step before has left it (``tokens``
+    holds a placeholder).  With it a decode step is launched while the step before it still
+    runs, and the host reads that step's tokens meanwhile."""
 
     request: object
     tokens: list[int]
     want: list[int] = field(default_factory=list)
+    feed: int | None = None
 
 
 class ModelRunner:
@@ -82,6 +88,8 @@ class ModelRunner:
         self._groups = groups
         self._ctx_len: dict[object, int] = {}
         self._graphs: dict[tuple, DecodeGraph] = {}
+        # where a sampler leaves its tokens for entries of the next step that ``feed`` on them
+        self.sampled = torch.zeros(max(max_requests, 1), dtype=torch.int32, device=self.device)
         self.graph_memory_bytes = int(graph_memory_bytes)
         self.step_memory_bytes = 0
         self.use_graphs = False
@@ -171,6 +179,9 @@ class ModelRunner:
                     f"request {e.request!r} would reach {total} tokens; the model's limit is {limit}")
             if any(not 0 <= w < len(e.tokens) for w in e.want):
                 raise ValueError(f"request {e.request!r} wants logits outside its {len(e.tokens)} tokens")
+            if e.feed is not None and (len(e.tokens) != 1 or not 0 <= e.feed < self.sampled.numel()):
+                raise ValueError(f"request {e.request!r}: a fed token is one token, from a row of the "
+                                 f"{self.sampled.numel()} that the sampler's output holds")
             if e.request not in self._ctx_len and self.manager.slots.slot_of(e.request) is None:
                 newcomers += 1
         if newcomers > self.manager.slots.num_free:
@@ -206,14 +217,22 @@ class ModelRunner:
                 request=e.request, tokens=list(e.tokens), ctx_len=ctx,
                 state_slot=self.manager.slots.slot_of(e.request),
                 tables=[self.manager.block_table(e.request, g) for g in range(self.num_groups)],
-                want=list(e.want)))
+                want=list(e.want), feed=e.feed))
         return spans
+
+    def _feed(self, batch: StepBatch) -> None:
+        """Put the tokens that are still on the GPU into the descriptor's token ids."""
+        if batch.num_feed:
+            ops.feed_tokens(batch.token_ids, self.sampled, batch.feed_slots, batch.feed_rows, batch.num_feed,
+                            self.sampled.numel())
 
     def prepare(self, entries: list[StepEntry]) -> StepBatch:
         """Reserve what the entries need and build the step's descriptor."""
         packed = pack_batch(self._spans(entries), self.num_groups)
         host = torch.from_numpy(packed.buf)
-        return batch_from_device(packed, host.pin_memory().to(self.device, non_blocking=True))
+        batch = batch_from_device(packed, host.pin_memory().to(self.device, non_blocking=True))
+        self._feed(batch)
+        return batch
 
     def _graph_step(self, entries: list[StepEntry]) -> torch.Tensor:
         """All entries bring one token: replay the captured step of this shape."""
@@ -229,13 +248,13 @@ class ModelRunner:
         graph = self._graphs.pop(key, None)
         if graph is None:
             # a new shape: this step runs eagerly, once, and is recorded for the next ones
-            graph = DecodeGraph(self.model, self.storage, packed, self.device)
+            graph = DecodeGraph(self.model, self.storage, packed, self.device, self._feed)
             logits, graph.first_logits = graph.first_logits, None
             self._graphs[key] = graph
             self._trim_graphs()
         else:
             self._graphs[key] = graph                # most recently used last
-            logits = graph.run(packed)
+            logits = graph.run(packed, self._feed)
         if len(wanted) == len(spans):
             return logits
         return logits[torch.tensor(wanted, dtype=torch.long, device=self.device)] if wanted else logits[:0]

@@ -13,6 +13,12 @@ request first, then fills what is left of ``max_num_batched_tokens`` with
 portions (at most ``prefill_chunk`` tokens) of requests whose tokens are not yet
 all cached, then admits from the waiting queue while slots, budget and pages
 allow.  Pages are reserved portion by portion.
+
+The step loop plans a step before it has read the tokens of the step before
+(``Request.unknown``): a decoding request's span may be that unread token (``Span.feed``);
+a request that is certain to end with it is left alone; one that was evicted with it waits
+at the head of the queue until it is read; and a plan may come back empty because
+everything left waits for tokens (``StepPlan.spans == []``).
 """
 
 from __future__ import annotations
@@ -34,6 +40,7 @@ class Span:
     start: int
     length: int
     samples: bool
+    feed: int | None = None     # its one token is still on the GPU: this row of the sampler's last output
 
 
 @dataclass
@@ -84,6 +91,8 @@ class Scheduler:
             spans = self._fill(evicted)
             if spans:
                 return StepPlan(spans, evicted)
+            if any(r.unknown for r in self.running) or (self.waiting and self.waiting[0].unknown):
+                return StepPlan([], evicted)     # what is left waits for tokens that are still on the GPU
             if self.running:
                 # nobody could move: every running request waits for pages
                 evicted.append(self._evict_newest())
@@ -105,7 +114,7 @@ class Scheduler:
             if not request.decoding:
                 at += 1
             elif self._reserve(request, 1):
-                spans.append(Span(request, request.cached, 1, True))
+                spans.append(Span(request, request.cached, 1, True, request.feed_row if request.unknown else None))
                 left -= 1
                 at += 1
             else:
@@ -114,7 +123,7 @@ class Scheduler:
         for request in self.running:
             if left <= 0:
                 break
-            if request.decoding:
+            if request.decoding or request.closing:
                 continue
             length = self._affordable(request, left)
             if length > 0 and self._reserve(request, length):
@@ -123,6 +132,8 @@ class Scheduler:
         # 3. newcomers, in arrival order, never past a head that does not fit
         while self.waiting and left > 0 and len(self.running) < self.max_batch_size:
             head = self.waiting[0]
+            if head.unknown:
+                break       # evicted with a token still on the GPU: its tokens are complete after the next read
             # the pool must be able to hold all the request has so far (reference:
             # scheduler.py:144-148); only its first portion is reserved
             if not self.manager.can_hold(head.rid, len(head.tokens)):

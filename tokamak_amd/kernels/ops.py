@@ -130,6 +130,7 @@ def _check(status: int, name: str) -> None:
 _SIGS = {
     "elementwise": {
         "tk_embed_gather": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "tk_feed_tokens": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
         "tk_add_rmsnorm": [c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p,
                            c_void_p, c_int, c_int, c_float, c_int, c_void_p],
         "tk_rope_tables": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -273,6 +274,18 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, resid: torch.Tensor) ->
     _note(f"{n}x{h}", n * h * (table.element_size() + 4))
     _check(_fn("elementwise", "tk_embed_gather")(_code(table.dtype), _p(table), _p(ids), _p(resid),
                                                  n, h, v, _stream()), "embed_gather")
+
+
+def feed_tokens(ids: torch.Tensor, sampled: torch.Tensor, slots: torch.Tensor, rows: torch.Tensor, count: int,
+                num_sampled: int) -> None:
+    """ids[slots[i]] = sampled[rows[i]] for i < count: token ids of a step that the sampler
+    of the step before left on the GPU.  The host has checked slots and rows against the
+    sizes (``num_sampled`` rows of ``sampled`` hold tokens)."""
+    _gpu(ids, sampled, slots, rows)
+    _need(ids.dtype == sampled.dtype == slots.dtype == rows.dtype == torch.int32, "token ids and indices are int32")
+    _need(0 <= count <= slots.numel() and count <= rows.numel() and 0 <= num_sampled <= sampled.numel(),
+          "more fed tokens than the index arrays hold")
+    _check(_fn("elementwise", "tk_feed_tokens")(_p(ids), _p(sampled), _p(slots), _p(rows), count, _stream()), "feed_tokens")
 
 
 def _partials(t: torch.Tensor | None, rows: int, width: int, dtype: torch.dtype, what: str):
