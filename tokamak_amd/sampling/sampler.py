@@ -58,7 +58,9 @@ def sample_tokens(logits: torch.Tensor, params: list[SamplingParams], seeds: lis
     floats[:m] = [p.temperature for p in params]
     floats[m:] = [p.top_p for p in params]
     host[6 * m:] = [p.top_k for p in params]
-    packed = torch.from_numpy(host).to(dev)
+    # through pinned memory and without waiting: a copy from pageable memory would hold the
+    # host until the GPU has run everything queued before it
+    packed = torch.from_numpy(host).pin_memory().to(dev, non_blocking=True)
     seed_t, draw_t = packed[:2 * m].view(torch.int64), packed[2 * m:4 * m].view(torch.int64)
     temperature, top_p = packed[4 * m:5 * m].view(torch.float32), packed[5 * m:6 * m].view(torch.float32)
     top_k = packed[6 * m:]
