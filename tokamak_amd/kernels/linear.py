@@ -101,7 +101,8 @@ def linear(x: torch.Tensor | DeferredNorm, weight: torch.Tensor, out_dtype: torc
     out_dtype = out_dtype or x.dtype
     m, n = x.shape[0], weight.shape[0]
     if isinstance(x, DeferredNorm):
-        if _few_rows_fit(m, x.scaled, weight, ops.ROW_SCALE_MAX_ROWS) and n >= gemm_bf16.STREAM_MIN_ROWS_OUT:
+        if (_few_rows_fit(m, x.scaled, weight, ops.ROW_SCALE_MAX_ROWS) and n >= gemm_bf16.STREAM_MIN_ROWS_OUT
+                and x.sumsq.shape[0] <= ops.ROW_SCALE_MAX_SLABS):
             splits = gemm_bf16.stream_splits(n, weight.shape[1], m) if allow_partials else 1
             if splits > 1:
                 out = torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
@@ -139,7 +140,7 @@ def gated_linear(x: torch.Tensor | DeferredNorm, gate_up: torch.Tensor) -> torch
     m = x.shape[0]
     inter = gate_up.shape[0] // 2
     if isinstance(x, DeferredNorm):
-        if _few_rows_fit(m, x.scaled, gate_up, ops.ROW_SCALE_MAX_ROWS):
+        if _few_rows_fit(m, x.scaled, gate_up, ops.ROW_SCALE_MAX_ROWS) and x.sumsq.shape[0] <= ops.ROW_SCALE_MAX_SLABS:
             out = torch.empty((m, inter), dtype=x.dtype, device=x.device)
             ops.gemm_stream_swiglu(x.scaled, gate_up, out, sumsq=x.sumsq, eps=x.eps)
             return out

@@ -419,7 +419,8 @@ def _row_scale(sumsq: torch.Tensor | None, m: int, what: str) -> int:
         return 0
     _gpu(sumsq)
     _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[1] == m and sumsq.shape[0] >= 1
-          and m <= ROW_SCALE_MAX_ROWS, f"{what}: the rows' sums of squares are float32 [slabs, M], M <= {ROW_SCALE_MAX_ROWS}")
+          and m <= ROW_SCALE_MAX_ROWS and sumsq.shape[0] <= ROW_SCALE_MAX_SLABS,
+          f"{what}: the rows' sums of squares are float32 [slabs <= {ROW_SCALE_MAX_SLABS}, M <= {ROW_SCALE_MAX_ROWS}]")
     return sumsq.shape[0]
 
 
@@ -480,6 +481,7 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, w
 
 WHOLEK_MAX_ROWS = 16    # rows of activations that the whole-K product takes
 ROW_SCALE_MAX_ROWS = 16  # rows up to which the streaming product applies a pending row scale
+ROW_SCALE_MAX_SLABS = 512  # ... and slabs of sums of squares it takes (csrc/gemm_mfma.hip: 16 * kRowScaleLoads)
 
 
 def wholek_waves(n: int, k: int, gated: bool = False) -> int:
