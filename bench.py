@@ -20,6 +20,12 @@ time.  Fractions are of the published peaks (HBM 8 TB/s, dense bf16 MFMA 2.5 PFL
 reads and copies of 4 GiB; back-to-back MFMA from registers), and ``frac_of_measured``
 the same fractions of those.  ``--profile`` adds ``kernels``: one decode step and one
 prefill step with every kernel call timed by events, summed by kind of call.
+
+Two further workloads go through ``LLM.generate`` (scheduler, prompt portions beside
+decode tokens, captured decode steps) and print a line of the same form:
+``--workload continuous`` (256 requests of uniform random lengths, Qwen3-0.6B shape) and
+``--workload trace`` (the reference's own 32-request throughput trace at 1, 4 and 16
+running requests, with its published figure as ``vs_baseline``).
 """
 
 from __future__ import annotations
@@ -362,6 +368,78 @@ def run_continuous(args) -> int:
     return 0
 
 
+# ---------------------------------------------------------------------------
+def reference_trace(num_requests: int, max_new_cap: int, seed: int, vocab_size: int):
+    """The lengths of the reference's throughput trace (benchmarks/workload.py:23-42): per
+    request, drawn in this order from ``random.Random(seed)``: a prompt length, log-normal
+    (mu 5.0, sigma 0.7) cut to 16..512; a number of new tokens, floor of an exponential of
+    mean 120, plus 8, at most ``max_new_cap``; then the prompt's ids (ids past the first
+    special token are folded back, which keeps the stream of draws as published).  With 32
+    requests, cap 256 and seed 0 this gives the 4,915 prompt and 2,901 output tokens of
+    benchmarks/README.md:87-90."""
+    import random
+
+    first_special = 151_643
+    rng = random.Random(seed)
+    prompts, new_tokens = [], []
+    for _ in range(num_requests):
+        length = int(min(512.0, max(16.0, rng.lognormvariate(5.0, 0.7))))
+        new_tokens.append(min(max_new_cap, 8 + int(rng.expovariate(1.0 / 120.0))))
+        prompts.append([rng.randrange(vocab_size) % first_special for _ in range(length)])
+    return prompts, new_tokens
+
+
+def run_trace(args) -> int:
+    """The reference's "throughput under concurrency" measurement (benchmarks/benchmark_throughput.py:
+    30-68, README.md:87-129): its seeded 32-request trace through ``LLM.generate`` on the
+    Qwen3-0.6B shape (random weights here), greedy, EOS ignored, a 16,384-token pool,
+    sequences of at most 1,024 tokens, at most 1, 4 and 16 running requests.  Every setting
+    runs twice; the second run is reported (the first also records the decode graphs)."""
+    import statistics
+
+    import torch
+
+    from tokamak_amd import LLM, SamplingParams
+    from tokamak_amd.config import find_preset
+
+    cfg = find_preset(args.model)[1]
+    prompts, new_tokens = reference_trace(32, 256, 0, cfg.vocab_size)
+    params = [SamplingParams(temperature=0.0, max_new_tokens=n, ignore_eos=True) for n in new_tokens]
+    config = {"model": f"{args.model}-shaped", "requests": len(prompts), "prompt_tokens": sum(map(len, prompts)),
+              "output_tokens": sum(new_tokens), "kv_pool_tokens": 16384, "max_seq_len": 1024}
+    value = steps = elapsed = None
+    for batch in (1, 4, 16):
+        llm = LLM(cfg, seed=0, random_weights_on_gpu=True, dtype=args.dtype, max_seq_len=1024,
+                  kv_pool_tokens=16384, max_batch_size=batch, tune_library_products=not args.no_tune)
+        for _ in range(2):
+            steps0 = llm.num_steps
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            outs = llm.generate(prompt_token_ids=prompts, sampling_params=params)
+            torch.cuda.synchronize()
+            elapsed, steps = time.perf_counter() - t0, llm.num_steps - steps0
+        assert [len(o.output_token_ids) for o in outs] == new_tokens
+        value = sum(new_tokens) / elapsed
+        ttft = sorted(o.ttft_s for o in outs)
+        config[f"b{batch}_out_tok_per_s"] = round(value, 1)
+        config[f"b{batch}_wall_s"] = round(elapsed, 4)
+        config[f"b{batch}_ttft_mean_ms"] = round(statistics.mean(ttft) * 1e3, 2)
+        config[f"b{batch}_ttft_p95_ms"] = round(ttft[min(int(0.95 * len(ttft)), len(ttft) - 1)] * 1e3, 2)
+        del llm
+        torch.cuda.empty_cache()
+    # the reference's best published figure for its own engine on this trace: continuous b=16 with its
+    # Triton kernel under Linux, 236.8 output tok/s on an RTX 3080 Laptop GPU (benchmarks/README.md:196)
+    config["baseline"] = "236.8 out tok/s, continuous b=16, RTX 3080 Laptop (reference benchmarks/README.md:196)"
+    print(json.dumps({
+        "metric": "output tok/s on the reference's 32-request trace, continuous batching, at most 16 running",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+        "ms_per_step": round(elapsed / steps * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": round(value / 236.8, 2), "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (the reference's seeded trace of lengths and token ids, random weights)", "config": config,
+    }))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -381,8 +459,9 @@ def main() -> int:
     ap.add_argument("--profile", action="store_true", help="add per-kernel times of one decode and one prefill step")
     ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
                     help="run only one part (for an external profiler); the other part's figures are null")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous"],
-                    help="decode: the headline measurement; continuous: LLM.generate over many requests")
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "trace"],
+                    help="decode: the headline measurement; continuous: LLM.generate over many requests; "
+                         "trace: the reference's 32-request throughput trace at 1, 4 and 16 running requests")
     ap.add_argument("--model", default="qwen3-0.6b", help="preset shape of the continuous workload")
     ap.add_argument("--shape", default="qwen3-8b",
                     help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
@@ -396,6 +475,8 @@ def main() -> int:
         return 2
     if args.workload == "continuous":
         return run_continuous(args)
+    if args.workload == "trace":
+        return run_trace(args)
 
     from tokamak_amd.config import find_preset
     from tokamak_amd.kernels import ops
