@@ -25,7 +25,8 @@ Two further workloads go through ``LLM.generate`` (scheduler, prompt portions be
 decode tokens, captured decode steps) and print a line of the same form:
 ``--workload continuous`` (256 requests of uniform random lengths, Qwen3-0.6B shape) and
 ``--workload trace`` (the reference's own 32-request throughput trace at 1, 4 and 16
-running requests, with its published figure as ``vs_baseline``).
+running requests, with its published figure as ``vs_baseline``).  ``--workload attention``
+is the reference's microbenchmark of one layer's decode attention at its six shapes.
 """
 
 from __future__ import annotations
@@ -440,6 +441,90 @@ def run_trace(args) -> int:
     return 0
 
 
+def run_attention(args) -> int:
+    """The reference's decode-attention microbenchmark (benchmarks/benchmark_attention.py,
+    README.md:41-53): the attention of one layer in one decode step, alone: the new token's key
+    and value written to its page, then attention over the request's pages; 16 query heads, 8
+    kv heads of 128, pages of 16, bfloat16, every request's pages scattered over the pool
+    (request i holds pages i, B + i, 2B + i, ...).  Here that is one kernel (plus the merge of the
+    key splits) that also norms and rotates the token's query and key.  ``call_us``: the
+    reference's method, one call and a synchronize on the host's clock, median of 50 (mostly the
+    launch from Python); ``graph_us``: a call inside a captured graph of 16, as decode steps run."""
+    import torch
+
+    from tokamak_amd.engine.batch import StepSpan, build_batch
+    from tokamak_amd.kernels import attention as attn
+
+    nh, nkv, hd, ps = 16, 8, 128, 16
+    published = {(1, 512): 241, (8, 512): 271, (16, 512): 323, (16, 2048): 806, (32, 512): 440, (32, 2048): 1409}
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    config = {"heads": nh, "kv_heads": nkv, "head_dim": hd, "page_size": ps}
+    last = None
+    for (batch_size, context), theirs in published.items():
+        pages_each = -(-(context + 1) // ps)
+        k_cache = torch.randn(pages_each * batch_size, nkv * hd * ps, device=dev, dtype=torch.bfloat16)
+        v_cache = torch.randn_like(k_cache)
+        spans = [StepSpan(request=i, tokens=[0], ctx_len=context, state_slot=i,
+                          tables=[[j * batch_size + i for j in range(pages_each)]]) for i in range(batch_size)]
+        batch = build_batch(spans, 1, dev)
+        qkv = torch.randn(batch_size, (nh + 2 * nkv) * hd, device=dev, dtype=torch.bfloat16)
+        weight = torch.ones(hd, device=dev, dtype=torch.float32)
+        angle = torch.rand(batch_size, hd // 2, device=dev, dtype=torch.float32)
+        cos, sin = torch.cos(angle), torch.sin(angle)
+        out = torch.empty(batch_size, nh * hd, device=dev, dtype=torch.bfloat16)
+
+        def call():
+            done = attn.decode_attention_fused(
+                qkv, weight, weight, cos, sin, k_cache, v_cache, batch.block_tables[0], batch, out, num_heads=nh,
+                num_kv_heads=nkv, head_dim=hd, rotary_dim=hd, page_size=ps, eps=1e-6, scale=hd ** -0.5, store=True)
+            assert done
+
+        for _ in range(10):
+            call()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(50):
+            t0 = time.perf_counter()
+            call()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        call_us = statistics.median(times) * 1e6
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for _ in range(16):
+                    call()
+        graph.replay()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(20):
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        graph_us = statistics.median(times) * 1e6 / 16
+        cache_bytes = batch_size * (context + 1) * 2 * nkv * hd * 2
+        tag = f"b{batch_size}_c{context}"
+        config[f"{tag}_call_us"] = round(call_us, 1)
+        config[f"{tag}_graph_us"] = round(graph_us, 2)
+        last = (theirs, call_us, graph_us, cache_bytes)
+    theirs, call_us, graph_us, cache_bytes = last
+    config["baseline"] = "Triton kernel, RTX 3080 Laptop: 241/271/323/806/440/1409 us (reference benchmarks/README.md:48-53)"
+    print(json.dumps({
+        "metric": "decode attention of one layer and step, batch 32 at context 2,048 (us per call, the reference's method)",
+        "value": round(call_us, 1), "unit": "us", "n_gpus": 1, "steps": 50, "warmup": 10,
+        "ms_per_step": round(call_us / 1e3, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": round(call_us / theirs, 4), "dtype": "bf16",
+        "data": "synthetic (random cache, scattered block tables)",
+        "roofline": {"bound": "hbm", "achieved": round(cache_bytes / graph_us / 1e3, 1), "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": round(cache_bytes / graph_us * 1e6 / HBM_PEAK, 4)},
+        "config": config,
+    }))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -459,9 +544,10 @@ def main() -> int:
     ap.add_argument("--profile", action="store_true", help="add per-kernel times of one decode and one prefill step")
     ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
                     help="run only one part (for an external profiler); the other part's figures are null")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "trace"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "trace", "attention"],
                     help="decode: the headline measurement; continuous: LLM.generate over many requests; "
-                         "trace: the reference's 32-request throughput trace at 1, 4 and 16 running requests")
+                         "trace: the reference's 32-request throughput trace at 1, 4 and 16 running requests; "
+                         "attention: the reference's decode-attention microbenchmark")
     ap.add_argument("--model", default="qwen3-0.6b", help="preset shape of the continuous workload")
     ap.add_argument("--shape", default="qwen3-8b",
                     help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
@@ -477,6 +563,8 @@ def main() -> int:
         return run_continuous(args)
     if args.workload == "trace":
         return run_trace(args)
+    if args.workload == "attention":
+        return run_attention(args)
 
     from tokamak_amd.config import find_preset
     from tokamak_amd.kernels import ops
