@@ -38,6 +38,40 @@ template <> struct Elem<bf16_t> {
   static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = float_to_bf16(v); }
 };
 
+// Four consecutive elements p[0..3] of which the first `valid` exist.  `wide`: p is 16-byte
+// (float32) or 8-byte (bfloat16) aligned, so four that all exist go out as one store: a
+// wave's 4-byte stores of an MFMA result tile are sixteen scattered pieces per row of it and
+// cost a product of 64 rows a fifth of its time.
+template <typename T>
+__device__ __forceinline__ void store_four(T* p, float a, float b, float c, float d, int valid, bool wide);
+template <>
+__device__ __forceinline__ void store_four<float>(float* p, float a, float b, float c, float d, int valid, bool wide) {
+  if (wide && valid >= 4) {
+    *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+    return;
+  }
+  if (valid > 0) p[0] = a;
+  if (valid > 1) p[1] = b;
+  if (valid > 2) p[2] = c;
+  if (valid > 3) p[3] = d;
+}
+template <>
+__device__ __forceinline__ void store_four<bf16_t>(bf16_t* p, float a, float b, float c, float d, int valid, bool wide) {
+  if (wide && valid >= 4) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
+    return;
+  }
+  if (valid > 0) p[0] = float_to_bf16(a);
+  if (valid > 1) p[1] = float_to_bf16(b);
+  if (valid > 2) p[2] = float_to_bf16(c);
+  if (valid > 3) p[3] = float_to_bf16(d);
+}
+// Whether rows of `ld` elements starting at p keep every fourth element aligned for store_four.
+template <typename T>
+__device__ __forceinline__ bool rows_take_wide_stores(const T* p, long ld) {
+  return (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T))) == 0 && ld % 4 == 0;
+}
+
 constexpr int kWave = 64;
 
 __device__ __forceinline__ float wave_sum(float v) {

@@ -127,6 +127,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
   }
 
   // acc[i][j][e] = C[batch row j*16 + r][weight row n0 + i*16 + kb*4 + e]
+  const bool wide = rows_take_wide_stores(C, ldc);
 #pragma unroll
   for (int j = 0; j < MT; ++j) {
     const int m = j * 16 + r;
@@ -134,10 +135,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
       const int n = n0 + i * 16 + kb * 4;
-      TO* cp = C + (size_t)m * ldc + n;
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (n + e < N) Elem<TO>::store(cp + e, acc[i][j][e]);
+      store_four<TO>(C + (size_t)m * ldc + n, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3], N - n, wide);
     }
   }
 }
@@ -405,16 +403,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
     }
   }
 
-  // acc[j][e] = C[batch row j*16 + r][column n_wave + kb*4 + e]
+  // acc[j][e] = C[batch row j*16 + r][column n_wave + kb*4 + e]: four columns a store
+  const bool wide = rows_take_wide_stores(C, ldc);
 #pragma unroll
   for (int j = 0; j < MT; ++j) {
     const int m = j * 16 + r;
     if (m >= M) continue;
     const int n = n_wave + kb * 4;
-    TO* cp = C + (size_t)m * ldc + n;
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-      if (n + e < N) Elem<TO>::store(cp + e, acc[j][e]);
+    store_four<TO>(C + (size_t)m * ldc + n, acc[j][0], acc[j][1], acc[j][2], acc[j][3], N - n, wide);
   }
 }
 

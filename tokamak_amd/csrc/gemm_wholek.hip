@@ -242,10 +242,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wholek_kernel(
     res[3] = total[0].w * rstd;
   }
   if (m >= M) return;
-  TO* cp = C + (size_t)m * ldc + n;
-#pragma unroll
-  for (int e = 0; e < 4; ++e)
-    if (n + e < N) Elem<TO>::store(cp + e, res[e]);
+  store_four<TO>(C + (size_t)m * ldc + n, res[0], res[1], res[2], res[3], N - n, rows_take_wide_stores(C, ldc));
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }

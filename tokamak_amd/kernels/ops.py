@@ -402,15 +402,19 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
                                               _stream()), "gemm_tiled")
 
 
+STREAM_SMALL_MATRIX_BYTES = 24 << 20   # below this a product's time is memory round trips, not bytes
+
+
 def stream_waves(rows: int, k: int, gated: bool = False, n: int = 0) -> int:
     """Waves a block of the streaming product.  Eight waves share a chunk of the
-    activations (the block then owns 128 weight rows), which pays when the chunk is large
-    (more than 32 rows) and the walk over K long (the gated product, whose halves meet in
-    one block, and K from 8192 on), and the gated product has columns (``n``) for at least
-    128 such blocks: a small one is spread over more blocks of four."""
-    if gated and 0 < n < 128 * 64:
-        return 4
-    return 8 if rows > 32 and (gated or k >= 8192) else 4
+    activations (the block then owns 128 weight rows, or 64 output columns of the gated
+    product), which pays from 33 rows of activations on, where that chunk is as large as a
+    block's weights, unless the matrix is small (blocks of four are spread over more CUs), has
+    so many rows (``n``: the logits head) that blocks of four already queue several deep on
+    every CU, or, gated, so few columns that blocks of eight would leave CUs idle."""
+    if gated:
+        return 4 if 0 < n < 128 * 64 or rows <= 32 else 8
+    return 8 if rows > 32 and n <= 256 * 128 and 2 * n * k >= STREAM_SMALL_MATRIX_BYTES else 4
 
 
 def _row_scale(sumsq: torch.Tensor | None, m: int, what: str) -> int:
@@ -453,7 +457,7 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
     slabs = _row_scale(sumsq, m, "gemm_stream")
     _note(f"{m}x{n}x{k}", (n * k + m * k) * 2 + splits * m * n * out.element_size(), 2.0 * m * n * k)
     used = _fn("gemm_mfma", "tk_gemm_stream")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
-                                              w.stride(0), ldc, splits, stride, waves or stream_waves(m, k),
+                                              w.stride(0), ldc, splits, stride, waves or stream_waves(m, k, False, n),
                                               _p(sumsq), slabs, float(eps), _stream())
     if used < 1:
         raise KernelError(f"gemm_stream failed with status {used}")
