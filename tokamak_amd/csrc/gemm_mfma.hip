@@ -247,8 +247,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
   constexpr int XP = 16 * MT * 32 / THREADS;  // 16-byte pieces of the activations a thread loads per chunk
   static_assert(XP * THREADS == 16 * MT * 32, "the activations' chunk divides among the threads");
   constexpr int HALF = WAVES / 2;
+  // XBUF: copies of the activations' chunk.  A wave reads weights from its own tile only, so with
+  // two copies written in turn one barrier a chunk is enough (a wave may start to write chunk
+  // i + 1 while others still read chunk i): 3-6 % for blocks of eight waves, which have a CU to
+  // themselves anyway; nothing at up to 16 rows, and blocks of four would lose a place on the CU.
+  constexpr int XBUF = (WAVES == 8 && MT >= 2) ? 2 : 1;
   __shared__ __attribute__((aligned(16))) bf16_t ws[WAVES][16][SLD];
-  __shared__ __attribute__((aligned(16))) bf16_t xs[16 * MT][SLD];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[XBUF][16 * MT][SLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, kb = lane >> 4;
   const int row_block = blockIdx.x, split = blockIdx.y;
@@ -313,13 +318,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
 #define TK_CHUNK(I_)                                                                                \
   {                                                                                                 \
     const int cur_ = chunk_at(I_);                                                                  \
-    __syncthreads(); /* the previous chunk's fragments have been read */                            \
+    const int xb_ = XBUF == 2 ? ((I_) & 1) : 0;                                                     \
+    if (XBUF == 1) __syncthreads(); /* the previous chunk's fragments have been read */             \
     _Pragma("unroll") for (int i = 0; i < 8; ++i)                                                   \
         *reinterpret_cast<u32x4*>(&ws[wave][2 * i + w_row0][w_col]) = wreg[i];                      \
     {                                                                                               \
       const bool inside_ = cur_ * SBK + x_col < K;                                                  \
       _Pragma("unroll") for (int i = 0; i < XP; ++i)                                                \
-          *reinterpret_cast<u32x4*>(&xs[i * (THREADS / 32) + x_row0][x_col]) = inside_ ? xreg[i] : zero; \
+          *reinterpret_cast<u32x4*>(&xs[xb_][i * (THREADS / 32) + x_row0][x_col]) = inside_ ? xreg[i] : zero; \
     }                                                                                               \
     __syncthreads();                                                                                \
     if ((I_) + 1 < nchunks) {                                                                       \
@@ -332,7 +338,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
       wf.u = *reinterpret_cast<const uint4*>(&ws[wave][r][s * 32 + kb * 8]);                        \
       _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                              \
         Frag8 xf;                                                                                   \
-        xf.u = *reinterpret_cast<const uint4*>(&xs[j * 16 + r][s * 32 + kb * 8]);                   \
+        xf.u = *reinterpret_cast<const uint4*>(&xs[xb_][j * 16 + r][s * 32 + kb * 8]);              \
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf.v, acc[j], 0, 0, 0);              \
       }                                                                                             \
     }                                                                                               \
