@@ -305,16 +305,20 @@ def test_qknorm_rope_store(dtype, nh, nkv, hd, ps, rot):
 
 @pytest.mark.parametrize("form", ["float32", "bfloat16", "partial sums", "no norm", "queries only"])
 @pytest.mark.parametrize("nh, nkv, hd, ps", [(8, 2, 128, 16), (3, 3, 64, 32), (14, 1, 128, 64), (5, 5, 64, 16)])
-def test_qknorm_rope_store_of_long_portions(form, nh, nkv, hd, ps):
+@pytest.mark.parametrize("lengths", [[(300, 11), (1, 77), (41, 0)], [(300, 12), (1, 77), (3, 5), (41, 8), (2, 30)]],
+                         ids=["inside a quad", "quads of four"])
+def test_qknorm_rope_store_of_long_portions(form, nh, nkv, hd, ps, lengths):
     """Portions of 300 and 41 tokens that start inside a page, beside a decode token, with a
     number of heads that is no multiple of a wave's share; pages scattered; partial sums as
-    input; what is not written stays as it was."""
+    input; what is not written stays as it was.  "quads of four": the long portions start where
+    both their first token's place in the step and its position are multiples of four, so
+    that the values of four tokens are written as one piece of the page (and a portion's
+    last, broken quad, a short portion in between and the others token by token)."""
     from tokamak_amd.kernels import ops
 
     dtype = torch.float32 if form == "float32" else torch.bfloat16
     eps, theta = 1e-5, 50000.0
     g = torch.Generator().manual_seed(nh + hd)
-    lengths = [(300, 11), (1, 77), (41, 0)]
     need = [-(-(n + ctx) // ps) for n, ctx in lengths]
     order = torch.randperm(sum(need) + 3, generator=g).tolist()
     spans, at = [], 0

@@ -339,22 +339,38 @@ __global__ void qknorm_rope_store_kernel(
 
 // Fast form for head sizes 64 and 128 rotated over their full width (rot == HD):
 // a lane owns 8 consecutive dims of one head (one 16-byte piece), so a wave covers
-// 64*8/HD heads; the rotation partner (dim +- HD/2) sits HD/16 lanes away, the sum
-// of squares is over HD/8 neighbouring lanes, and nothing goes through LDS.
+// 64*8/HD (token, head) pairs; the rotation partner (dim +- HD/2) sits HD/16 lanes away, the
+// sum of squares is over HD/8 neighbouring lanes.  The query heads come token by token; the
+// pairs behind them are the key heads and then the value heads, each head with its tokens in
+// order, so that a wave holds consecutive tokens of one head and its cache writes fall next
+// to each other in the page: a key piece (8 dims of one token) beside those of the next
+// tokens, and the values of four tokens that fill one quad of a page (bfloat16: exchanged
+// through LDS inside the wave) as the page's own 16-byte pieces of two dims by four keys,
+// where token by token they are 2-byte stores 8 bytes apart.
 template <typename T, typename TIN, int HD>
 __global__ __launch_bounds__(256) void qknorm_rope_store_vec_kernel(
     const TIN* __restrict__ qkv, int parts, long part_stride, const float* __restrict__ q_weight,
     const float* __restrict__ k_weight, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const int* __restrict__ positions,
     const int* __restrict__ req_of_token, const int* __restrict__ block_tables,
-    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int nkv_in,
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int N, int nh, int nkv_in,
     int nkv, int ps, int max_pages, float eps, long num_pairs) {
   constexpr int LPH = HD / 8;  // lanes per head
+  __shared__ uint4 s_quad[sizeof(T) == 2 ? 256 : 1];
   const long slot = ((long)blockIdx.x * blockDim.x + threadIdx.x) / LPH;  // (token, head) pair
   if (slot >= num_pairs) return;  // whole LPH-lane groups leave together
   const int sub = threadIdx.x % LPH, d0 = sub * 8;
   const int heads = nh + 2 * nkv_in;
-  const int n = (int)(slot / heads), head = (int)(slot - (long)n * heads);
+  const long q_pairs = (long)N * nh;
+  int n, head;
+  if (slot < q_pairs) {
+    n = (int)((unsigned)slot / (unsigned)nh);
+    head = (int)((unsigned)slot - (unsigned)n * (unsigned)nh);
+  } else {
+    const unsigned behind = (unsigned)(slot - q_pairs), kv = behind / (unsigned)N;
+    n = (int)(behind - kv * (unsigned)N);
+    head = nh + (int)kv;
+  }
   const bool is_q = head < nh, is_k = !is_q && head < nh + nkv_in;
   const TIN* src = qkv + (size_t)n * heads * HD + (size_t)head * HD + d0;
   float x[8];
@@ -412,6 +428,36 @@ __global__ __launch_bounds__(256) void qknorm_rope_store_vec_kernel(
     Store4<T>::at(dst + 4, make_float4(x[4], x[5], x[6], x[7]));
   } else {
     T* base = v_cache + (size_t)page * page_elems + (size_t)(head - nh - nkv_in) * HD * ps;
+    if constexpr (sizeof(T) == 2) {
+      // Four pairs in a row (a "quad" of this wave) that are four consecutive tokens of one
+      // request and head and fill one quad of keys in a page?
+      constexpr int QL = 4 * LPH;  // lanes of a quad
+      const int lane = threadIdx.x & 63, t = (lane / LPH) & 3;
+      const int first = lane / QL * QL + sub;  // the lane with these dims in the quad's first pair
+      const int req = req_of_token[n];
+      const bool fits = n == __shfl(n, first, kWave) + t && pos == __shfl(pos, first, kWave) + t &&
+                        req == __shfl(req, first, kWave) && head == __shfl(head, first, kWave) && ((pos - t) & 3) == 0;
+      const unsigned long long all = QL == 64 ? ~0ull : ((1ull << (QL & 63)) - 1) << (lane / QL * QL);
+      if ((__builtin_amdgcn_ballot_w64(fits) & all) == all) {
+        // every lane leaves its four dim pairs; lane t of the quad takes pair t of all four tokens
+        s_quad[threadIdx.x] = make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]),
+                                         pack_bf16x2(x[6], x[7]));
+        wave_lds_sync();
+        const unsigned* words = reinterpret_cast<const unsigned*>(s_quad);
+        const int quad0 = (int)threadIdx.x / QL * QL + sub;  // thread of the quad's first pair, these dims
+        unsigned r[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) r[k] = words[(quad0 + k * LPH) * 4 + t];  // token k: dims d, d + 1
+        const int d = d0 + 2 * t;
+        uint4 piece;  // [dim d: keys 0..3][dim d + 1: keys 0..3]
+        piece.x = (r[0] & 0xffffu) | (r[1] << 16);
+        piece.y = (r[2] & 0xffffu) | (r[3] << 16);
+        piece.z = (r[0] >> 16) | (r[1] & 0xffff0000u);
+        piece.w = (r[2] >> 16) | (r[3] & 0xffff0000u);
+        *reinterpret_cast<uint4*>(base + ((size_t)(d >> 4) * (ps >> 2) + (off >> 2)) * 64 + (d & 15) * 4) = piece;
+        return;
+      }
+    }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int d = d0 + e;
@@ -442,7 +488,7 @@ TK_API int tk_qknorm_rope_store(int dtype, const void* qkv, int in_f32, int part
 #define TK_QKV(T_, TIN_, HD_)                                                                     \
   qknorm_rope_store_vec_kernel<T_, TIN_, HD_><<<vgrid, 256, 0, stream>>>(                         \
       (const TIN_*)qkv, parts, part_stride, q_weight, k_weight, cos_t, sin_t, positions,          \
-      req_of_token, block_tables, (T_*)q_out, (T_*)k_cache, (T_*)v_cache, nh, nkv_in, nkv, ps,    \
+      req_of_token, block_tables, (T_*)q_out, (T_*)k_cache, (T_*)v_cache, N, nh, nkv_in, nkv, ps, \
       max_pages, eps, pairs)
     if (hd == 128) {
       if (dtype == 0) TK_QKV(float, float, 128);
