@@ -218,9 +218,28 @@ def test_command_line(folders, capsys):
     from tokamak_amd import cli
 
     assert cli.main(["--model", str(folders["A"]), "--prompt-ids", "5,6,7", "--max-new-tokens", "5",
-                     "--temperature", "0", "--dtype", "float32"]) == 0
+                     "--temperature", "0", "--dtype", "float32", "--quiet"]) == 0
     out = capsys.readouterr().out
     assert "[completion (length)]" in out and "[prompt ids]" in out
+
+
+def test_load_is_reported_and_progress_counts_finished_requests(folders, caplog, capsys):
+    """What the reference reports (src/tokamak/engine/llm.py:180-189,299; model/loader.py:95): one
+    line when loading starts, one with the number of tensors read, a bar over finished requests."""
+    import logging
+
+    from tokamak_amd import LLM, SamplingParams
+
+    with caplog.at_level(logging.INFO, logger="tokamak_amd.engine.llm"):
+        llm = LLM(folders["A"], dtype="float32", max_seq_len=64, max_batch_size=2)
+    text = caplog.text
+    assert "Loading" in text and "Qwen3ForCausalLM" in text and "float32" in text
+    tensors = len(plain.read_folder(folders["A"])[1])
+    assert f"Loaded {tensors} tensors" in text and "cache pool of 128 tokens" in text
+    outs = llm.generate(prompt_token_ids=[[1, 2, 3], [4, 5], [6]],
+                        sampling_params=SamplingParams(temperature=0.0, max_new_tokens=3, ignore_eos=True), use_tqdm=True)
+    assert [len(o.output_token_ids) for o in outs] == [3, 3, 3]
+    assert "Generating" in capsys.readouterr().err and "3/3" in llm.last_progress
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

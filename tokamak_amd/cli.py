@@ -32,10 +32,15 @@ def main(argv: list[str] | None = None) -> int:
     parser.add_argument("--random-weights", default=None, metavar="PRESET",
                         help="write a folder of seeded random weights of this shape and use it")
     parser.add_argument("--weights-seed", type=int, default=0)
+    parser.add_argument("--quiet", action="store_true", help="no load report and no progress bar")
     args = parser.parse_args(argv)
 
     from tokamak_amd import LLM, SamplingParams
 
+    if not args.quiet:
+        import logging
+
+        logging.basicConfig(level=logging.INFO, format="%(name)s: %(message)s")
     if (args.model is None) == (args.random_weights is None):
         parser.error("give exactly one of --model and --random-weights")
     tmp = None
@@ -55,12 +60,12 @@ def main(argv: list[str] | None = None) -> int:
                             max_new_tokens=args.max_new_tokens, seed=args.seed)
     if args.prompt_ids is not None:
         ids = [int(t) for t in args.prompt_ids.split(",") if t.strip()]
-        outputs = llm.generate(prompt_token_ids=[ids], sampling_params=params)
+        outputs = llm.generate(prompt_token_ids=[ids], sampling_params=params, use_tqdm=not args.quiet)
         print(f"\n[prompt ids]\n{ids}\n")
     else:
         if llm.tokenizer is None:
             parser.error("the model folder has no tokenizer.json: use --prompt-ids")
-        outputs = llm.generate(llm.chat_prompt(args.prompt), params)
+        outputs = llm.generate(llm.chat_prompt(args.prompt), params, use_tqdm=not args.quiet)
         print(f"\n[prompt]\n{args.prompt}\n")
     out = outputs[0]
     print(f"[completion ({out.finish_reason.value})]")

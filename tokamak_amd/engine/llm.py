@@ -8,6 +8,7 @@ load once, then ``generate`` runs a scheduler-driven step loop and returns one
 from __future__ import annotations
 
 import json
+import logging
 import random
 import time
 from collections.abc import Sequence as AbcSequence
@@ -26,6 +27,8 @@ from tokamak_amd.sampling.params import SamplingParams
 from tokamak_amd.sampling.sampler import sample_tokens
 from tokamak_amd.weights.random_init import expected_tensors_of
 from tokamak_amd.weights.sources import RandomSource, SafetensorsSource
+
+logger = logging.getLogger(__name__)
 
 
 @dataclass
@@ -127,6 +130,11 @@ class LLM:
         self.prefill_chunk = prefill_chunk
         self.eos_token_ids = tuple(plan.eos_token_ids)
         ops.set_library_tuning(tune_library_products)
+        # what the reference reports at load (src/tokamak/engine/llm.py:180-189, model/loader.py:95)
+        logger.info("Loading %s (%s) on %s as %s (max_seq_len=%d, max_batch_size=%d, block_size=%d)",
+                    folder if folder is not None else "seeded random weights", self.architecture.name, device,
+                    self.dtype, self.max_seq_len, max_batch_size, block_size)
+        started = time.perf_counter()
         self.runner = ModelRunner(plan, source, dtype=self.dtype,
                                   page_size=block_size, kv_pool_tokens=kv_pool_tokens,
                                   max_requests=max_batch_size, device=device,
@@ -134,6 +142,8 @@ class LLM:
                                   max_step_tokens=self.max_num_batched_tokens)
         if self.runner.kv_pool_tokens < self.max_seq_len:
             raise RuntimeError(f"the GPU has no room for a cache of max_seq_len ({self.max_seq_len}) tokens")
+        logger.info("Loaded %d tensors in %.1f s; cache pool of %d tokens in pages of %d",
+                    self.runner.num_tensors, time.perf_counter() - started, self.runner.kv_pool_tokens, block_size)
         self.folder = folder
         self.tokenizer = self._load_tokenizer(folder) if folder is not None else None
         self.num_steps = 0
@@ -143,6 +153,8 @@ class LLM:
         self._host_tokens = [torch.empty(max_batch_size, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self._copied = [torch.cuda.Event(), torch.cuda.Event()]
         self._turn = 0
+        self._progress = None
+        self.last_progress = ""   # finished/all requests of the last generate() that showed a bar
 
     @staticmethod
     def _load_tokenizer(folder: Path):
@@ -214,6 +226,14 @@ class LLM:
             scheduler.submit(request)
         for request in requests:
             request.context_limit = self._context_limit(request)
+        # a bar over finished requests, as the reference shows (src/tokamak/engine/llm.py:299)
+        self._progress = None
+        if use_tqdm:
+            try:
+                from tqdm.auto import tqdm
+                self._progress = tqdm(total=len(requests), desc="Generating")
+            except ImportError:
+                pass
         try:
             # One step ahead: a step is planned and launched while the one before it runs; the
             # tokens that one sampled are read (and stop rules applied) meanwhile.  A decoding
@@ -231,6 +251,10 @@ class LLM:
                     self._read(in_flight)
                     in_flight = None
         finally:
+            if self._progress is not None:
+                self.last_progress = f"{self._progress.n}/{self._progress.total}"
+                self._progress.close()
+                self._progress = None
             # also what the scheduler reserved for requests that never reached a step
             self.runner.end_all()
             for request in scheduler.live_requests():
@@ -285,6 +309,8 @@ class LLM:
             if request.accept(token, eos_token_ids=self.eos_token_ids, context_limit=request.context_limit):
                 request.finished_at = stamp
                 self.runner.end(request.rid)
+                if self._progress is not None:
+                    self._progress.update(1)
 
     # ------------------------------------------------------------------
     def _context_limit(self, request: Request) -> int:

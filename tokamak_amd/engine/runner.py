@@ -82,7 +82,7 @@ class ModelRunner:
         self.plan = plan
         self.page_size = page_size
         self.model = LayeredModel(plan, dtype=self.dtype, device=self.device)
-        load_weights(self.model, source, dtype=self.dtype, device=self.device)
+        self.num_tensors = load_weights(self.model, source, dtype=self.dtype, device=self.device)
         groups, layouts = self.model.cache_layout()
         self.num_groups = len(groups)
         self._groups = groups
