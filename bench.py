@@ -18,7 +18,8 @@ the cache of the live requests at the mean context of the timed steps, divided b
 time.  Fractions are of the published peaks (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s);
 ``peaks`` holds what two microbenchmarks of this program reach on this GPU (streaming
 reads and copies of 4 GiB; back-to-back MFMA from registers), and ``frac_of_measured``
-the same fractions of those.  ``--profile`` adds ``kernels``: one decode step and one
+the same fractions of those.  ``peak_memory_gib`` is the most GPU memory allocated at any
+time of the run.  ``--profile`` adds ``kernels``: one decode step and one
 prefill step with every kernel call timed by events, summed by kind of call.
 
 Two further workloads go through ``LLM.generate`` (scheduler, prompt portions beside
@@ -636,6 +637,11 @@ def main() -> int:
         if step_s is None:
             result.update({"value": result["prefill"]["value"], "ms_per_step": result["prefill"]["ms"], "steps": 5})
     result["points"] = points
+    # as the reference's latency benchmark reads it (benchmarks/benchmark_latency.py:144-146): weights,
+    # the cache pools of every measured batch size (one at a time) and the largest step's activations
+    import torch
+
+    result["peak_memory_gib"] = round(torch.cuda.max_memory_allocated() / 2 ** 30, 2)
     if peaks:
         result["peaks"] = peaks
     if kernels:
