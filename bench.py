@@ -27,7 +27,8 @@ decode tokens, captured decode steps) and print a line of the same form:
 ``--workload continuous`` (256 requests of uniform random lengths, Qwen3-0.6B shape) and
 ``--workload trace`` (the reference's own 32-request throughput trace at 1, 4 and 16
 running requests, with its published figure as ``vs_baseline``).  ``--workload attention``
-is the reference's microbenchmark of one layer's decode attention at its six shapes.
+is the reference's microbenchmark of one layer's decode attention at its six shapes, and
+``--workload latency`` its single-sequence latency measurement (512 prompt + 128 new tokens).
 """
 
 from __future__ import annotations
@@ -526,6 +527,54 @@ def run_attention(args) -> int:
     return 0
 
 
+def run_latency(args) -> int:
+    """The reference's single-sequence latency measurement (benchmarks/benchmark_latency.py:63-98,
+    126-129; README.md:16-24): one random prompt of 512 tokens through the model in one step, its first
+    token read on the host (prefill_ms), then 128 greedy tokens one step at a time, every token read on the
+    host before the next step starts (decode tok/s, inter-token ms), on the Qwen3-0.6B shape (random weights
+    here), pages of 16; one untimed pass, then the median of three.  The published figures are for an RTX
+    3080 Laptop GPU: 70.7 ms, 21.0 tok/s and 1.47 GiB with the reference's Triton kernel."""
+    import torch
+
+    from tokamak_amd.config import find_preset
+    from tokamak_amd.engine.runner import StepEntry
+    from tokamak_amd.kernels import ops
+    from tokamak_amd.sampling.sampler import greedy_tokens
+
+    prompt_tokens, new_tokens = 512, 128
+    arch, cfg = find_preset(args.model)
+    ops.set_library_tuning(not args.no_tune)
+    runner = make_runner(arch, cfg, args.dtype, prompt_tokens + new_tokens, 1)
+    prompt = random_prompt(cfg.vocab_size, prompt_tokens, 0)
+    passes = []
+    for _ in range(1 + 3):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        token = int(greedy_tokens(runner.step([StepEntry("one", prompt, [prompt_tokens - 1])]))[0])
+        t1 = time.perf_counter()
+        for _ in range(new_tokens):
+            token = int(greedy_tokens(runner.step([StepEntry("one", [token], [0])]))[0])
+        t2 = time.perf_counter()
+        runner.end("one")
+        passes.append((t1 - t0, t2 - t1))
+    prefill_s = statistics.median(p for p, _ in passes[1:])
+    decode_s = statistics.median(d for _, d in passes[1:])
+    value = new_tokens / decode_s
+    print(json.dumps({
+        "metric": "decode tok/s of one sequence, 512 prompt tokens + 128 greedy tokens, every token read before the next step",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": new_tokens, "warmup": new_tokens,
+        "ms_per_step": round(decode_s / new_tokens * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": round(value / 21.0, 2), "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (seeded random token ids, random weights)",
+        "prefill": {"value": round(prompt_tokens / prefill_s, 1), "tokens": prompt_tokens, "ms": round(prefill_s * 1e3, 3)},
+        "peak_memory_gib": round(torch.cuda.max_memory_allocated() / 2 ** 30, 2),
+        "config": {"model": f"{args.model}-shaped", "prompt_tokens": prompt_tokens, "new_tokens": new_tokens, "page_size": PAGE_SIZE,
+                   "baseline": "70.7 ms prefill, 21.0 tok/s, 1.47 GiB: paged cache + Triton kernel, RTX 3080 Laptop "
+                               "(reference benchmarks/README.md:24)"},
+    }))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -545,10 +594,11 @@ def main() -> int:
     ap.add_argument("--profile", action="store_true", help="add per-kernel times of one decode and one prefill step")
     ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
                     help="run only one part (for an external profiler); the other part's figures are null")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "trace", "attention"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "trace", "attention", "latency"],
                     help="decode: the headline measurement; continuous: LLM.generate over many requests; "
                          "trace: the reference's 32-request throughput trace at 1, 4 and 16 running requests; "
-                         "attention: the reference's decode-attention microbenchmark")
+                         "attention: the reference's decode-attention microbenchmark; "
+                         "latency: its single-sequence latency measurement (512 + 128 tokens)")
     ap.add_argument("--model", default="qwen3-0.6b", help="preset shape of the continuous workload")
     ap.add_argument("--shape", default="qwen3-8b",
                     help="preset whose layer sizes the decode/prefill measurement uses (default: the headline one)")
@@ -566,6 +616,8 @@ def main() -> int:
         return run_trace(args)
     if args.workload == "attention":
         return run_attention(args)
+    if args.workload == "latency":
+        return run_latency(args)
 
     from tokamak_amd.config import find_preset
     from tokamak_amd.kernels import ops

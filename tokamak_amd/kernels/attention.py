@@ -9,6 +9,7 @@ from tokamak_amd.kernels import ops
 MFMA_HEAD_DIMS = (64, 128)
 DECODE_WAVES = 16           # waves of a decode block (csrc/attention_mfma.hip: kDecodeWaves)
 TARGET_DECODE_WAVES = 4096  # waves wanted in flight; beyond that splits only cost a merge
+MERGE_WORTH_TILES = 2       # tiles of 16 keys a wave must save for a split of the keys to pay for its merge
 TILE_SPLIT_BELOW_BLOCKS = 256   # a portion with fewer blocks than this has its keys split ...
 TILE_SPLIT_MIN_KEYS = 512       # ... into pieces no shorter than this
 TARGET_TILE_BLOCKS = 1024
@@ -34,7 +35,17 @@ def decode_split(num_decode: int, num_kv_heads: int, max_len: int) -> tuple[int,
     most = max(1, -(-max_len // least))
     nsplit = min(most, max(1, -(-TARGET_DECODE_WAVES // (DECODE_WAVES * pairs))))
     split = -(-(-(-max_len // nsplit)) // least) * least
-    return split, max(1, -(-max_len // split))
+    nsplit = max(1, -(-max_len // split))
+    # A wave walks its tiles of 16 keys one after the other, about 2 us each from HBM, and the
+    # merge is a kernel of its own (4-5 us): splitting pays when it saves a wave two tiles or
+    # more (measured on a 0.6B-shaped model: 16 requests of some 600 keys, where two splits
+    # save one tile, +3 % a step without them; one request of 600 keys, where three splits
+    # save two, 3 % slower without them).
+    if nsplit > 1:
+        whole = -(-(-(-max_len // 16)) // DECODE_WAVES)
+        if whole - split // least < MERGE_WORTH_TILES:
+            return -(-max_len // least) * least, 1
+    return split, nsplit
 
 
 def tile_split(num_tiles: int, blocks_per_tile: int, max_len: int) -> tuple[int, int]:
