@@ -1,7 +1,8 @@
 """Layers of Qwen3-8B's shape (width 4096, 32 query and 8 kv heads of 128, feed-forward
 12288; two layers and a vocabulary of 8192 to keep it small), of Qwen3-32B's (width 5120,
-64 query heads in groups of 8, feed-forward 25600; one layer) and of Qwen3-0.6B's (width
-1024, 16 query heads in groups of 2, tied embeddings): float32 and bfloat16 logits
+64 query heads in groups of 8, feed-forward 25600; one layer), of Qwen3-0.6B's (width
+1024, 16 query heads in groups of 2, tied embeddings) and of Qwen3-14B's (40 query heads in
+groups of 5, feed-forward 17408; one layer): float32 and bfloat16 logits
 against the plain implementation, whole, in portions and token by token, and mixed
 with a second request."""
 
@@ -17,8 +18,8 @@ from tokamak_amd.models import qwen3
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module", params=[("qwen3-8b", 2), ("qwen3-32b", 1), ("qwen3-0.6b", 2)],
-                ids=["8b", "32b", "0.6b"])
+@pytest.fixture(scope="module", params=[("qwen3-8b", 2), ("qwen3-32b", 1), ("qwen3-0.6b", 2), ("qwen3-14b", 1)],
+                ids=["8b", "32b", "0.6b", "14b"])
 def model(request):
     from tokamak_amd.weights.random_init import expected_tensors_of
     from tokamak_amd.weights.sources import RandomSource

@@ -203,7 +203,10 @@ PRESETS = {
     "tiny-a": _shape(256, 64, 2, 4, 2, 16, 128, 10000.0, 128, True),
     "tiny-b": _shape(384, 96, 3, 6, 3, 32, 200, 1000000.0, 256, False, eps=1e-5),
     "qwen3-0.6b": _shape(151936, 1024, 28, 16, 8, 128, 3072, 1000000.0, 40960, True),
+    "qwen3-1.7b": _shape(151936, 2048, 28, 16, 8, 128, 6144, 1000000.0, 40960, True),
+    "qwen3-4b": _shape(151936, 2560, 36, 32, 8, 128, 9728, 1000000.0, 40960, True),
     "qwen3-8b": _shape(151936, 4096, 36, 32, 8, 128, 12288, 1000000.0, 40960, False),
+    "qwen3-14b": _shape(151936, 5120, 40, 40, 8, 128, 17408, 1000000.0, 40960, False),
     "qwen3-32b": _shape(151936, 5120, 64, 64, 8, 128, 25600, 1000000.0, 40960, False),
 }
 
