@@ -82,11 +82,12 @@ class LayerRecording:
     result: object
 
     def launch(self, tensors: dict[tuple, torch.Tensor], then):
+        address = {key: t.data_ptr() for key, t in tensors.items()}     # once a layer, not once a patch
         for fn, args, patches, status in self.calls:
             if patches:
                 args = list(args)
                 for index, key, offset in patches:
-                    args[index] = c_void_p(tensors[key].data_ptr() + offset)
+                    args[index] = address[key] + offset     # a plain int is taken for a pointer argument
             got = fn(*args)
             if got != status:
                 raise ops.KernelError(f"a replayed launch returned {got}, the recorded one {status}")
