@@ -549,13 +549,14 @@ def test_consumers_add_partial_sums():
 
 
 @pytest.mark.parametrize("M, I, K", [(1, 64, 64), (8, 12288, 4096), (64, 200, 96), (33, 3072, 1024), (17, 136, 120)])
-def test_fused_gate_up_silu_product(M, I, K):
+@pytest.mark.parametrize("waves", [0, 2, 4, 8], ids=["chosen", "two waves", "four", "eight"])
+def test_fused_gate_up_silu_product(M, I, K, waves):
     from tokamak_amd.kernels import ops
 
     x = rand(M, K, seed=1).to(torch.bfloat16)
     w = rand(2 * I, K, seed=2, scale=2 * K ** -0.5).to(torch.bfloat16)
     out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ops.gemm_stream_swiglu(x.to(DEV), w.to(DEV), out)
+    ops.gemm_stream_swiglu(x.to(DEV), w.to(DEV), out, waves=waves)
     g = x.double() @ w[:I].double().T
     u = x.double() @ w[I:].double().T
     torch.testing.assert_close(out.cpu().double(), g / (1 + torch.exp(-g)) * u, rtol=2e-2, atol=1e-2)
@@ -599,7 +600,8 @@ def test_whole_k_product_adds_into_the_stream(M, N, K, waves):
     assert torch.equal(again, sumsq)
 
 
-@pytest.mark.parametrize("M, N, K", [(1, 6144, 4096), (8, 4096, 4096), (16, 1000, 264), (5, 100, 72), (3, 2048, 200)])
+@pytest.mark.parametrize("M, N, K", [(1, 6144, 4096), (8, 4096, 4096), (16, 1000, 264), (5, 100, 72), (3, 2048, 200),
+                                     (4, 96, 8136)])
 def test_products_apply_a_pending_row_scale(M, N, K):
     """RMSNorm = row scale x column scale; given bf16(x * gamma) and the rows' sums of squares
     in slabs, the streaming products (plain, split over K, gated) and the whole-K product
@@ -634,7 +636,9 @@ def test_products_apply_a_pending_row_scale(M, N, K):
         g, u = want[:, :half], want[:, half:]
         gated = g / (1 + torch.exp(-g)) * u
         gtol = dict(rtol=2e-2, atol=1e-2 * gated.abs().max().item())
-        for fn in (ops.gemm_stream_swiglu, lambda a, b, c, **kw: ops.gemm_wholek(a, b, c, gated=True, **kw)):
+        for fn in (ops.gemm_stream_swiglu, lambda a, b, c, **kw: ops.gemm_stream_swiglu(a, b, c, waves=2, **kw),
+                   lambda a, b, c, **kw: ops.gemm_stream_swiglu(a, b, c, waves=4, **kw),
+                   lambda a, b, c, **kw: ops.gemm_wholek(a, b, c, gated=True, **kw)):
             out = torch.full((M, half), float("nan"), dtype=torch.bfloat16, device=DEV)
             fn(*args, out, sumsq=sumsq.to(DEV), eps=eps)
             torch.testing.assert_close(out.cpu().double(), gated, **gtol)

@@ -29,8 +29,15 @@ def test_splits_stay_within_the_chunks_and_fill_the_gpu_evenly(n, k, m):
         assert waves == 4
 
 
-def test_the_gated_product_takes_eight_waves_only_when_it_has_the_columns():
-    assert ops.stream_waves(64, 4096, True, 12288) == 8
-    assert ops.stream_waves(64, 1024, True, 3072) == 4      # too few columns for blocks of eight
-    assert ops.stream_waves(32, 4096, True, 12288) == 4
-    assert ops.stream_waves(8, 4096, True, 12288) == 4
+def test_the_gated_product_picks_its_block_size_by_rows_columns_and_row_length():
+    # (rows, K, output columns) -> waves: the shapes the rule was measured on
+    cases = {
+        (1, 1024, 3072): 2, (16, 1024, 3072): 2, (48, 1024, 3072): 2, (64, 1024, 3072): 4,       # 0.6B
+        (8, 2048, 6144): 2, (32, 2048, 6144): 2, (48, 2048, 6144): 2, (64, 2048, 6144): 4,        # 1.7B
+        (8, 2560, 9728): 2, (32, 2560, 9728): 2, (48, 2560, 9728): 8,                             # 4B
+        (1, 4096, 12288): 4, (16, 4096, 12288): 4, (32, 4096, 12288): 4, (64, 4096, 12288): 8,    # 8B: rows of 8 KB
+        (8, 5120, 17408): 2, (24, 5120, 17408): 4, (64, 5120, 17408): 8,                          # 14B
+        (8, 5120, 25600): 2, (32, 5120, 25600): 4, (33, 5120, 25600): 8,                          # 32B
+    }
+    for (rows, k, n), waves in cases.items():
+        assert ops.stream_waves(rows, k, True, n) == waves, (rows, k, n)

@@ -232,7 +232,7 @@ constexpr int SLD = SBK + 8;    // LDS row stride in elements
 // leaves, gemm_wholek.hip); the product is linear in a row's scale, so the block multiplies
 // row m of its sums by rstd[m] = rsqrt(sum_s sumsq[s][m] / K + eps) before it stores them
 // (partial sums of a split too: their sum is scaled alike) or gates them.
-constexpr int kRowScaleLoads = 32;  // slab sums a thread of a four-wave block holds: slabs <= 16 * this
+constexpr int kRowScaleSlabs = 512;  // most slabs of sums of squares: a thread holds kRowScaleSlabs / (threads / 16) of them
 struct RowScale {
   const float* sumsq;  // [slabs][M]: sums of squares of the rows over slabs of columns; nullptr: no scaling
   int slabs;
@@ -352,13 +352,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
   // RowScale: the slab sums are asked for now and first looked at after the walk over K (a
   // block that waited for them here would start its walk a memory round trip late).
   constexpr int STAT_STEP = THREADS / 16;
-  float stat[MT == 1 ? kRowScaleLoads : 1];
+  constexpr int STAT_LOADS = kRowScaleSlabs / STAT_STEP;
+  float stat[MT == 1 ? STAT_LOADS : 1];
   if constexpr (MT == 1) {
 #pragma unroll
-    for (int u = 0; u < kRowScaleLoads; ++u) stat[u] = 0.f;
+    for (int u = 0; u < STAT_LOADS; ++u) stat[u] = 0.f;
     if (scaled && (tid & 15) < M) {
 #pragma unroll
-      for (int u = 0; u < kRowScaleLoads; ++u) {
+      for (int u = 0; u < STAT_LOADS; ++u) {
         const int sl = (tid >> 4) + u * STAT_STEP;
         if (sl < scale.slabs) stat[u] = scale.sumsq[(size_t)sl * M + (tid & 15)];
       }
@@ -377,7 +378,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
     if (scaled) {
       float ss = 0.f;
 #pragma unroll
-      for (int u = 0; u < kRowScaleLoads; ++u) ss += stat[u];
+      for (int u = 0; u < STAT_LOADS; ++u) ss += stat[u];
       s_stat[tid] = ss;
       __syncthreads();
       float total = 0.f;
@@ -439,13 +440,18 @@ static int launch_stream_shape(const void* A, const void* W, void* C, int M, int
   return launch_status();
 }
 
-// waves: 4 or 8 a block.
+// waves: 4 or 8 a block; the gated product also 2.
 template <typename TO, bool GATED>
 static int launch_stream(int waves, const void* A, const void* W, void* C, int M, int N, int K,
                          long lda, long ldw, long ldc, int cps, int KS, long split_stride, RowScale scale,
                          hipStream_t stream) {
   if (waves >= 8)
     return launch_stream_shape<TO, GATED, 8>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, scale, stream);
+  if constexpr (GATED) {
+    // two waves (one gate tile, one up tile: 16 output columns a block): more, smaller blocks
+    if (waves == 2)
+      return launch_stream_shape<TO, GATED, 2>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, scale, stream);
+  }
   return launch_stream_shape<TO, GATED, 4>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, scale, stream);
 }
 
@@ -459,7 +465,7 @@ TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, 
                           const float* sumsq, int slabs, float eps, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535) return -1;
-  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > 16 * kRowScaleLoads || waves >= 8)) return -1;
+  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 8)) return -1;
   const RowScale scale{sumsq, slabs, eps};
   if (splits > 1 && out_dtype != 0) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
@@ -477,7 +483,7 @@ TK_API int tk_gemm_stream_swiglu(const void* A, const void* W, void* C, int M, i
                                  hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
-  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > 16 * kRowScaleLoads || waves >= 8)) return -1;
+  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 8)) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
   return launch_stream<bf16_t, true>(waves, A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0,
                                      RowScale{sumsq, slabs, eps}, stream);

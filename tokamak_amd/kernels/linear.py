@@ -26,7 +26,7 @@ from tokamak_amd.kernels import ops
 # longer K the split product and the norm kernel after it are as fast (measured: the o
 # projection of an 8B-shaped layer gains 2 us, its down projection nothing).
 ADD_INTO_MAX_K = 16 * 256
-GATED_WHOLEK_MAX_BYTES = 64 << 20   # gate and up together, up to which the whole-K form takes the gated product
+GATED_WHOLEK_MAX_BYTES = 32 << 20   # gate and up together, up to which the whole-K form takes the gated product
 
 
 @dataclass
@@ -140,10 +140,10 @@ def gated_linear(x: torch.Tensor | DeferredNorm, gate_up: torch.Tensor) -> torch
     """
     m = x.shape[0]
     inter = gate_up.shape[0] // 2
-    # A small pair of matrices has too few columns for the streaming kernel's blocks, which cannot
-    # split K under the gate: the whole-K form covers 16 columns a block and lets its waves split K
-    # (0.6B-shaped, 13 MB: 6.6 against 8.6 us; 1.7B-shaped, 50 MB: 13.8 against 16.0 us at one row, the
-    # same at sixteen; 4B-shaped, 100 MB: 26 against 23 us).
+    # A very small pair of matrices (0.6B-shaped: 13 MB) goes to the whole-K form, whose blocks of 16
+    # columns let their waves split K, which the streaming kernel cannot do under the gate: in a
+    # decode step 6.6 us against 8.6 with blocks of four waves and 7.8 with blocks of two (whose start
+    # costs more than their size saves there); from 50 MB on the streaming kernel is ahead.
     small = 2 * gate_up.numel() <= GATED_WHOLEK_MAX_BYTES
     if isinstance(x, DeferredNorm):
         if _few_rows_fit(m, x.scaled, gate_up, ops.ROW_SCALE_MAX_ROWS) and x.sumsq.shape[0] <= ops.ROW_SCALE_MAX_SLABS:
