@@ -521,3 +521,123 @@ def test_a_state_mixer_recorded_into_a_graph_sees_every_token_once(dtype):
             last[r] = int(x[row].argmax())
     assert len(graphed._graphs) == 2
     assert sum(g.replays for g in graphed._graphs.values()) == 12 - 2     # each shape's first step ran eagerly
+
+
+# ---------------------------------------------------------------------------
+# a whole toy architecture: config.json keys of its own -> registry -> folder -> LLM -> command line
+# ---------------------------------------------------------------------------
+def register_toy_architecture():
+    """An architecture defined in this file: its own config.json keys and tensor names, a state
+    mixer between two attention layers (one windowed), a routed feed-forward.  Nothing under
+    tokamak_amd/ knows it."""
+    from dataclasses import dataclass
+
+    from tokamak_amd.config import LayerCall, LayerSpec, ModelPlan, PartSpec, SubPart
+    from tokamak_amd.config.registry import Architecture, register_architecture
+
+    register_toys()
+    name = "ToyMemoryForCausalLM"
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str
+        vocab: int
+        width: int
+        heads: int
+        kv_heads: int
+        head_size: int
+        inner: int
+        window: int
+        eps: float
+        longest: int
+        eos_token_ids: tuple = ()
+
+    def parse(raw, eos_ids=()):
+        if raw.get("toy_memory_layers", 1) != 1:
+            raise ValueError("this toy has one memory layer")
+        return ToyConfig(name, int(raw["toy_vocab"]), int(raw["toy_width"]), int(raw["toy_heads"]), int(raw["toy_kv_heads"]),
+                         int(raw["toy_head_size"]), int(raw["toy_inner"]), int(raw["toy_window"]),
+                         float(raw["toy_eps"]), int(raw["toy_longest"]), tuple(eos_ids))
+
+    def to_json(cfg):
+        return {"architectures": [name], "toy_vocab": cfg.vocab, "toy_width": cfg.width, "toy_heads": cfg.heads,
+                "toy_kv_heads": cfg.kv_heads, "toy_head_size": cfg.head_size, "toy_inner": cfg.inner,
+                "toy_window": cfg.window, "toy_eps": cfg.eps, "toy_longest": cfg.longest}
+
+    def plan(cfg):
+        norm = PartSpec.of("rmsnorm", dim=cfg.width, eps=cfg.eps)
+        n = lambda prefix: SubPart("norm", norm, prefix)   # noqa: E731
+        attn = lambda window: SubPart("mixer", PartSpec.of(   # noqa: E731
+            "gqa_attention", hidden_size=cfg.width, num_heads=cfg.heads, num_kv_heads=cfg.kv_heads, head_dim=cfg.head_size,
+            qk_norm_eps=cfg.eps, softmax_scale=cfg.head_size ** -0.5, window=window), "attend.")
+        rope = SubPart("position", PartSpec.of("rotary_half", rotary_dim=cfg.head_size, theta=5000.0), shared=True)
+        dense = SubPart("feed_forward", PartSpec.of("swiglu", hidden_size=cfg.width, intermediate_size=cfg.inner), "ff.")
+        routed = SubPart("feed_forward", PartSpec.of("toy_top1", hidden_size=cfg.width), "experts.")
+        layers = (
+            LayerSpec.of(PartSpec.of("pre_norm"), mixer_norm=n("a."), mixer=attn(None), feed_forward_norm=n("b."),
+                         feed_forward=dense, position=rope),
+            LayerSpec.of(PartSpec.of("pre_norm"), mixer_norm=n("a."),
+                         mixer=SubPart("mixer", PartSpec.of("toy_running_mean", hidden_size=cfg.width), "memory."),
+                         feed_forward_norm=n("b."), feed_forward=routed),
+            LayerSpec.of(PartSpec.of("pre_norm"), mixer_norm=n("a."), mixer=attn(cfg.window), feed_forward_norm=n("b."),
+                         feed_forward=dense, position=rope),
+        )
+        return ModelPlan(vocab_size=cfg.vocab, hidden_size=cfg.width, max_position_embeddings=cfg.longest,
+                         tie_word_embeddings=False, embedding=PartSpec.of("token_embedding", vocab_size=cfg.vocab, dim=cfg.width),
+                         layers=layers, order=(LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 2)), final_norm=norm,
+                         head=PartSpec.of("linear_head", vocab_size=cfg.vocab, dim=cfg.width, tied=False),
+                         embedding_prefix="words.", layer_prefix="stack.{}.", final_norm_prefix="last.", head_prefix="out.",
+                         eos_token_ids=cfg.eos_token_ids)
+
+    presets = {"toy-memory": ToyConfig(name, 90, 48, 3, 1, 16, 80, 24, 1e-5, 160)}
+    register_architecture(Architecture(name=name, parse=parse, plan=plan, to_json=to_json, presets=presets), replace=True)
+    return presets["toy-memory"]
+
+
+def test_a_toy_architecture_goes_from_config_json_to_generated_tokens(tmp_path, capsys):
+    """Registered from here, the toy is found by the name in its folder's config.json, its weights
+    are bound by its own tensor names (and a missing one is reported), it generates the same tokens
+    with a roomy pool and whole prompts as with a tight pool and prompts in portions, and the command
+    line finds its preset."""
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+
+    from tokamak_amd import LLM, SamplingParams, cli
+    from tokamak_amd.config import find_preset
+    from tokamak_amd.weights import write_random_model
+    from tokamak_amd.weights.loader import WeightError
+
+    cfg = register_toy_architecture()
+    assert find_preset("toy-memory")[1] == cfg
+    folder = write_random_model(tmp_path / "toy", cfg, seed=4, matrix_std=0.15, vector_jitter=0.1)
+    with safe_open(str(folder / "model.safetensors"), framework="pt") as f:
+        names = set(f.keys())
+        tensors = {k: f.get_tensor(k) for k in names}
+    assert {"words.weight", "out.weight", "last.weight", "stack.1.memory.mix.weight", "stack.1.experts.router.weight",
+            "stack.2.attend.q_proj.weight"} <= names
+
+    params = SamplingParams(temperature=0.0, max_new_tokens=40, ignore_eos=True)
+    prompts = [random_ids(cfg.vocab, n, 70 + i) for i, n in enumerate([40, 9, 75, 3, 28])]
+    roomy = LLM(folder, dtype="float32", block_size=8, max_batch_size=8)
+    assert roomy.architecture.name == "ToyMemoryForCausalLM" and roomy.max_seq_len == 160
+    want = roomy.generate(prompt_token_ids=prompts, sampling_params=params)
+    tight = LLM(folder, dtype="float32", block_size=8, kv_pool_tokens=160, max_batch_size=4, max_num_batched_tokens=16,
+                prefill_chunk=7)
+    got = tight.generate(prompt_token_ids=prompts, sampling_params=params)
+    assert [o.output_token_ids for o in got] == [o.output_token_ids for o in want]
+    assert tight.num_preemptions > 0
+    tight.runner.manager.check()
+    half = LLM(folder, dtype="bfloat16", block_size=8, max_batch_size=8).generate(prompt_token_ids=prompts, sampling_params=params)
+    assert all(len(o.output_token_ids) == 40 for o in half)
+
+    broken = tmp_path / "broken"
+    broken.mkdir()
+    (broken / "config.json").write_text((folder / "config.json").read_text())
+    del tensors["stack.1.memory.mix.weight"]
+    save_file(tensors, str(broken / "model.safetensors"))
+    with pytest.raises(WeightError, match="stack.1.memory.mix.weight"):
+        LLM(broken, dtype="float32", block_size=8)
+
+    assert cli.main(["--random-weights", "toy-memory", "--prompt-ids", "5,6,7", "--max-new-tokens", "4", "--temperature", "0",
+                     "--dtype", "float32", "--page-size", "8", "--quiet"]) == 0
+    assert "[completion (length)]" in capsys.readouterr().out
