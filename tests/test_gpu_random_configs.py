@@ -66,3 +66,71 @@ def test_random_configurations_replayed_mixed_match_plain(tmp_path, first):
             except AssertionError as e:
                 raise AssertionError(f"{what}, {dtype}: {e}") from None
             del runner
+
+
+def drawn_wide(seed):
+    """Sizes at which the weight-streaming products, their split plans and the matrix-core
+    attention kernels run: widths of 256 to 5,600 in steps of 8, feed-forwards up to 26,000,
+    batches of 1 to 64 requests."""
+    rng = random.Random(77_000 + seed)
+    head_dim = rng.choice([64, 128, 128, 96, 256, 80])
+    kv_heads = rng.choice([1, 2, 4, 8])
+    groups = rng.choice([1, 2, 3, 4, 5, 6, 7, 8])
+    hidden = rng.choice([8 * rng.randrange(32, 700), 256 * rng.randrange(2, 22), 128 * rng.randrange(4, 44)])
+    inter = rng.choice([8 * rng.randrange(64, 3300), 256 * rng.randrange(4, 100), 128 * rng.randrange(8, 200)])
+    vocab = rng.choice([rng.randrange(1000, 20000), 8192, 16 * rng.randrange(100, 1200)])
+    cfg = Qwen3Config("Qwen3ForCausalLM", vocab_size=vocab, hidden_size=hidden, num_layers=rng.randint(1, 2),
+                      num_attention_heads=kv_heads * groups, num_kv_heads=kv_heads, head_dim=head_dim,
+                      intermediate_size=inter, rms_norm_eps=1e-6, rope_theta=1e6, max_position_embeddings=4096,
+                      tie_word_embeddings=rng.random() < 0.5)
+    batch = rng.choice([1, 2, 3, 5, 8, 9, 16, 17, 24, 32, 33, 40, 48, 49, 64])
+    prompts = [[rng.randrange(vocab) for _ in range(rng.randint(3, 40))] for _ in range(batch)]
+    fed = [[rng.randrange(vocab) for _ in range(3)] for _ in range(batch)]
+    return cfg, prompts, fed, sorted(rng.sample(range(batch), min(batch, 3)))
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 5, 8, 13, 21])
+def test_random_wide_configurations_prefilled_together_and_decoded_match_plain(seed):
+    """All prompts in one step, then three decode steps of the whole batch; three of the
+    requests are compared with the plain implementation at every step."""
+    import torch
+
+    from tokamak_amd.engine.runner import ModelRunner, StepEntry
+    from tokamak_amd.models import qwen3
+    from tokamak_amd.weights.random_init import expected_tensors_of
+    from tokamak_amd.weights.sources import RandomSource
+
+    cfg, prompts, fed, checked = drawn_wide(seed)
+    what = (f"seed {seed}: width {cfg.hidden_size}, heads {cfg.num_attention_heads}/{cfg.num_kv_heads} of "
+            f"{cfg.head_dim}, feed-forward {cfg.intermediate_size}, vocabulary {cfg.vocab_size}, "
+            f"{cfg.num_layers} layers, batch {len(prompts)}")
+    plan = qwen3.plan(cfg)
+    expected = {n: s for n, s in expected_tensors_of(plan).items() if not s.ignored}
+    source = RandomSource(expected, seed=seed, matrix_std=0.02, vector_jitter=0.1, dtype=torch.bfloat16)
+    weights = {name: source.fetch(name) for name in expected}
+
+    class Fixed:
+        def names(self):
+            return {n: (tuple(t.shape), t.dtype) for n, t in weights.items()}
+
+        def fetch(self, name):
+            return weights[name]
+
+    cfg_json = qwen3.to_config_json(cfg)
+    w = {n: t.float() for n, t in weights.items()}
+    want = {i: plain.logits(prompts[i] + fed[i], cfg_json, w) for i in checked}
+    for dtype in ("float32", "bfloat16"):
+        runner = ModelRunner(plan, Fixed(), dtype=dtype, page_size=16, kv_pool_tokens=64 * 80, max_requests=64)
+        steps = [[StepEntry(f"r{i}", p, [len(p) - 1]) for i, p in enumerate(prompts)]]
+        steps += [[StepEntry(f"r{i}", [f[t]], [0]) for i, f in enumerate(fed)] for t in range(3)]
+        for t, entries in enumerate(steps):
+            out = runner.step(entries).cpu()
+            for i in checked:
+                row = want[i][len(prompts[i]) - 1 + t]
+                tol = TOL[dtype]["tol_abs"] + TOL[dtype].get("tol_rel_to_scale", 0.0) * float(row.abs().max())
+                err = (out[i] - row).abs().max().item()
+                assert err < tol, f"{what}, {dtype}, step {t}, request {i}: {err:.3e} > {tol:.3e}"
+        for i in range(len(prompts)):
+            runner.end(f"r{i}")
+        runner.manager.check()
+        del runner
