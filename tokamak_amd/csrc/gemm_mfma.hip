@@ -226,6 +226,10 @@ constexpr int SLD = SBK + 8;    // LDS row stride in elements
 // A second chunk of weights in flight per wave was measured too and gained nothing: at 64
 // rows the kernel is held by LDS traffic (seven bytes through LDS per byte of weights),
 // at 16 rows and fewer by the launch and drain of blocks that live for a few microseconds.
+// Four waves of two row tiles each (the same 128 rows a block, the activations' fragments
+// read half as often) were slower than eight waves of one at 40 to 64 rows on every
+// projection shape of an 8B model (down at 64 rows 27.4 us against 24.2, gated 52.4 against
+// 46.0): one wave a SIMD hides too little of the LDS round trips.
 //
 // RowScale (up to 16 rows): the activations may be given as bf16(x * gamma) of an RMSNorm whose
 // row statistics are not applied yet (what the product that adds into the residual stream
