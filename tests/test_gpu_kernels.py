@@ -461,6 +461,26 @@ def test_float32_product_is_true_32_bit_and_row_independent():
     assert torch.equal(whole[41:42], one)
 
 
+@pytest.mark.parametrize("M, N, K", [(1, 64, 64), (3, 331, 200), (8, 1000, 4096), (16, 77, 1028), (17, 130, 516),
+                                     (40, 200, 260), (64, 65, 12), (5, 70000, 264)])
+def test_float32_product_of_few_rows_equals_the_tiled_one_bit_for_bit(M, N, K):
+    """Up to 64 rows the float32 product streams the weights (a lane a weight row, a wave a
+    piece of K or all of them); it sums in the tiled kernel's order, so the same rows inside
+    a batch of 100 (the tiled kernel) give the same bits, with and without the split."""
+    from tokamak_amd.kernels import ops
+
+    x = rand(100, K, seed=1)
+    w = rand(N, K, seed=2, scale=K ** -0.5)
+    whole = torch.empty(100, N, device=DEV)
+    ops.gemm_tiled(x.to(DEV), w.to(DEV), whole)
+    torch.testing.assert_close(whole.cpu().double(), x.double() @ w.double().T, rtol=1e-5, atol=1e-5)
+    for at in (0, 100 - M):
+        for split in (None, False, True):
+            out = torch.full((M, N), float("nan"), device=DEV)
+            ops.gemm_tiled(x[at:at + M].to(DEV), w.to(DEV), out, fewrows_split=split)
+            assert torch.equal(out, whole[at:at + M]), (at, split)
+
+
 @pytest.mark.parametrize("M, N, K", [(1, 64, 64), (8, 6144, 4096), (64, 4096, 4096), (33, 331, 200), (17, 4096, 12288), (64, 1000, 264)])
 def test_streaming_product_and_its_partial_sums(M, N, K):
     """The LDS-staged weight-streaming kernel, unsplit and split over K: the

@@ -80,6 +80,14 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Orders one wave's LDS accesses (a wave's LDS instructions execute in order; this
+// keeps the compiler from moving them across the point).
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));

@@ -251,14 +251,6 @@ TK_API int tk_rope_tables(const int* positions, const float* inv_freq, float* co
 constexpr int kMaxHeadDim = 512;
 constexpr int kPairsPerBlock = 4;  // (token, head) pairs per block, one per wave
 
-// Orders one wave's LDS accesses (a wave's LDS instructions execute in order; this
-// keeps the compiler from moving them across the point).
-__device__ __forceinline__ void wave_lds_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 template <typename T, typename TIN>
 __global__ void qknorm_rope_store_kernel(
     const TIN* __restrict__ qkv, int parts, long part_stride, const float* __restrict__ q_weight,

@@ -82,6 +82,95 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const TI* __restrict__ 
   }
 }
 
+// Few rows (M <= 16, float32): the tiles above leave most of a block idle and read the weights
+// in pieces of 64 bytes.  Here a lane owns one weight row and walks it with 16-byte loads, a
+// cache line in eight loads one after the other; the activations are the same for every lane
+// (the compiler reads them through the scalar path).  The order of the sum is the one of the
+// tiled kernel, bit for bit: k ascending within a piece of kPiece, the pieces' sums added to the
+// total one after the other; so a row's result is still the same whatever the batch holds.
+// With `partial` a wave sums one piece only and writes it to partial[piece][M][N]; the second
+// kernel adds the pieces in order (for matrices of too few rows to fill the GPU otherwise).
+template <int MT>
+__global__ __launch_bounds__(64) void gemm_fewrows_kernel(const float* __restrict__ A,
+                                                          const float* __restrict__ W,
+                                                          float* __restrict__ C, float* __restrict__ partial,
+                                                          int M, int N, int K, long lda, long ldw, long ldc) {
+  const int lane = threadIdx.x;
+  const int n = blockIdx.x * 64 + lane;
+  const float* wrow = W + (size_t)min(n, N - 1) * ldw;
+  const int pieces = (K + kPiece - 1) / kPiece;
+  const int p_begin = partial ? blockIdx.y : 0;
+  const int p_end = partial ? p_begin + 1 : pieces;
+  float total[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) total[m] = 0.f;
+  for (int p = p_begin; p < p_end; ++p) {
+    float acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m] = 0.f;
+    const int k_end = min(K, (p + 1) * kPiece);
+#pragma unroll 8
+    for (int k = p * kPiece; k < k_end; k += 4) {
+      const float4 w = *reinterpret_cast<const float4*>(wrow + k);
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const float4 a = *reinterpret_cast<const float4*>(A + (size_t)min(m, M - 1) * lda + k);
+        acc[m] = fmaf(a.x, w.x, acc[m]);
+        acc[m] = fmaf(a.y, w.y, acc[m]);
+        acc[m] = fmaf(a.z, w.z, acc[m]);
+        acc[m] = fmaf(a.w, w.w, acc[m]);
+      }
+    }
+    if (partial) {
+      if (n < N) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+          if (m < M) partial[((size_t)p * M + m) * N + n] = acc[m];
+      }
+      return;
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) total[m] += acc[m];
+  }
+  if (n < N) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+      if (m < M) C[(size_t)m * ldc + n] = total[m];
+  }
+}
+
+__global__ __launch_bounds__(256) void gemm_fewrows_add_kernel(const float* __restrict__ partial,
+                                                               float* __restrict__ C, int M, int N,
+                                                               int pieces, long ldc) {
+  const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+  if (n >= N) return;
+  float total = 0.f;
+  for (int p = 0; p < pieces; ++p) total += partial[((size_t)p * M + m) * N + n];
+  C[(size_t)m * ldc + n] = total;
+}
+
+// float32 in and out, M <= 16, K and the row strides multiples of 4, 16-byte aligned rows.
+// partial: null, or room for ceil(K / 256) * M * N floats: then every piece of K has a wave of its own.
+TK_API int tk_gemm_fewrows(const float* A, const float* W, float* C, float* partial, int M, int N, int K,
+                           long lda, long ldw, long ldc, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 16 || K < 4 || K % 4 != 0 || lda % 4 != 0 || ldw % 4 != 0) return -1;
+  if (reinterpret_cast<uintptr_t>(A) % 16 != 0 || reinterpret_cast<uintptr_t>(W) % 16 != 0) return -1;
+  const int pieces = (K + kPiece - 1) / kPiece;
+  if (pieces > 65535) return -1;
+  dim3 grid((N + 63) / 64, partial ? pieces : 1);
+#define TK_FEW(MT_) gemm_fewrows_kernel<MT_><<<grid, 64, 0, stream>>>(A, W, C, partial, M, N, K, lda, ldw, ldc)
+  if (M == 1) TK_FEW(1);
+  else if (M == 2) TK_FEW(2);
+  else if (M <= 4) TK_FEW(4);
+  else if (M <= 8) TK_FEW(8);
+  else TK_FEW(16);
+#undef TK_FEW
+  if (partial)
+    gemm_fewrows_add_kernel<<<dim3((N + 255) / 256, M), 256, 0, stream>>>(partial, C, M, N, pieces, ldc);
+  return launch_status();
+}
+
 // in_dtype / out_dtype: 0 = float32, 1 = bfloat16
 TK_API int tk_gemm_tiled(int in_dtype, int out_dtype, const void* A, const void* W, void* C, int M,
                          int N, int K, long lda, long ldw, long ldc, hipStream_t stream) {

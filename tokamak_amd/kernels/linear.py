@@ -1,7 +1,7 @@
 """y = x @ W^T for the projections of a step.
 
-float32: the hand-written tiled kernel (true 32-bit multiply-add, row-wise
-deterministic).  bfloat16: hand-written MFMA kernels for up to 64 rows, else
+float32: hand-written kernels with true 32-bit multiply-add and one summation order
+(tiled, or weight-streaming for up to 64 rows; row-wise deterministic, equal bits).  bfloat16: hand-written MFMA kernels for up to 64 rows, else
 the library product that torch binds (as the reference's nn.Linear does).
 
 Decode steps of few rows (bfloat16, up to 16) can do without the kernels between the

@@ -142,6 +142,8 @@ _SIGS = {
     "gemm_tiled": {
         "tk_gemm_tiled": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long,
                           c_long, c_long, c_void_p],
+        "tk_gemm_fewrows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
+                            c_long, c_void_p],
     },
     "gemm_mfma": {
         "tk_gemm_stream": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long,
@@ -387,8 +389,15 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
                                              _stream()), "silu_mul")
 
 
-def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
-    """out[M, N] = a[M, K] @ w[N, K]^T, float32 multiply-add (rows may be strided)."""
+FEWROWS_MAX_ROWS = 64          # float32 products of up to this many rows stream the weights, a lane a weight row,
+FEWROWS_GROUP = 16             # this many rows a pass over the weights
+FEWROWS_SPLIT_BELOW = 65536    # weight rows below which every piece of 256 k gets a wave of its own
+
+
+def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, fewrows_split: bool | None = None) -> None:
+    """out[M, N] = a[M, K] @ w[N, K]^T, float32 multiply-add (rows may be strided).  float32
+    operands of up to 64 rows go to the weight-streaming kernel, which gives the same bits
+    (``fewrows_split``: a wave per piece of K or not; None chooses by the matrix's rows)."""
     for t in (a, w, out):
         _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
     m, k = a.shape
@@ -397,6 +406,19 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     _need(a.dtype == w.dtype, "gemm inputs must share a dtype")
     _need(m <= 64 * 65535, "too many rows for one launch")
     _note(f"{m}x{n}x{k}", (n * k + m * k) * a.element_size() + m * n * out.element_size(), 2.0 * m * n * k)
+    if (m <= FEWROWS_MAX_ROWS and a.dtype == torch.float32 and out.dtype == torch.float32 and k % 4 == 0 and k >= 4
+            and a.stride(0) % 4 == 0 and w.stride(0) % 4 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        # the same sums in the same order, by a kernel that streams the weights; a wave for every
+        # piece of K where the matrix has too few rows to fill the GPU with a wave per 64 of them
+        pieces = -(-k // 256)
+        split = fewrows_split if fewrows_split is not None else (n < FEWROWS_SPLIT_BELOW and pieces > 1)
+        for at in range(0, m, FEWROWS_GROUP):
+            rows = min(FEWROWS_GROUP, m - at)
+            partial = torch.empty((pieces, rows, n), dtype=torch.float32, device=a.device) if split else None
+            _check(_fn("gemm_tiled", "tk_gemm_fewrows")(_p(a[at:]), _p(w), _p(out[at:]), _p(partial),
+                                                        rows, n, k, a.stride(0), w.stride(0), out.stride(0), _stream()),
+                   "gemm_fewrows")
+        return
     _check(_fn("gemm_tiled", "tk_gemm_tiled")(_code(a.dtype), _code(out.dtype), _p(a), _p(w), _p(out),
                                               m, n, k, a.stride(0), w.stride(0), out.stride(0),
                                               _stream()), "gemm_tiled")
