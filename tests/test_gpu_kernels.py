@@ -239,6 +239,22 @@ def test_window_edge(dtype):
             assert g[-1].abs().max() < 50
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("nh, nkv, hd, ps, window", [(4, 2, 16, 8, None), (5, 5, 48, 16, None), (6, 2, 256, 16, None),
+                                                      (8, 2, 128, 16, 37), (3, 1, 80, 32, 70), (2, 1, 512, 8, None)])
+def test_generic_attention_gives_equal_bits_for_tokens_alone_and_in_tiles(dtype, nh, nkv, hd, ps, window):
+    """The generic kernel takes the tokens of a prompt portion in tiles that share the keys
+    and values they load; a token's result is the same bit for bit as when it runs alone
+    (rounds of 64 keys go to waves by their place in the context, sums keep their order),
+    with a window too, whose first key differs from token to token of a tile."""
+    requests = [(0, 70), (130, 21), (64, 1), (5, 16), (300, 1), (63, 2)]
+    tiled, want = run_attention(dtype, nh, nkv, hd, ps, requests, window=window, seed=11)
+    alone, _ = run_attention(dtype, nh, nkv, hd, ps, requests, window=window, seed=11, force_generic=True)
+    for a, b, w in zip(tiled, alone, want):
+        torch.testing.assert_close(a, w, **TOL[dtype])
+        assert torch.equal(a, b)
+
+
 def test_unsupported_sizes_are_refused_not_wrong():
     from tokamak_amd.kernels import ops
 

@@ -4,12 +4,15 @@
 // and decode tokens alike: every query token walks its own request's block table
 // from the first visible position to its own position.
 //
-// One block of kWaves waves per (token, query head).  Keys are taken 64 at a time, one
-// key per lane; round i of a token's keys goes to wave i % kWaves, which keeps a running
-// maximum, a running sum and an output of its own in float32 (online softmax); at the end
-// the waves' results are merged in wave order.  Which wave takes which keys follows from
-// the token's own position alone, so the result does not depend on how the request was
-// cut into steps or what else is in the batch.
+// One block of kWaves waves per (item, query head); an item is one token, or up to QT
+// consecutive tokens of one request (a piece of a 16-token tile of a prompt portion), which
+// then share every key and value they load.  Keys are taken 64 at a time, one key per lane;
+// the round that starts at key 64 i goes to wave i % kWaves, which keeps a running maximum,
+// a running sum and an output of its own in float32 for every query (online softmax); at
+// the end the waves' results are merged in wave order.  Which wave takes which keys, and
+// the order of every sum, follow from the query's own position alone: the result does not
+// depend on how the request was cut into steps, on what else is in the batch, or on
+// whether the token ran alone or in a tile (equal bits).
 //
 // Cache pages: K [nkv][hd/8][ps][8], V [nkv][hd/16][ps/4][16][4] (see elementwise.hip).
 #include "common.h"
@@ -17,124 +20,220 @@
 using namespace tk;
 
 constexpr int kMaxHd = 512;
-constexpr int kAccPerLane = kMaxHd / kWave;
 constexpr int kWaves = 8;  // waves of a block; kWaves * 64 threads cover every dimension of the widest head
 static_assert(kWaves * kWave >= kMaxHd, "the merge gives every dimension a thread");
+constexpr int kTileTokens = 16;  // tokens of a tile in the work list
+constexpr int kQueries = 8;      // queries a block of the tile kernel takes
 
-template <typename T>
+struct GenericItems {
+  const int* single;      // token rows that run alone (null: every token of the step does)
+  const int* tile_first;  // first token row of each tile
+  const int* tile_count;  // tokens in it (1..kTileTokens), consecutive positions of one request
+};
+
+// QT: queries of a block.  SLOTS: dimensions a lane owns (hd <= 64 * SLOTS).
+template <typename T, int QT, int SLOTS>
 __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, const int* __restrict__ positions,
-    const int* __restrict__ req_of_token, T* __restrict__ out, int nh, int nkv, int hd, int ps,
-    int max_pages, float scale, int window) {
-  __shared__ float q_s[kMaxHd];
-  __shared__ float p_s[kWaves][kWave];
+    const int* __restrict__ req_of_token, GenericItems items, T* __restrict__ out, int nh, int nkv,
+    int hd, int ps, int max_pages, float scale, int window) {
+  __shared__ __attribute__((aligned(16))) float q_s[QT][kMaxHd];
+  __shared__ __attribute__((aligned(16))) float p_s[kWaves][kWave][QT];
   __shared__ long base_s[kWaves][kWave];
   __shared__ float m_s[kWaves], l_s[kWaves];
   __shared__ float acc_s[kWaves][kMaxHd];
 
-  const int n = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+  const int head = blockIdx.y, tid = threadIdx.x;
   const int lane = tid & (kWave - 1), wave = tid / kWave;
+  int n0, cnt;
+  if (QT == 1) {
+    n0 = items.single ? items.single[blockIdx.x] : (int)blockIdx.x;
+    cnt = 1;
+  } else {
+    n0 = items.tile_first[blockIdx.x] + blockIdx.z * QT;
+    cnt = min(QT, items.tile_count[blockIdx.x] - (int)blockIdx.z * QT);
+    if (cnt <= 0) return;
+  }
   const int kvh = head / (nh / nkv);
-  const int pos = positions[n];
-  const int* table = block_tables + (size_t)req_of_token[n] * max_pages;
-  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
+  int pos[QT], first[QT];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    pos[t] = positions[n0 + min(t, cnt - 1)];
+    first[t] = (window > 0 && pos[t] - window + 1 > 0) ? pos[t] - window + 1 : 0;
+  }
+  const int lo = first[0], hi = pos[QT - 1];  // positions ascend within an item
   const size_t page_elems = (size_t)nkv * hd * ps;
   const size_t head_off = (size_t)kvh * hd * ps;
 
-  const T* qrow = q + ((size_t)n * nh + head) * hd;
-  for (int d = tid; d < hd; d += kWaves * kWave) q_s[d] = Elem<T>::load(qrow + d) * scale;
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const T* qrow = q + ((size_t)(n0 + min(t, cnt - 1)) * nh + head) * hd;
+    for (int d = tid; d < hd; d += kWaves * kWave) q_s[t][d] = Elem<T>::load(qrow + d) * scale;
+  }
   __syncthreads();
 
-  float m = -INFINITY, l = 0.f;
-  float acc[kAccPerLane];
+  float m[QT], l[QT], acc[SLOTS][QT];
 #pragma unroll
-  for (int i = 0; i < kAccPerLane; ++i) acc[i] = 0.f;
+  for (int t = 0; t < QT; ++t) {
+    m[t] = -INFINITY;
+    l[t] = 0.f;
+#pragma unroll
+    for (int i = 0; i < SLOTS; ++i) acc[i][t] = 0.f;
+  }
 
-  // this wave's rounds of 64 keys; every round starts at or before the token's own position
-  // and, but for the first, at or after the first visible one: none is empty
-  for (int c0 = (first / kWave + wave) * kWave; c0 <= pos; c0 += kWaves * kWave) {
-    const int c = c0 + lane;
-    const bool valid = c >= first && c <= pos;
-    float s = -INFINITY;
+  // this wave's rounds: those whose index is wave modulo kWaves, from the one that holds lo
+  const int round0 = lo / kWave;
+  for (int rd = round0 + (wave - round0 % kWaves + kWaves) % kWaves; rd * kWave <= hi; rd += kWaves) {
+    const int c0 = rd * kWave, c = c0 + lane;
+    const bool loaded = c >= lo && c <= hi;
+    float dot[QT];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) dot[t] = 0.f;
     long vbase = -1;
-    if (valid) {
+    if (loaded) {
       const int page = table[c / ps];
       const int off = c % ps;
       const T* kp = k_cache + (size_t)page * page_elems + head_off;
-      float dot = 0.f;
       for (int j = 0; j < hd / 8; ++j) {
         const T* kk = kp + ((size_t)j * ps + off) * 8;
+        float k8[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) dot = fmaf(q_s[j * 8 + e], Elem<T>::load(kk + e), dot);
+        for (int e = 0; e < 8; ++e) k8[e] = Elem<T>::load(kk + e);
+#pragma unroll
+        for (int t = 0; t < QT; ++t) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dot[t] = fmaf(q_s[t][j * 8 + e], k8[e], dot[t]);
+        }
       }
-      s = dot;
       vbase = (long)((size_t)page * page_elems + head_off + (size_t)(off >> 2) * 64 + (off & 3));
     }
-    const float m_new = fmaxf(m, wave_max(s));
-    const float p = valid ? expf(s - m_new) : 0.f;
-    const float alpha = expf(m - m_new);  // m = -inf on the first round: alpha = 0
-    l = l * alpha + wave_sum(p);
-    m = m_new;
+    float alpha[QT], p[QT];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+      // a round that holds none of query t's keys leaves its sums as they are
+      const bool takes = c0 <= pos[t] && c0 + kWave - 1 >= first[t];
+      alpha[t] = 1.f;
+      p[t] = 0.f;
+      if (takes) {
+        const bool valid = c >= first[t] && c <= pos[t];
+        const float sc = valid ? dot[t] : -INFINITY;
+        const float m_new = fmaxf(m[t], wave_max(sc));
+        p[t] = valid ? expf(sc - m_new) : 0.f;
+        alpha[t] = expf(m[t] - m_new);  // m = -inf on the first round: alpha = 0
+        l[t] = l[t] * alpha[t] + wave_sum(p[t]);
+        m[t] = m_new;
+      }
+    }
     wave_lds_sync();   // the wave has read its last round's probabilities
-    p_s[wave][lane] = p;
+#pragma unroll
+    for (int t = 0; t < QT; ++t) p_s[wave][lane][t] = p[t];
     base_s[wave][lane] = vbase;
     wave_lds_sync();
-    const int count = (pos - c0 + 1 < kWave) ? pos - c0 + 1 : kWave;
+    const int count = (hi - c0 + 1 < kWave) ? hi - c0 + 1 : kWave;
 #pragma unroll
-    for (int i = 0; i < kAccPerLane; ++i) {
+    for (int i = 0; i < SLOTS; ++i) {
       const int d = lane + i * kWave;
       if (d < hd) {
         const size_t v_dim_off = (size_t)(d >> 4) * (ps >> 2) * 64 + (d & 15) * 4;
-        float a = acc[i] * alpha;
-        for (int t = 0; t < count; ++t) {
-          const long b = base_s[wave][t];
-          if (b >= 0) a = fmaf(p_s[wave][t], Elem<T>::load(v_cache + b + v_dim_off), a);
+        float a[QT];
+#pragma unroll
+        for (int t = 0; t < QT; ++t) a[t] = acc[i][t] * alpha[t];
+        for (int key = 0; key < count; ++key) {
+          const long b = base_s[wave][key];
+          if (b >= 0) {
+            const float v = Elem<T>::load(v_cache + b + v_dim_off);
+#pragma unroll
+            for (int t = 0; t < QT; ++t) a[t] = fmaf(p_s[wave][key][t], v, a[t]);
+          }
         }
-        acc[i] = a;
+#pragma unroll
+        for (int t = 0; t < QT; ++t) acc[i][t] = a[t];
       }
     }
   }
-  // merge: a wave that had no round brings m = -inf, l = 0 and zeros, which weigh nothing
-  if (lane == 0) {
-    m_s[wave] = m;
-    l_s[wave] = l;
-  }
+  // merge, one query after the other: a wave that had no round of the query's brings
+  // m = -inf, l = 0 and zeros, which weigh nothing
 #pragma unroll
-  for (int i = 0; i < kAccPerLane; ++i) {
-    const int d = lane + i * kWave;
-    if (d < hd) acc_s[wave][d] = acc[i];
-  }
-  __syncthreads();
-  if (tid >= hd) return;
-  float top = m_s[0];   // wave 0 always has the first round
+  for (int t = 0; t < QT; ++t) {
+    if (t >= cnt) break;
+    __syncthreads();   // the last query's merge has read the waves' results
+    if (lane == 0) {
+      m_s[wave] = m[t];
+      l_s[wave] = l[t];
+    }
 #pragma unroll
-  for (int w = 1; w < kWaves; ++w) top = fmaxf(top, m_s[w]);
-  float sum = 0.f, o = 0.f;
+    for (int i = 0; i < SLOTS; ++i) {
+      const int d = lane + i * kWave;
+      if (d < hd) acc_s[wave][d] = acc[i][t];
+    }
+    __syncthreads();
+    if (tid < hd) {
+      float top = m_s[0];
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) {
-    const float e = expf(m_s[w] - top);
-    sum = fmaf(l_s[w], e, sum);
-    o = fmaf(acc_s[w][tid], e, o);
+      for (int w = 1; w < kWaves; ++w) top = fmaxf(top, m_s[w]);
+      float sum = 0.f, o = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        const float e = expf(m_s[w] - top);
+        sum = fmaf(l_s[w], e, sum);
+        o = fmaf(acc_s[w][tid], e, o);
+      }
+      Elem<T>::store(out + ((size_t)(n0 + t) * nh + head) * hd + tid, o / sum);
+    }
   }
-  Elem<T>::store(out + ((size_t)n * nh + head) * hd + tid, o / sum);
 }
 
+template <typename T, int SLOTS>
+static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const int* block_tables,
+                           const int* positions, const int* req_of_token, GenericItems items,
+                           int num_single, int num_tiles, T* out, int nh, int nkv, int hd, int ps,
+                           int max_pages, float scale, int window, hipStream_t stream) {
+  if (num_single > 0)
+    paged_attention_generic_kernel<T, 1, SLOTS><<<dim3(num_single, nh), kWaves * kWave, 0, stream>>>(
+        q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, ps,
+        max_pages, scale, window);
+  if (num_tiles > 0)
+    paged_attention_generic_kernel<T, kQueries, SLOTS>
+        <<<dim3(num_tiles, nh, kTileTokens / kQueries), kWaves * kWave, 0, stream>>>(
+            q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, ps,
+            max_pages, scale, window);
+}
+
+// tile_first / tile_count (num_tiles of them) and single (num_single token rows): the step's work
+// lists, which together name every token once.  With tile_first null every one of the N tokens
+// runs alone.
 TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_cache,
                                       const void* v_cache, const int* block_tables,
                                       const int* positions, const int* req_of_token, void* out,
                                       int N, int nh, int nkv, int hd, int ps, int max_pages,
-                                      float scale, int window, hipStream_t stream) {
+                                      float scale, int window, const int* tile_first,
+                                      const int* tile_count, int num_tiles, const int* single,
+                                      int num_single, hipStream_t stream) {
   if (N <= 0) return 0;
   if (hd > kMaxHd || hd % 16 != 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || ps % 4 != 0 || nh > 65535) return -1;
-  dim3 grid(N, nh);
-  if (dtype == 0)
-    paged_attention_generic_kernel<float><<<grid, kWaves * kWave, 0, stream>>>(
-        (const float*)q, (const float*)k_cache, (const float*)v_cache, block_tables, positions,
-        req_of_token, (float*)out, nh, nkv, hd, ps, max_pages, scale, window);
-  else
-    paged_attention_generic_kernel<bf16_t><<<grid, kWaves * kWave, 0, stream>>>(
-        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, positions,
-        req_of_token, (bf16_t*)out, nh, nkv, hd, ps, max_pages, scale, window);
+  if (tile_first == nullptr) {
+    num_tiles = 0;
+    single = nullptr;
+    num_single = N;
+  } else if (num_tiles < 0 || num_single < 0 || tile_count == nullptr || (num_single > 0 && single == nullptr)) {
+    return -1;
+  }
+  const GenericItems items{single, tile_first, tile_count};
+#define TK_GENERIC(T_, SLOTS_)                                                                      \
+  launch_generic<T_, SLOTS_>((const T_*)q, (const T_*)k_cache, (const T_*)v_cache, block_tables,    \
+                             positions, req_of_token, items, num_single, num_tiles, (T_*)out, nh,   \
+                             nkv, hd, ps, max_pages, scale, window, stream)
+  if (dtype == 0) {
+    if (hd <= 128) TK_GENERIC(float, 2);
+    else if (hd <= 256) TK_GENERIC(float, 4);
+    else TK_GENERIC(float, 8);
+  } else {
+    if (hd <= 128) TK_GENERIC(bf16_t, 2);
+    else if (hd <= 256) TK_GENERIC(bf16_t, 4);
+    else TK_GENERIC(bf16_t, 8);
+  }
+#undef TK_GENERIC
   return launch_status();
 }

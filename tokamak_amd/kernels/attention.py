@@ -141,4 +141,5 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     ops.paged_attention_generic(
         q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
         num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
-        scale=scale, window=window)
+        scale=scale, window=window,
+        tiles=(batch.tile_first, batch.tile_count, batch.num_tiles, batch.decode_tokens, batch.num_decode))

@@ -167,7 +167,7 @@ _SIGS = {
     "attention_generic": {
         "tk_paged_attention_generic": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                       c_float, c_int, c_void_p],
+                                       c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p],
     },
     "attention_mfma": {
         "tk_attention_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
@@ -663,8 +663,12 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             block_tables: torch.Tensor, positions: torch.Tensor,
                             req_of_token: torch.Tensor, out: torch.Tensor, *, num_heads: int,
                             num_kv_heads: int, head_dim: int, page_size: int, scale: float,
-                            window: int | None = None) -> None:
-    """Causal attention of each query token over its request's pages."""
+                            window: int | None = None, tiles: tuple | None = None) -> None:
+    """Causal attention of each query token over its request's pages.  ``tiles``:
+    (tile_first, tile_count, num_tiles, single_tokens, num_single), the step's work lists (tiles
+    of up to 16 consecutive tokens of one request, and token rows that run alone), which together
+    name every token once; tokens of a tile share the keys and values they load.  Without it every
+    token runs alone; the result is the same bit for bit."""
     _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, out)
     n = positions.numel()
     _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "attention tensors must share a dtype")
@@ -675,10 +679,20 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _need(k_cache.numel() % page_elems == 0 and v_cache.numel() == k_cache.numel(), "cache size is not whole pages")
     _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32
           and block_tables.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
+    tile_first = tile_count = single = None
+    num_tiles = num_single = 0
+    if tiles is not None and tiles[2] > 0:
+        tile_first, tile_count, num_tiles, single, num_single = tiles
+        _gpu(tile_first, tile_count)
+        _need(tile_first.dtype == torch.int32 and tile_count.dtype == torch.int32
+              and tile_first.numel() >= num_tiles and tile_count.numel() >= num_tiles, "bad tile list")
+        _need(num_single == 0 or (single is not None and single.is_cuda and single.dtype == torch.int32
+                                  and single.numel() >= num_single), "bad list of single tokens")
     _check(_fn("attention_generic", "tk_paged_attention_generic")(
         _code(q.dtype), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(positions),
         _p(req_of_token), _p(out), n, num_heads, num_kv_heads, head_dim, page_size,
-        block_tables.shape[1], float(scale), int(window or 0), _stream()), "paged_attention_generic")
+        block_tables.shape[1], float(scale), int(window or 0), _p(tile_first), _p(tile_count), num_tiles,
+        _p(single), num_single, _stream()), "paged_attention_generic")
 
 
 NOT_INSTANTIATED = -2
