@@ -22,7 +22,7 @@ def rand(*shape, seed=0, scale=1.0):
 # attention
 # ---------------------------------------------------------------------------
 def run_attention(dtype, nh, nkv, hd, ps, requests, *, window=None, poison=True, force_generic=False,
-                  seed=0, boost=None):
+                  seed=0, boost=None, share_heads=None):
     """requests: list of (ctx_len, q_len).  Builds scattered tables, fills pages,
     runs the dispatcher (or the generic kernel) and returns (got, want) lists."""
     from tokamak_amd.kernels import ops
@@ -56,7 +56,7 @@ def run_attention(dtype, nh, nkv, hd, ps, requests, *, window=None, poison=True,
     if force_generic:
         ops.paged_attention_generic(q_all, kc, vc, batch.block_tables[0], batch.positions, batch.req_of_token,
                                     out, num_heads=nh, num_kv_heads=nkv, head_dim=hd, page_size=ps,
-                                    scale=scale, window=window)
+                                    scale=scale, window=window, share_heads=share_heads)
     else:
         paged_attention(q_all, kc, vc, batch.block_tables[0], batch, out, num_heads=nh, num_kv_heads=nkv,
                         head_dim=hd, page_size=ps, scale=scale, window=window)
@@ -251,6 +251,19 @@ def test_generic_attention_gives_equal_bits_for_tokens_alone_and_in_tiles(dtype,
     tiled, want = run_attention(dtype, nh, nkv, hd, ps, requests, window=window, seed=11)
     alone, _ = run_attention(dtype, nh, nkv, hd, ps, requests, window=window, seed=11, force_generic=True)
     for a, b, w in zip(tiled, alone, want):
+        torch.testing.assert_close(a, w, **TOL[dtype])
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("nh, nkv, hd", [(6, 2, 48), (16, 2, 80), (4, 4, 32)])
+def test_generic_attention_gives_equal_bits_whether_heads_share_a_block_or_not(dtype, nh, nkv, hd):
+    """With many single tokens the query heads of a group share a block and the keys it loads;
+    with few every head has a block of its own.  Both give the same bits."""
+    requests = [(3 + 37 * i, 1) for i in range(12)] + [(0, 5), (70, 3)]
+    many, want = run_attention(dtype, nh, nkv, hd, 16, requests, seed=13, force_generic=True, share_heads=True)
+    few, _ = run_attention(dtype, nh, nkv, hd, 16, requests, seed=13, force_generic=True, share_heads=False)
+    for a, b, w in zip(many, few, want):
         torch.testing.assert_close(a, w, **TOL[dtype])
         assert torch.equal(a, b)
 

@@ -4,9 +4,10 @@
 // and decode tokens alike: every query token walks its own request's block table
 // from the first visible position to its own position.
 //
-// One block of kWaves waves per (item, query head); an item is one token, or up to QT
-// consecutive tokens of one request (a piece of a 16-token tile of a prompt portion), which
-// then share every key and value they load.  Keys are taken 64 at a time, one key per lane;
+// A block of kWaves waves takes up to QT queries that walk the same keys and values and
+// share every one they load: consecutive tokens of one request at one query head (a piece
+// of a 16-token tile of a prompt portion), or the query heads of one kv head's group at one
+// token (a token that runs alone, a decode token).  Keys are taken 64 at a time, one key per lane;
 // the round that starts at key 64 i goes to wave i % kWaves, which keeps a running maximum,
 // a running sum and an output of its own in float32 for every query (online softmax); at
 // the end the waves' results are merged in wave order.  Which wave takes which keys, and
@@ -31,8 +32,10 @@ struct GenericItems {
   const int* tile_count;  // tokens in it (1..kTileTokens), consecutive positions of one request
 };
 
-// QT: queries of a block.  SLOTS: dimensions a lane owns (hd <= 64 * SLOTS).
-template <typename T, int QT, int SLOTS>
+// QT: queries of a block; HEADS: they are heads of one group at one token (blockIdx.y is the kv
+// head, blockIdx.z the piece of the group), else tokens of one tile at one head (blockIdx.y).
+// SLOTS: dimensions a lane owns (hd <= 64 * SLOTS).
+template <typename T, int QT, bool HEADS, int SLOTS>
 __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, const int* __restrict__ positions,
@@ -44,32 +47,40 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
   __shared__ float m_s[kWaves], l_s[kWaves];
   __shared__ float acc_s[kWaves][kMaxHd];
 
-  const int head = blockIdx.y, tid = threadIdx.x;
+  const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1), wave = tid / kWave;
-  int n0, cnt;
-  if (QT == 1) {
+  const int group = nh / nkv;
+  int n0, cnt, head0, kvh;
+  if (HEADS) {
     n0 = items.single ? items.single[blockIdx.x] : (int)blockIdx.x;
-    cnt = 1;
+    kvh = blockIdx.y;
+    head0 = kvh * group + blockIdx.z * QT;
+    cnt = min(QT, group - (int)blockIdx.z * QT);
   } else {
     n0 = items.tile_first[blockIdx.x] + blockIdx.z * QT;
     cnt = min(QT, items.tile_count[blockIdx.x] - (int)blockIdx.z * QT);
-    if (cnt <= 0) return;
+    head0 = blockIdx.y;
+    kvh = head0 / group;
   }
-  const int kvh = head / (nh / nkv);
+  if (cnt <= 0) return;
   const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
+  // query t: its row of q and out, its position and the first key it sees
+  size_t row[QT];
   int pos[QT], first[QT];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    pos[t] = positions[n0 + min(t, cnt - 1)];
+    const int u = min(t, cnt - 1);
+    row[t] = HEADS ? (size_t)n0 * nh + head0 + u : (size_t)(n0 + u) * nh + head0;
+    pos[t] = positions[HEADS ? n0 : n0 + u];
     first[t] = (window > 0 && pos[t] - window + 1 > 0) ? pos[t] - window + 1 : 0;
   }
-  const int lo = first[0], hi = pos[QT - 1];  // positions ascend within an item
+  const int lo = first[0], hi = pos[QT - 1];  // positions ascend within a tile
   const size_t page_elems = (size_t)nkv * hd * ps;
   const size_t head_off = (size_t)kvh * hd * ps;
 
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
-    const T* qrow = q + ((size_t)(n0 + min(t, cnt - 1)) * nh + head) * hd;
+    const T* qrow = q + row[t] * hd;
     for (int d = tid; d < hd; d += kWaves * kWave) q_s[t][d] = Elem<T>::load(qrow + d) * scale;
   }
   __syncthreads();
@@ -180,7 +191,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
         sum = fmaf(l_s[w], e, sum);
         o = fmaf(acc_s[w][tid], e, o);
       }
-      Elem<T>::store(out + ((size_t)(n0 + t) * nh + head) * hd + tid, o / sum);
+      Elem<T>::store(out + row[t] * hd + tid, o / sum);
     }
   }
 }
@@ -189,13 +200,26 @@ template <typename T, int SLOTS>
 static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const int* block_tables,
                            const int* positions, const int* req_of_token, GenericItems items,
                            int num_single, int num_tiles, T* out, int nh, int nkv, int hd, int ps,
-                           int max_pages, float scale, int window, hipStream_t stream) {
-  if (num_single > 0)
-    paged_attention_generic_kernel<T, 1, SLOTS><<<dim3(num_single, nh), kWaves * kWave, 0, stream>>>(
-        q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, ps,
-        max_pages, scale, window);
+                           int max_pages, float scale, int window, int share_heads, hipStream_t stream) {
+  const int group = nh / nkv;
+#define TK_ALONE(QT_)                                                                               \
+  paged_attention_generic_kernel<T, QT_, true, SLOTS>                                               \
+      <<<dim3(num_single, nkv, (group + QT_ - 1) / QT_), kWaves * kWave, 0, stream>>>(              \
+          q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, ps,  \
+          max_pages, scale, window)
+  if (num_single > 0) {
+    // the heads of a group share a block if that still gives every CU one (the result is the
+    // same either way): at batch 64 of an 8B-shaped layer a third faster, at batch 8 slower
+    const int qt = group <= 4 ? 4 : kQueries;
+    const bool shared = group > 1 && (share_heads < 0 ? (long)num_single * nkv * ((group + qt - 1) / qt) >= 256
+                                                      : share_heads > 0);
+    if (!shared) TK_ALONE(1);
+    else if (qt == 4) TK_ALONE(4);
+    else TK_ALONE(kQueries);
+  }
+#undef TK_ALONE
   if (num_tiles > 0)
-    paged_attention_generic_kernel<T, kQueries, SLOTS>
+    paged_attention_generic_kernel<T, kQueries, false, SLOTS>
         <<<dim3(num_tiles, nh, kTileTokens / kQueries), kWaves * kWave, 0, stream>>>(
             q, k_cache, v_cache, block_tables, positions, req_of_token, items, out, nh, nkv, hd, ps,
             max_pages, scale, window);
@@ -203,14 +227,15 @@ static void launch_generic(const T* q, const T* k_cache, const T* v_cache, const
 
 // tile_first / tile_count (num_tiles of them) and single (num_single token rows): the step's work
 // lists, which together name every token once.  With tile_first null every one of the N tokens
-// runs alone.
+// runs alone.  share_heads: whether the query heads of a group share a block for the tokens
+// that run alone (1), or not (0), or as fills the GPU (-1); the result is the same.
 TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_cache,
                                       const void* v_cache, const int* block_tables,
                                       const int* positions, const int* req_of_token, void* out,
                                       int N, int nh, int nkv, int hd, int ps, int max_pages,
                                       float scale, int window, const int* tile_first,
                                       const int* tile_count, int num_tiles, const int* single,
-                                      int num_single, hipStream_t stream) {
+                                      int num_single, int share_heads, hipStream_t stream) {
   if (N <= 0) return 0;
   if (hd > kMaxHd || hd % 16 != 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || ps % 4 != 0 || nh > 65535) return -1;
   if (tile_first == nullptr) {
@@ -224,7 +249,7 @@ TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_ca
 #define TK_GENERIC(T_, SLOTS_)                                                                      \
   launch_generic<T_, SLOTS_>((const T_*)q, (const T_*)k_cache, (const T_*)v_cache, block_tables,    \
                              positions, req_of_token, items, num_single, num_tiles, (T_*)out, nh,   \
-                             nkv, hd, ps, max_pages, scale, window, stream)
+                             nkv, hd, ps, max_pages, scale, window, share_heads, stream)
   if (dtype == 0) {
     if (hd <= 128) TK_GENERIC(float, 2);
     else if (hd <= 256) TK_GENERIC(float, 4);

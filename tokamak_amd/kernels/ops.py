@@ -167,7 +167,7 @@ _SIGS = {
     "attention_generic": {
         "tk_paged_attention_generic": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                       c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p],
+                                       c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     },
     "attention_mfma": {
         "tk_attention_mfma": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
@@ -663,12 +663,15 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             block_tables: torch.Tensor, positions: torch.Tensor,
                             req_of_token: torch.Tensor, out: torch.Tensor, *, num_heads: int,
                             num_kv_heads: int, head_dim: int, page_size: int, scale: float,
-                            window: int | None = None, tiles: tuple | None = None) -> None:
+                            window: int | None = None, tiles: tuple | None = None,
+                            share_heads: bool | None = None) -> None:
     """Causal attention of each query token over its request's pages.  ``tiles``:
     (tile_first, tile_count, num_tiles, single_tokens, num_single), the step's work lists (tiles
     of up to 16 consecutive tokens of one request, and token rows that run alone), which together
     name every token once; tokens of a tile share the keys and values they load.  Without it every
-    token runs alone; the result is the same bit for bit."""
+    token runs alone; the result is the same bit for bit.  ``share_heads``: whether the query heads
+    of a group share a block (and the keys it loads) for the tokens that run alone; None chooses by
+    how many there are; the same bits again."""
     _gpu(q, k_cache, v_cache, block_tables, positions, req_of_token, out)
     n = positions.numel()
     _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "attention tensors must share a dtype")
@@ -692,7 +695,7 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         _code(q.dtype), _p(q), _p(k_cache), _p(v_cache), _p(block_tables), _p(positions),
         _p(req_of_token), _p(out), n, num_heads, num_kv_heads, head_dim, page_size,
         block_tables.shape[1], float(scale), int(window or 0), _p(tile_first), _p(tile_count), num_tiles,
-        _p(single), num_single, _stream()), "paged_attention_generic")
+        _p(single), num_single, -1 if share_heads is None else int(share_heads), _stream()), "paged_attention_generic")
 
 
 NOT_INSTANTIATED = -2
