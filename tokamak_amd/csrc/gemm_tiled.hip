@@ -1,8 +1,8 @@
 // C[M,N] = A[M,K] * W[N,K]^T with float32 multiply-add and float32 accumulation
 // for any M, N, K.  It is the true 32-bit matrix product of the float32 path
 // (no reduced-precision matrix mode), and also accepts bf16 inputs.  Every
-// output element is summed by one thread in one fixed order, so a row's result does
-// not depend on which other rows are in the batch: k ascending within pieces of
+// output element is summed in one fixed order, whichever kernel below does it, so a row's
+// result does not depend on which other rows are in the batch: k ascending within pieces of
 // kPiece, whose sums are added to the total one after the other.  The two levels
 // keep the rounding error of a sum over K terms near sqrt(kPiece) + sqrt(K / kPiece)
 // units instead of sqrt(K) (K is 25,600 in the widest feed-forward).
@@ -97,8 +97,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const TI* __restrict__ 
   }
 }
 
-// Few rows (M <= 16, float32): the tiles above leave most of a block idle.  Here a lane owns one weight row and walks it with 16-byte loads, a
-// cache line in eight loads one after the other; the activations are the same for every lane
+// Few rows (M <= 16, float32): the tiles above leave most of a block idle.  Here a lane owns
+// one weight row and walks it with 16-byte loads, a cache line in eight loads one after the other; the activations are the same for every lane
 // (the compiler reads them through the scalar path).  The order of the sum is the one of the
 // tiled kernel, bit for bit: k ascending within a piece of kPiece, the pieces' sums added to the
 // total one after the other; so a row's result is still the same whatever the batch holds.
