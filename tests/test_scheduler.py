@@ -311,3 +311,128 @@ def test_a_request_evicted_with_a_token_on_its_way_waits_until_it_is_read():
     assert b.tokens[-1] == 4 and b.unknown == 0 and len(b.tokens) == 9
     third = sched.plan()
     assert all(s.request is not b or s.feed is None for s in third.spans)
+
+
+# ---------------------------------------------------------------------------
+# the whole step loop one step ahead, as LLM.generate runs it, without a GPU
+# ---------------------------------------------------------------------------
+def ahead_loop(sched, manager, token_of, eos=(), context_limit=10 ** 6, in_turn=False):
+    """The step loop of the entry point: plan and launch step i+1, then read step i.
+    ``token_of(request, draw)`` is the sampler.  Returns the plans, in order."""
+    plans = []
+    in_flight = None
+
+    def read_back(step, tokens):
+        for span, token in zip([s for s in step.spans if s.samples], tokens):
+            request = span.request
+            if request.finished:
+                continue
+            if request.accept(token, eos_token_ids=tuple(eos), context_limit=context_limit):
+                manager.free(request.rid)
+
+    guard = 0
+    while sched.busy or in_flight is not None:
+        guard += 1
+        assert guard < 5000
+        plan = sched.plan() if sched.busy else None
+        launched = None
+        if plan is not None:
+            plans.append(plan)
+            for span in plan.spans:
+                request = span.request
+                assert not request.finished, f"a span was planned for finished request {request.rid}"
+                assert span.start == request.cached
+                assert len(manager.block_table(request.rid)) * manager.page_size >= span.start + span.length
+            ids = [s.request.rid for s in plan.spans]
+            assert len(set(ids)) == len(ids)
+            if plan.spans:
+                tokens = [token_of(s.request, s.request.num_drawn) for s in plan.spans if s.samples]
+                launch(plan)
+                launched = (plan, tokens) if tokens else None
+        if in_flight is not None:
+            read_back(*in_flight)
+        else:
+            assert plan is not None and plan.spans, "unfinished requests, but no step"
+        in_flight = launched
+        if in_flight is not None and in_turn:
+            read_back(*in_flight)
+            in_flight = None
+        manager.check()
+    return plans
+
+
+def test_a_request_that_ends_while_it_waits_is_never_planned_again():
+    # ten pages of eight tokens, three prompts of twenty; request 2 draws its EOS as its fifth
+    # token and is evicted while that token is on its way
+    EOS = 99
+    manager = CacheManager([CacheGroupSpec("full", (0,))], 10, 8, 3)
+    sched = Scheduler(manager, 3, 64)
+    requests = [Request.from_prompt(i, [1] * 20, SamplingParams(max_new_tokens=30)) for i in range(3)]
+    for r in requests:
+        sched.submit(r)
+
+    def token_of(request, draw):
+        return EOS if request.rid == 2 and draw == 4 else 7
+
+    plans = ahead_loop(sched, manager, token_of, eos=(EOS,))
+    assert any(requests[2] in p.evicted for p in plans)            # the case is the one meant
+    assert requests[2].finish_reason == FinishReason.STOP and requests[2].generated[-1] == EOS
+    assert len(requests[2].generated) == 5
+    assert all(r.finished for r in requests)
+    assert requests[0].num_generated == 30 and requests[1].num_generated == 30
+    assert manager.num_free_pages() == 10 and manager.slots.num_free == 3
+    assert not sched.waiting or all(r.finished for r in sched.waiting)
+
+
+def test_a_victim_that_ends_with_the_token_on_its_way_is_released_not_queued():
+    sched, manager = make(num_pages=4, page_size=4, max_batch=2, budget=16)
+    a, b = make_seq(0, prompt_len=8, max_new=8), make_seq(1, prompt_len=8, max_new=1)
+    sched.submit(a)
+    sched.submit(b)
+    first = sched.plan()
+    launch(first)                               # the pool is full; b's only token is on its way
+    assert b.closing
+    second = sched.plan()                       # a needs a third page: b gives its pages back ...
+    assert second.released == [b] and second.evicted == []
+    assert [s.request.rid for s in second.spans] == [0]
+    assert b not in sched.running and b not in sched.waiting and b.evictions == 0   # ... and is not queued
+    assert manager.block_table(1) == []
+    launch(second)
+    read(first, token=4)
+    assert b.finished and b.generated == [4]
+    manager.free(b.rid)                         # what the reader does; nothing is left to give back
+    manager.check()
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_workloads_one_step_ahead_with_stops(seed):
+    rng = random.Random(1000 + seed)
+    EOS = 5
+    pages = rng.randint(6, 14)
+    sched, manager = make(num_pages=pages, page_size=4, max_batch=rng.randint(1, 4), budget=16,
+                          chunk=rng.choice([None, 3, 7]))
+    limit = pages * 4
+    seqs = [make_seq(i, rng.randint(1, min(20, limit - 2)), rng.randint(1, 14)) for i in range(rng.randint(3, 12))]
+    for s in seqs:
+        sched.submit(s)
+        s.context_limit = min(limit, s.prompt_len + s.params.max_new_tokens)
+    draws = {}
+
+    def token_of(request, draw):
+        # a fixed token per (request, draw): the same under any schedule
+        return draws.setdefault((request.rid, draw), EOS if rng.random() < 0.12 else rng.randint(6, 50))
+
+    ahead_loop(sched, manager, token_of, eos=(EOS,), context_limit=limit)
+    assert all(s.finished for s in seqs)
+    assert manager.num_free_pages() == pages and manager.slots.num_free == manager.slots.num_slots
+    ahead = [list(s.generated) for s in seqs]
+
+    # the same requests read in turn give the same tokens
+    sched2, manager2 = make(num_pages=pages, page_size=4, max_batch=sched.max_batch_size, budget=16,
+                            chunk=None if sched.chunk == 16 else sched.chunk)
+    again = [make_seq(s.rid, s.prompt_len, s.params.max_new_tokens) for s in seqs]
+    for s in again:
+        sched2.submit(s)
+        s.context_limit = min(limit, s.prompt_len + s.params.max_new_tokens)
+    ahead_loop(sched2, manager2, token_of, eos=(EOS,), context_limit=limit, in_turn=True)
+    assert [list(s.generated) for s in again] == ahead

@@ -267,6 +267,8 @@ class LLM:
         for victim in plan.evicted:
             self.runner.forget(victim.rid)      # the scheduler has already freed its pages
             self.num_preemptions += 1
+        for leaver in plan.released:
+            self.runner.forget(leaver.rid)      # ends with the token on its way; nothing is recomputed
         if not plan.spans:
             return None
         entries, sampling = [], []

@@ -16,9 +16,12 @@ allow.  Pages are reserved portion by portion.
 
 The step loop plans a step before it has read the tokens of the step before
 (``Request.unknown``): a decoding request's span may be that unread token (``Span.feed``);
-a request that is certain to end with it is left alone; one that was evicted with it waits
-at the head of the queue until it is read; and a plan may come back empty because
-everything left waits for tokens (``StepPlan.spans == []``).
+a request that is certain to end with it is left alone (and when it is the victim of an
+eviction its pages go back and it is not queued again: ``StepPlan.released``); one that was
+evicted with it waits at the head of the queue until it is read; and a plan may come back
+empty because everything left waits for tokens (``StepPlan.spans == []``).  A request may
+end while it waits (it was evicted with its EOS token on its way): a finished request is
+never planned, wherever it sits.
 """
 
 from __future__ import annotations
@@ -46,7 +49,8 @@ class Span:
 @dataclass
 class StepPlan:
     spans: list[Span]
-    evicted: list[Request] = field(default_factory=list)
+    evicted: list[Request] = field(default_factory=list)     # pages freed, queued again at the front
+    released: list[Request] = field(default_factory=list)    # pages freed, ending with the token on its way
 
     @property
     def num_tokens(self) -> int:
@@ -76,7 +80,7 @@ class Scheduler:
 
     @property
     def busy(self) -> bool:
-        return bool(self.waiting) or any(not r.finished for r in self.running)
+        return any(not r.finished for r in self.waiting) or any(not r.finished for r in self.running)
 
     def live_requests(self) -> list[Request]:
         """Every request that may hold pages or a slot."""
@@ -86,23 +90,28 @@ class Scheduler:
     def plan(self) -> StepPlan | None:
         """The next step, or None when nothing is left to do."""
         self.running = [r for r in self.running if not r.finished]
+        if any(r.finished for r in self.waiting):
+            # evicted with its last token on its way, and ended when that was read: whoever read
+            # it has given back what it held
+            self.waiting = deque(r for r in self.waiting if not r.finished)
         evicted: list[Request] = []
+        released: list[Request] = []
         while True:
-            spans = self._fill(evicted)
+            spans = self._fill(evicted, released)
             if spans:
-                return StepPlan(spans, evicted)
+                return StepPlan(spans, evicted, released)
             if any(r.unknown for r in self.running) or (self.waiting and self.waiting[0].unknown):
-                return StepPlan([], evicted)     # what is left waits for tokens that are still on the GPU
+                return StepPlan([], evicted, released)   # what is left waits for tokens that are still on the GPU
             if self.running:
                 # nobody could move: every running request waits for pages
-                evicted.append(self._evict_newest())
+                self._evict_newest(evicted, released)
             elif self.waiting:
                 raise OutOfPagesError(
                     f"request {self.waiting[0].rid} needs more pages than the pool can ever provide")
             else:
                 return None
 
-    def _fill(self, evicted: list[Request]) -> list[Span]:
+    def _fill(self, evicted: list[Request], released: list[Request]) -> list[Span]:
         spans: list[Span] = []
         left = self.token_budget
         # 1. a token for every decoding request, oldest first.  When the pool cannot give
@@ -118,7 +127,7 @@ class Scheduler:
                 left -= 1
                 at += 1
             else:
-                evicted.append(self._evict_newest())     # may be ``request`` itself
+                self._evict_newest(evicted, released)    # may be ``request`` itself
         # 2. portions of running requests whose tokens are not all cached yet
         for request in self.running:
             if left <= 0:
@@ -166,11 +175,16 @@ class Scheduler:
         free = min(manager.num_free_pages(g) for g in range(len(manager.groups))) * page
         return max(0, min(request.pending, self.chunk, left, reserved + free - request.cached))
 
-    def _evict_newest(self) -> Request:
+    def _evict_newest(self, evicted: list[Request], released: list[Request]) -> None:
         """Free the newest running request's pages and slot; it keeps its tokens and
-        goes to the front of the queue (it is older than anything waiting)."""
+        goes to the front of the queue (it is older than anything waiting).  A victim that
+        is certain to end with the token on its way will never run again: it only gives
+        back what it holds, and whoever reads that token finishes it."""
         victim = self.running.pop()
         self.manager.free(victim.rid)
+        if victim.closing:
+            released.append(victim)
+            return
         victim.rewind()
         self.waiting.appendleft(victim)
-        return victim
+        evicted.append(victim)
