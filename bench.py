@@ -142,12 +142,8 @@ class StepCost:
         _, layouts = model.cache_layout()
         self.kv_bytes_per_token = sum(lay.request.bytes_per_token(runner.dtype) for lay in layouts.values())
         # attention flops of a layer call: 4 * heads * head_dim per (query, visible key) pair
-        self.pair_flops = 0.0
-        for call in plan.order:
-            for _, sub in plan.layers[call.layer].parts:
-                params = sub.spec.as_dict()
-                if sub.family == "mixer" and "num_heads" in params and "head_dim" in params:
-                    self.pair_flops += 4.0 * params["num_heads"] * params["head_dim"]
+        self.pair_flops = sum(mixer.pair_flops() for call in plan.order
+                              for mixer in model.blocks[call.layer].mixers.values())
 
     def decode_bytes(self, batch: int, mean_keys: float) -> float:
         return self.weight_bytes + batch * (self.embedding_row_bytes + mean_keys * self.kv_bytes_per_token)
@@ -351,7 +347,7 @@ def run_continuous(args) -> int:
         steps0 = llm.num_steps
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        outs = llm.generate(prompt_token_ids=prompts, sampling_params=params)
+        outs = llm.generate(prompt_token_ids=prompts, sampling_params=params, use_tqdm=False)
         torch.cuda.synchronize()
         runs.append((time.perf_counter() - t0, llm.num_steps - steps0))
     elapsed, steps = runs[-1]
@@ -418,7 +414,7 @@ def run_trace(args) -> int:
             steps0 = llm.num_steps
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            outs = llm.generate(prompt_token_ids=prompts, sampling_params=params)
+            outs = llm.generate(prompt_token_ids=prompts, sampling_params=params, use_tqdm=False)
             torch.cuda.synchronize()
             elapsed, steps = time.perf_counter() - t0, llm.num_steps - steps0
         assert [len(o.output_token_ids) for o in outs] == new_tokens
@@ -469,7 +465,7 @@ def run_attention(args) -> int:
         v_cache = torch.randn_like(k_cache)
         spans = [StepSpan(request=i, tokens=[0], ctx_len=context, state_slot=i,
                           tables=[[j * batch_size + i for j in range(pages_each)]]) for i in range(batch_size)]
-        batch = build_batch(spans, 1, dev)
+        batch = build_batch(spans, 1, dev, [attn.ATTENTION_WORK])
         qkv = torch.randn(batch_size, (nh + 2 * nkv) * hd, device=dev, dtype=torch.bfloat16)
         weight = torch.ones(hd, device=dev, dtype=torch.float32)
         angle = torch.rand(batch_size, hd // 2, device=dev, dtype=torch.float32)

@@ -6,6 +6,7 @@ from __future__ import annotations
 import torch
 
 from tokamak_amd.engine.batch import StepSpan, build_batch
+from tokamak_amd.kernels.attention import ATTENTION_WORK
 
 
 def pack_pages(k_cache, v_cache, k_seq, v_seq, table, ps):
@@ -48,7 +49,8 @@ def reference_attention(q, k, v, positions, scale, window=None):
 
 
 def make_batch(spans, device="cuda"):
-    """spans: list of (tokens_count, ctx_len, table) -> StepBatch with one cache group."""
+    """spans: list of (tokens_count, ctx_len, table) -> StepBatch with one cache group and
+    the attention kernels' work lists."""
     ss = [StepSpan(request=i, tokens=[0] * n, ctx_len=ctx, state_slot=i, tables=[table])
           for i, (n, ctx, table) in enumerate(spans)]
-    return build_batch(ss, 1, device)
+    return build_batch(ss, 1, device, [ATTENTION_WORK])

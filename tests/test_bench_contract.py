@@ -20,7 +20,7 @@ def test_more_than_one_gpu_is_refused_with_one_line_and_code_2():
 
 def test_the_reference_trace_has_the_published_totals():
     # 32 requests, cap 256, seed 0: 4,915 prompt and 2,901 output tokens
-    # (/root/reference/benchmarks/README.md:87-90); every prompt 16..512 tokens, every request
+    # (reference: benchmarks/README.md:87-90); every prompt 16..512 tokens, every request
     # within the 1,024 tokens the measurement allows a sequence
     import bench
 

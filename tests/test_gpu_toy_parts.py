@@ -16,7 +16,7 @@ DEV = "cuda"
 def register_toys():
     from tokamak_amd.config import register_part
     from tokamak_amd.parts.base import (Block, CacheRequest, FeedForward, Mixer, PagedArray, PositionData,
-                                        PositionEncoding, StateArray)
+                                        PositionEncoding, StateArray, StepPlanner)
     from tokamak_amd.weights.spec import TensorSpec
 
     class RunningMeanMixer(Mixer):
@@ -133,6 +133,77 @@ def register_toys():
                 out[starts[i]:starts[i + 1]] = (mean_a @ self.oa.float().T + mean_b @ self.ob.float().T).to(h.dtype)
             return out
 
+    class ScanChunks(StepPlanner):
+        """The cut of a step that the decaying-sum mixer below wants: every span in chunks of up
+        to 64 consecutive tokens, each with its request's row, in the order they must run."""
+
+        name = "toy_scan"
+
+        def lists(self, q_lens, ctx_lens):
+            first, count, request = [], [], []
+            at = 0
+            for row, q in enumerate(q_lens):
+                for t in range(0, q, SCAN_CHUNK):
+                    first.append(at + t)
+                    count.append(min(SCAN_CHUNK, q - t))
+                    request.append(row)
+                at += q
+            return ({"first": first, "count": count, "request": request},
+                    {"num_chunks": len(first), "longest": max(count, default=0)})
+
+        def bucket(self, facts):
+            facts["longest"] = 1 if facts["longest"] <= 1 else SCAN_CHUNK
+            return facts
+
+    scan_chunks = ScanChunks()
+
+    class DecayingSumMixer(Mixer):
+        """out[t] = W s[t], s[t] = decay * s[t-1] + h[t]: state of fixed size, advanced chunk
+        by chunk from a work list of the mixer's own (``batch.lists["toy_scan.*"]``), which the
+        step's descriptor carries because ``step_planner`` asks for it.  It refuses pages that
+        do not divide its chunk, although it has none: the engine only passes the question on."""
+
+        def __init__(self, *, hidden_size, decay, dtype, device):
+            super().__init__(dtype=dtype, device=device)
+            self.h, self.decay = hidden_size, float(decay)
+            self.w = None
+
+        def expected_tensors(self, prefix):
+            return {prefix + "mix.weight": TensorSpec((self.h, self.h), held="float32")}    # a matrix kept in 32-bit
+
+        def bind(self, prefix, fetch):
+            self.w = fetch(prefix + "mix.weight")
+
+        def state_request(self):
+            return {"s": StateArray((self.h,))}
+
+        def step_planner(self):
+            return scan_chunks
+
+        def check_page_size(self, page_size):
+            if SCAN_CHUNK % page_size:
+                raise ValueError(f"the toy scan's chunks of {SCAN_CHUNK} need a page size that divides them, got {page_size}")
+
+        def forward(self, h, batch, store, writes_cache=True, position=None):
+            assert self.w.dtype == torch.float32
+            n = batch.facts["toy_scan.num_chunks"]
+            first = batch.lists["toy_scan.first"].tolist()
+            count = batch.lists["toy_scan.count"].tolist()
+            request = batch.lists["toy_scan.request"].tolist()
+            assert len(first) == n and sum(count) == batch.num_tokens and max(count) <= batch.facts["toy_scan.longest"]
+            slots = batch.state_slots.tolist()
+            out = torch.empty_like(h)
+            state = store.state["s"]
+            for a, c, r in zip(first, count, request):
+                # a chunk at once: s[t] = decay^(t+1) s_in + sum_{u<=t} decay^(t-u) h[u]
+                x = h[a:a + c].float()
+                steps = torch.arange(c, device=h.device, dtype=torch.float32)
+                powers = self.decay ** (steps[:, None] - steps[None, :]).clamp(min=0) * (steps[:, None] >= steps[None, :])
+                s = powers @ x + (self.decay ** (steps + 1))[:, None] * state[slots[r]][None, :]
+                out[a:a + c] = (s @ self.w.T).to(h.dtype)
+                state[slots[r]] = s[-1]
+            return out
+
     class Top1RoutedFF(FeedForward):
         """Two experts, each one matrix; a router picks one per token."""
 
@@ -224,7 +295,26 @@ def register_toys():
         def forward(self, resid, pending, batch, store, writes_cache):
             return self.parts["mixer"].forward(self.parts["norm"].forward(resid, pending), batch, store, writes_cache, None)
 
+    class TwoMixerBlock(Block):
+        """Two mixers side by side behind one norm, each with a cache slot of its own:
+        x += attend(n(x)) + remember(n(x)).  ``store`` is a dict of slot stores by role."""
+
+        roles = ("norm", "attend", "remember")
+        optional = ("position",)
+
+        def forward(self, resid, pending, batch, store, writes_cache):
+            p = self.parts
+            assert set(store) == {"attend", "remember"} and list(self.mixers) == ["attend", "remember"]
+            position = p["position"].prepare(batch) if "position" in p else None
+            h = p["norm"].forward(resid, pending)
+            a = p["attend"].forward(h, batch, store["attend"], writes_cache, position)
+            b = p["remember"].forward(h, batch, store["remember"], writes_cache, None)
+            a = a.sum(0) if a.dim() == 3 else a
+            return a.float() + b.float()
+
     for family, kind, cls in (("mixer", "toy_running_mean", RunningMeanMixer),
+                              ("mixer", "toy_decaying_sum", DecayingSumMixer),
+                              ("block", "toy_two_mixers", TwoMixerBlock),
                               ("mixer", "toy_last_token", LastTokenMixer),
                               ("mixer", "toy_two_width", TwoWidthCacheMixer),
                               ("feed_forward", "toy_top1", Top1RoutedFF),
@@ -237,6 +327,7 @@ def register_toys():
 
 
 H, V = 64, 100
+SCAN_CHUNK = 64
 
 
 def _specs():
@@ -523,6 +614,102 @@ def test_a_state_mixer_recorded_into_a_graph_sees_every_token_once(dtype):
     assert sum(g.replays for g in graphed._graphs.values()) == 12 - 2     # each shape's first step ran eagerly
 
 
+def scan_plan():
+    """A mixer with a work list of its own, alone in a layer; then a layer with two mixers
+    side by side (attention with pages, the scan with state), a cache slot each."""
+    from tokamak_amd.config import LayerCall, LayerSpec, PartSpec, SubPart
+
+    s = _specs()
+    scan = lambda prefix: SubPart("mixer", PartSpec.of("toy_decaying_sum", hidden_size=H, decay=0.9), prefix)   # noqa: E731
+    layers = (
+        LayerSpec.of(PartSpec.of("toy_mixer_only"), norm=s["n"]("n."), mixer=scan("scan.")),
+        LayerSpec.of(PartSpec.of("toy_two_mixers"), norm=s["n"]("n."), attend=SubPart("mixer", s["attn"](), "attn."),
+                     remember=scan("scan."), position=s["rope"]),
+    )
+    return _plan(layers, (LayerCall(0, 0), LayerCall(1, (1, 2))))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_brings_its_own_work_lists_and_a_layer_holds_two_mixers(dtype):
+    """The decaying-sum mixer consumes chunks of 64 tokens from lists that its own planner
+    makes; the step descriptor carries them beside the attention kernels' lists without the
+    engine knowing either.  The second layer has two mixers, each with its own cache slot.
+    Logits are those of the formula computed here on whole sequences, under every cutting."""
+    from tokamak_amd.engine.runner import StepEntry
+
+    plan = scan_plan()
+    runner = make_runner(dtype, pool_tokens=512, plan=plan)
+    assert [p.name for p in runner.model.step_planners()] == ["toy_scan", "attention"]
+    groups, layouts = runner.model.cache_layout()
+    assert sorted(layouts) == [1] and [n for n, _ in layouts[1].request.arrays] == ["k", "v"]
+    assert sorted(runner.model.state_requests()) == [0, 2]          # the two scans' state, a slot each
+    assert runner.storage.slot(0).state["s"].data_ptr() != runner.storage.slot(2).state["s"].data_ptr()
+    assert runner.model.blocks[0].mixer is not None and runner.model.blocks[1].mixer is None
+    assert list(runner.model.blocks[1].mixers) == ["attend", "remember"]
+
+    prompts = {"a": random_ids(V, 150, 21), "b": random_ids(V, 70, 22)}
+    whole = {}
+    for rid, toks in prompts.items():
+        whole[rid] = runner.step([StepEntry(rid, toks, list(range(len(toks))))]).cpu()
+        runner.end(rid)
+
+    if dtype == "float32":
+        # the first layer's formula, written out: s[t] = 0.9 s[t-1] + n(x)[t]; x += W s
+        model = runner.model
+        x = model.embedding.weight.float()[torch.tensor(prompts["a"], device=DEV)]
+        gamma = model.blocks[0].parts["norm"].weight.float()
+        n = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-5) * gamma
+        s = torch.zeros(H, device=DEV, dtype=torch.float64)
+        rows = []
+        for t in range(n.shape[0]):
+            s = 0.9 * s + n[t].double()
+            rows.append(s)
+        after_first = x.double() + torch.stack(rows) @ model.blocks[0].mixer.w.double().T
+        # ... which is what the second layer's norm reads: compare through a model of the first layer alone
+        first_only = make_runner(dtype, pool_tokens=512, plan=_plan(plan.layers[:1], plan.order[:1]))
+        got = first_only.step([StepEntry("a", prompts["a"], list(range(150)))])
+        gamma_out = first_only.model.final_norm.weight.double()
+        y = after_first * torch.rsqrt((after_first * after_first).mean(-1, keepdim=True) + 1e-5) * gamma_out
+        want = y @ first_only.model.head.weight.double().T
+        torch.testing.assert_close(got.double(), want, rtol=0, atol=2e-4)
+
+    tol = cutting_tolerance(dtype, whole, plan, prompts)
+    # cut at and off the chunk's edges, beside the other request, then token by token
+    rows = {"a": [], "b": []}
+    done = {"a": 0, "b": 0}
+    steps = ([("a", 64)], [("a", 2), ("b", 65)], [("a", 70), ("b", 1)], [("a", 1), ("b", 1)], [("a", 13), ("b", 3)])
+    for step in steps:
+        batch_entries = [StepEntry(r, prompts[r][done[r]:done[r] + n], list(range(n))) for r, n in step]
+        out = runner.step(batch_entries).cpu()
+        at = 0
+        for r, n in step:
+            rows[r].append(out[at:at + n])
+            at += n
+            done[r] += n
+    assert done == {"a": 150, "b": 70}
+    for r in rows:
+        torch.testing.assert_close(torch.cat(rows[r]), whole[r], **tol)
+    runner.end_all()
+    runner.manager.check()
+
+
+def test_a_part_may_refuse_a_page_size():
+    """The engine asks every part whether it can work with the cache's page size; it has no
+    rule of its own."""
+    from tokamak_amd.engine.model import LayeredModel
+    from tokamak_amd.engine.runner import ModelRunner
+    from tokamak_amd.weights.sources import RandomSource
+
+    register_toys()
+    plan = scan_plan()
+    expected = {n: s for n, s in LayeredModel(plan, dtype=torch.float32, device="meta").expected_tensors().items() if not s.ignored}
+    source = RandomSource(expected, seed=5)
+    with pytest.raises(ValueError, match="toy scan's chunks"):
+        ModelRunner(plan, source, dtype="float32", page_size=24, kv_pool_tokens=96, max_requests=2)
+    with pytest.raises(ValueError, match="attention kernels"):
+        ModelRunner(plan, source, dtype="float32", page_size=4, kv_pool_tokens=96, max_requests=2)
+
+
 # ---------------------------------------------------------------------------
 # a whole toy architecture: config.json keys of its own -> registry -> folder -> LLM -> command line
 # ---------------------------------------------------------------------------
@@ -629,6 +816,20 @@ def test_a_toy_architecture_goes_from_config_json_to_generated_tokens(tmp_path, 
     tight.runner.manager.check()
     half = LLM(folder, dtype="bfloat16", block_size=8, max_batch_size=8).generate(prompt_token_ids=prompts, sampling_params=params)
     assert all(len(o.output_token_ids) == 40 for o in half)
+    # every bfloat16 token is the float32 model's best token for the sequence so far, or one whose
+    # float32 logit lies within bfloat16 rounding of the best (twice the replay tests' bound)
+    from tokamak_amd.engine.runner import StepEntry
+
+    best = 0
+    for prompt, out in zip(prompts, half):
+        tokens = out.output_token_ids
+        rows = roomy.runner.step([StepEntry("check", prompt + tokens[:-1], list(range(len(prompt) - 1, len(prompt) + 39)))])
+        roomy.runner.end("check")
+        for i, token in enumerate(tokens):
+            slack = 2 * (2e-3 + 2e-2 * float(rows[i].abs().max()))
+            assert float(rows[i, token]) >= float(rows[i].max()) - slack, f"bfloat16 token {i} of a {len(prompt)}-token prompt"
+            best += int(token == int(rows[i].argmax()))
+    assert best >= 0.9 * 40 * len(prompts)
 
     broken = tmp_path / "broken"
     broken.mkdir()

@@ -113,3 +113,24 @@ def test_float32_checkpoint_converts_to_compute_dtype(tmp_path):
     assert model.final_norm.weight.dtype == torch.float32  # stored in 32-bit, stays so
     stored = load_file(folder / "model.safetensors")["model.norm.weight"]
     assert torch.equal(model.final_norm.weight, stored)
+
+
+def test_a_tensor_is_held_as_its_spec_says_whatever_its_role():
+    """Matrices in the compute dtype, vectors in float32, tables as int32 by habit; ``held``
+    overrides that without changing what kind of numbers the tensor is."""
+    from tokamak_amd.weights.loader import target_dtype
+    from tokamak_amd.weights.spec import TensorSpec
+
+    bf16, f32 = torch.bfloat16, torch.float32
+    assert target_dtype(TensorSpec((4, 4)), bf16, bf16) == bf16
+    assert target_dtype(TensorSpec((4, 4)), f32, bf16) == bf16
+    assert target_dtype(TensorSpec((4,), role="vector"), bf16, bf16) == f32
+    assert target_dtype(TensorSpec((4,), role="table"), torch.int64, bf16) == torch.int32
+    router = TensorSpec((2, 4), held="float32")                # a matrix that must not be rounded
+    assert router.role == "matrix" and target_dtype(router, f32, bf16) == f32
+    assert target_dtype(TensorSpec((4, 4), held="stored"), torch.float16, bf16) == torch.float16
+    assert target_dtype(TensorSpec((4,), role="vector", held="compute"), f32, bf16) == bf16
+    with pytest.raises(ValueError, match="held"):
+        TensorSpec((4,), held="float64")
+    with pytest.raises(ValueError, match="role"):
+        TensorSpec((4,), role="scalar")

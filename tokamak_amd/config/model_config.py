@@ -96,14 +96,19 @@ class LayerCall:
 
     ``layer`` indexes ``ModelPlan.layers`` (the weights); the same layer may be
     called more than once.  ``cache`` is the cache slot the call's mixer uses;
-    two calls with the same slot share what is stored there.  A call with
-    ``writes_cache=False`` only reads the slot (it attends over keys and values
-    another call stored) and stores nothing itself.
+    two calls with the same slot share what is stored there.  A layer whose block
+    holds several mixers brings a tuple of slots, one for each mixer in the order
+    the layer names them.  A call with ``writes_cache=False`` only reads its slots
+    (it attends over keys and values another call stored) and stores nothing itself.
     """
 
     layer: int
-    cache: int
+    cache: int | tuple[int, ...]
     writes_cache: bool = True
+
+    @property
+    def slots(self) -> tuple[int, ...]:
+        return self.cache if isinstance(self.cache, tuple) else (self.cache,)
 
 
 @dataclass(frozen=True)
@@ -130,17 +135,15 @@ class ModelPlan:
         for call in self.order:
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"run order names layer {call.layer}, model has {len(self.layers)}")
-        writers: dict[int, int] = {}
+        written = {slot for call in self.order if call.writes_cache for slot in call.slots}
         for call in self.order:
-            if call.writes_cache:
-                writers[call.cache] = writers.get(call.cache, 0) + 1
-        for call in self.order:
-            if not call.writes_cache and call.cache not in writers:
-                raise ValueError(f"cache slot {call.cache} is read but never written")
+            for slot in call.slots:
+                if not call.writes_cache and slot not in written:
+                    raise ValueError(f"cache slot {slot} is read but never written")
 
     @property
     def num_cache_slots(self) -> int:
-        return 1 + max((c.cache for c in self.order), default=-1)
+        return 1 + max((slot for c in self.order for slot in c.slots), default=-1)
 
 
 def default_order(num_layers: int) -> tuple[LayerCall, ...]:

@@ -1,7 +1,6 @@
 // Entry points for callers that cannot allocate device memory.
 //
-// tk_argmax_no_alloc has no counterpart in the reference (its sampler calls
-// torch.argmax, src/tokamak/sampling/sampler.py:58-59).  It is for callers that
+// tk_argmax_no_alloc has no counterpart in the reference.  It is for callers that
 // cannot call hipMalloc: code under HIP graph capture, tight serving loops,
 // harnesses that forbid allocation.  It computes what tk_argmax computes with
 // the same kernels, but keeps the per-segment winners (the scratch that tk_argmax

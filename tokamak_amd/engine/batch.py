@@ -6,14 +6,52 @@ tokens from R requests; request r contributes ``q_len[r]`` consecutive tokens
 that start at absolute position ``ctx_len[r]`` (what its cache already holds).
 A decode token is a span of length one, a prompt portion a longer one; any
 mixture is one batch.
+
+The descriptor itself knows nothing of how a part cuts a step into work for its
+kernels.  A part that wants lists of its own (tiles of a portion's tokens, chunks
+of a scan, rows that run alone) declares a ``StepPlanner``: it is
+asked once a step, with the step's span lengths and cached lengths, and what it
+returns travels to the device in the same buffer as the descriptor and is found
+under the planner's name (``batch.lists["<planner>.<list>"]``,
+``batch.facts["<planner>.<fact>"]``).
 """
 
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from typing import Sequence
 
 import numpy as np
 import torch
+
+
+class StepPlanner:
+    """How a part's kernels want a step cut into work.
+
+    ``lists(q_lens, ctx_lens)`` is called once a step with, per request of the step, the
+    number of tokens it brings and the number its cache already holds.  It returns
+    (arrays, facts): ``arrays`` maps a key to a list of integers, which reaches the device
+    as int32 in the same copy as the step's descriptor and is found as
+    ``batch.lists["<name>.<key>"]``; ``facts`` maps a key to a host integer (a count, a
+    longest context) from which the part picks kernels and grids,
+    ``batch.facts["<name>.<key>"]``.  The length of every array must follow from ``q_lens``
+    and the facts alone.
+
+    ``bucket(facts)`` is applied before a step of single tokens is recorded for replay:
+    a recorded step serves every later step with equal facts, so a fact that moves with
+    every token (a longest context) is rounded up here to a few values; the kernels must
+    be right for any true value up to the rounded one.
+
+    Parts that return planners of the same ``name`` share one (the lists are made once).
+    """
+
+    name = ""
+
+    def lists(self, q_lens: list[int], ctx_lens: list[int]) -> tuple[dict[str, list[int]], dict[str, int]]:
+        return {}, {}
+
+    def bucket(self, facts: dict[str, int]) -> dict[str, int]:
+        return facts
 
 
 @dataclass
@@ -42,23 +80,13 @@ class StepBatch:
     state_slots: torch.Tensor    # [R] int32
     logit_rows: torch.Tensor     # [M] int32, token rows whose logits are wanted
     block_tables: list[torch.Tensor]  # per cache group [R, max_pages] int32
-    # work lists for the attention kernels: single (decode) tokens, and tiles of up to
-    # 16, and of up to 32, consecutive tokens of the longer spans
-    decode_tokens: torch.Tensor | None = None   # [num_decode] int32 token rows
-    tile_first: torch.Tensor | None = None      # [num_tiles] int32 first token row
-    tile_count: torch.Tensor | None = None      # [num_tiles] int32 tokens in the tile
-    wide_first: torch.Tensor | None = None      # [num_wide] int32 first token row of a 32-token tile
-    wide_count: torch.Tensor | None = None      # [num_wide] int32 tokens in it
     feed_slots: torch.Tensor | None = None      # [N] int32: the first num_feed name token rows whose id ...
     feed_rows: torch.Tensor | None = None       # [N] int32: ... is that row of the sampler's last output
     num_feed: int = 0
-    num_decode: int = 0
-    num_tiles: int = 0
-    num_wide: int = 0
-    num_tile_tokens: int = 0                    # tokens of the spans that are cut into tiles
-    max_decode_len: int = 0                     # longest context among the decode tokens
-    max_tile_len: int = 0                       # longest context (with the portion) among the tiled spans
-    min_tile_ctx: int = 0                       # shortest cached context among the tiled spans
+    # what the parts' planners asked for: int32 device arrays, and host integers that
+    # choose kernels and grids, both under "<planner name>.<key>"
+    lists: dict[str, torch.Tensor] = field(default_factory=dict)
+    facts: dict[str, int] = field(default_factory=dict)
     # host copies, for choosing kernels and grids
     q_lens: list[int] = field(default_factory=list)
     ctx_lens: list[int] = field(default_factory=list)
@@ -67,9 +95,7 @@ class StepBatch:
     memo: dict = field(default_factory=dict)  # per-step data shared between layers
 
 
-TILE_TOKENS = 16   # tokens per attention tile of a prompt portion
-WIDE_TOKENS = 32   # and per tile of the wide attention kernel
-NUM_FIXED = 14     # arrays in the packed buffer before the block tables
+NUM_FIXED = 9      # arrays in the packed buffer before the block tables
 
 
 @dataclass
@@ -83,16 +109,17 @@ class PackedBatch:
     num_tokens: int
     num_requests: int
     num_logit_rows: int
-    num_decode: int
-    num_tiles: int
-    num_wide: int
     q_lens: list[int]
     ctx_lens: list[int]
-    max_decode_len: int
-    max_tile_len: int = 0
-    min_tile_ctx: int = 0
+    list_names: list[str] = field(default_factory=list)   # planners' lists, in buffer order after the tables
+    facts: dict[str, int] = field(default_factory=dict)
     num_feed: int = 0
     max_feed_row: int = -1
+
+    def shape_key(self) -> tuple:
+        """What two steps must share to use one recorded step: the buffer's cut and the
+        planners' facts (kernels and grids are chosen from them)."""
+        return (tuple(self.offsets), tuple(sorted(self.facts.items())))
 
 
 def table_width(longest: int, fixed: int | None = None) -> int:
@@ -103,38 +130,41 @@ def table_width(longest: int, fixed: int | None = None) -> int:
     return max(4, -(-longest // 4) * 4)
 
 
-def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] | None = None) -> PackedBatch:
+def pack_batch(spans: list[StepSpan], num_groups: int, planners: Sequence = (),
+               fixed_widths: list[int] | None = None, bucket: bool = False) -> PackedBatch:
+    """``planners``: the ``StepPlanner`` objects of the model's parts (one per name).
+    ``bucket``: round the planners' facts as they ask for recorded steps, so that steps of
+    nearly the same shape share a recording."""
     r = len(spans)
     n = sum(len(s.tokens) for s in spans)
     widths = [table_width(max((len(s.tables[g]) for s in spans), default=0),
                           None if fixed_widths is None else fixed_widths[g])
               for g in range(num_groups)]
     m = sum(len(s.want) for s in spans)
-    decode_rows, tiles, wide = [], [], []
-    at = 0
-    for s in spans:
-        q = len(s.tokens)
-        if q == 1:
-            decode_rows.append(at)
-        else:
-            tiles.extend((at + t, min(TILE_TOKENS, q - t)) for t in range(0, q, TILE_TOKENS))
-            wide.extend((at + t, min(WIDE_TOKENS, q - t)) for t in range(0, q, WIDE_TOKENS))
-        at += q
-    nd, nt, nw = len(decode_rows), len(tiles), len(wide)
-    sizes = [n, n, n, r + 1, r, r, m, nd, nt, nt, nw, nw, n, n] + [r * w for w in widths]
+    q_lens = [len(s.tokens) for s in spans]
+    ctx_lens = [s.ctx_len for s in spans]
+    extra: list[tuple[str, Sequence[int]]] = []
+    facts: dict[str, int] = {}
+    for planner in planners:
+        arrays, found = planner.lists(q_lens, ctx_lens)
+        if bucket:
+            found = planner.bucket(dict(found))
+        for key, values in arrays.items():
+            extra.append((f"{planner.name}.{key}", values))
+        for key, value in found.items():
+            facts[f"{planner.name}.{key}"] = int(value)
+    sizes = [n, n, n, r + 1, r, r, m, n, n] + [r * w for w in widths] + [len(values) for _, values in extra]
     offsets = [0]
     for size in sizes:
         offsets.append(offsets[-1] + size)
     buf = np.zeros(offsets[-1], dtype=np.int32)
-    tok, pos, req, qs, ctx, slots, rows, dec, tfirst, tcount, wfirst, wcount, fslots, frows = (
+    tok, pos, req, qs, ctx, slots, rows, fslots, frows = (
         buf[offsets[i]:offsets[i + 1]] for i in range(NUM_FIXED))
     tabs = [buf[offsets[NUM_FIXED + g]:offsets[NUM_FIXED + 1 + g]].reshape(r, widths[g])
             for g in range(num_groups)]
-    dec[:] = decode_rows
-    tfirst[:] = [t[0] for t in tiles]
-    tcount[:] = [t[1] for t in tiles]
-    wfirst[:] = [t[0] for t in wide]
-    wcount[:] = [t[1] for t in wide]
+    for i, (_, values) in enumerate(extra):
+        at = NUM_FIXED + num_groups + i
+        buf[offsets[at]:offsets[at + 1]] = values
     at = 0
     mi = 0
     fed = 0
@@ -164,11 +194,7 @@ def pack_batch(spans: list[StepSpan], num_groups: int, fixed_widths: list[int] |
     qs[r] = at
     return PackedBatch(
         buf=buf, offsets=offsets, widths=widths, num_tokens=n, num_requests=r, num_logit_rows=m,
-        num_decode=nd, num_tiles=nt, num_wide=nw, q_lens=[len(s.tokens) for s in spans],
-        ctx_lens=[s.ctx_len for s in spans],
-        max_decode_len=max((s.ctx_len + 1 for s in spans if len(s.tokens) == 1), default=0),
-        max_tile_len=max((s.ctx_len + len(s.tokens) for s in spans if len(s.tokens) > 1), default=0),
-        min_tile_ctx=min((s.ctx_len for s in spans if len(s.tokens) > 1), default=0),
+        q_lens=q_lens, ctx_lens=ctx_lens, list_names=[name for name, _ in extra], facts=facts,
         num_feed=fed, max_feed_row=max((s.feed for s in spans if s.feed is not None), default=-1))
 
 
@@ -176,26 +202,24 @@ def batch_from_device(packed: PackedBatch, dev: torch.Tensor) -> StepBatch:
     """Cut the device copy ``dev`` of ``packed.buf`` into the descriptor's arrays."""
     o, r, widths = packed.offsets, packed.num_requests, packed.widths
     parts = [dev[o[i]:o[i + 1]] for i in range(len(o) - 1)]
+    first_list = NUM_FIXED + len(widths)
     return StepBatch(
         num_tokens=packed.num_tokens, num_requests=r, num_logit_rows=packed.num_logit_rows,
         token_ids=parts[0], positions=parts[1], req_of_token=parts[2], q_start=parts[3],
         ctx_len=parts[4], state_slots=parts[5], logit_rows=parts[6],
         block_tables=[parts[NUM_FIXED + g].view(r, widths[g]) for g in range(len(widths))],
-        decode_tokens=parts[7], tile_first=parts[8], tile_count=parts[9],
-        wide_first=parts[10], wide_count=parts[11], feed_slots=parts[12], feed_rows=parts[13],
-        num_feed=packed.num_feed, num_decode=packed.num_decode, num_tiles=packed.num_tiles, num_wide=packed.num_wide,
-        num_tile_tokens=sum(q for q in packed.q_lens if q > 1),
-        max_decode_len=packed.max_decode_len, max_tile_len=packed.max_tile_len,
-        min_tile_ctx=packed.min_tile_ctx,
+        feed_slots=parts[7], feed_rows=parts[8], num_feed=packed.num_feed,
+        lists={name: parts[first_list + i] for i, name in enumerate(packed.list_names)},
+        facts=dict(packed.facts),
         q_lens=packed.q_lens, ctx_lens=packed.ctx_lens,
         max_q_len=max(packed.q_lens, default=0),
         max_seq_len=max((c + q for c, q in zip(packed.ctx_lens, packed.q_lens)), default=0),
     )
 
 
-def build_batch(spans: list[StepSpan], num_groups: int, device) -> StepBatch:
+def build_batch(spans: list[StepSpan], num_groups: int, device, planners: Sequence = ()) -> StepBatch:
     """Pack the descriptor into one host buffer and copy it to the device once."""
-    packed = pack_batch(spans, num_groups)
+    packed = pack_batch(spans, num_groups, planners)
     host = torch.from_numpy(packed.buf)
     if torch.device(device).type == "cuda":
         dev = host.pin_memory().to(device, non_blocking=True)

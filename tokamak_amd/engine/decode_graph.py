@@ -1,7 +1,8 @@
 """Captured decode steps.
 
 A step in which every request brings exactly one token has a fixed shape once
-the batch size, the block-table width and the split of the context are fixed.
+the batch size, the block-table width and what the parts' planners say of the step
+(for attention: how the context is split) are fixed.
 Such a step is recorded once into a HIP graph and replayed: one launch instead
 of several hundred.  The graph reads its descriptor from a static device
 buffer that is refilled (one host-to-device copy) before every replay; nothing
@@ -24,18 +25,6 @@ def pow2_at_least(n: int, floor: int) -> int:
     while v < n:
         v *= 2
     return v
-
-
-def quarter_octave_at_least(n: int, floor: int) -> int:
-    """The smallest of floor, 1.25 floor, 1.5 floor, 1.75 floor, 2 floor, 2.5 floor, ...
-    that is >= n: four buckets an octave, so a bucket overshoots by a quarter at most."""
-    v = floor
-    while 2 * v < n:
-        v *= 2
-    if n <= v:
-        return v
-    step = v // 4
-    return v + -(-(n - v) // step) * step
 
 
 class DecodeGraph:

@@ -52,16 +52,27 @@ def pending_kind(pending) -> tuple:
     return (type(pending).__name__, tuple((name, tuple(t.shape), t.dtype, t.stride()) for name, t in pending_tensors(pending)))
 
 
+def _stores(store) -> list[tuple[str, object]]:
+    """(role, slot store) pairs of what a block receives as ``store``: one slot, or a dict of
+    slots by the roles of its mixers."""
+    return list(store.items()) if isinstance(store, dict) else [("", store)]
+
+
+def store_groups(store) -> tuple[int, ...]:
+    return tuple(s.group for _, s in _stores(store))
+
+
 def own_tensors(block, store) -> dict[tuple, torch.Tensor]:
-    """The tensors that belong to one layer call: its parts' and its cache slot's."""
+    """The tensors that belong to one layer call: its parts' and its cache slots'."""
     out: dict[tuple, torch.Tensor] = {}
     for role, part in block.parts.items():
         for name, t in _fields(part):
             out[("part", role, name)] = t
-    for name, t in store.arrays.items():
-        out[("cache", name)] = t
-    for name, t in store.state.items():
-        out[("state", name)] = t
+    for role, slot in _stores(store):
+        for name, t in slot.arrays.items():
+            out[("cache", role, name)] = t
+        for name, t in slot.state.items():
+            out[("state", role, name)] = t
     return out
 
 

@@ -7,7 +7,6 @@ load once, then ``generate`` runs a scheduler-driven step loop and returns one
 
 from __future__ import annotations
 
-import json
 import logging
 import random
 import time
@@ -18,6 +17,7 @@ from pathlib import Path
 import torch
 
 from tokamak_amd.config.registry import get_architecture, load_model_description
+from tokamak_amd.engine import text
 from tokamak_amd.engine.outputs import RequestOutput
 from tokamak_amd.engine.runner import ModelRunner, StepEntry, resolve_dtype
 from tokamak_amd.kernels import ops
@@ -145,7 +145,7 @@ class LLM:
         logger.info("Loaded %d tensors in %.1f s; cache pool of %d tokens in pages of %d",
                     self.runner.num_tensors, time.perf_counter() - started, self.runner.kv_pool_tokens, block_size)
         self.folder = folder
-        self.tokenizer = self._load_tokenizer(folder) if folder is not None else None
+        self.tokenizer = text.load_tokenizer(folder)
         self.num_steps = 0
         self.num_preemptions = 0
         # the step loop runs one step ahead of the tokens it has read (see generate)
@@ -156,41 +156,16 @@ class LLM:
         self._progress = None
         self.last_progress = ""   # finished/all requests of the last generate() that showed a bar
 
-    @staticmethod
-    def _load_tokenizer(folder: Path):
-        path = folder / "tokenizer.json"
-        if not path.is_file():
-            return None
-        try:
-            from tokenizers import Tokenizer
-        except ImportError:
-            return None
-        return Tokenizer.from_file(str(path))
-
     def chat_prompt(self, user_text: str) -> str:
-        """``user_text`` as a single user turn, ready to tokenize.  The folder's own
-        chat template (``tokenizer_config.json``, rendered in a sandbox with
-        ``enable_thinking=False`` as the reference's example asks,
-        examples/basic_generation.py:25-30) when it has one; else the architecture's."""
-        template = None
-        if self.folder is not None and (self.folder / "tokenizer_config.json").is_file():
-            template = json.loads((self.folder / "tokenizer_config.json").read_text()).get("chat_template")
-        if isinstance(template, str):
-            from jinja2.sandbox import ImmutableSandboxedEnvironment
-
-            env = ImmutableSandboxedEnvironment(trim_blocks=True, lstrip_blocks=True)
-            return env.from_string(template).render(
-                messages=[{"role": "user", "content": user_text}], add_generation_prompt=True,
-                enable_thinking=False)
-        if self.architecture.chat_prompt is not None:
-            return self.architecture.chat_prompt(user_text)
-        return user_text
+        """``user_text`` as a single user turn, ready to tokenize: by the folder's chat
+        template, else the architecture's (engine/text.py)."""
+        return text.chat_prompt(self.folder, self.architecture, user_text)
 
     # ------------------------------------------------------------------
     def generate(self, prompts: str | AbcSequence[str] | None = None,
                  sampling_params: SamplingParams | AbcSequence[SamplingParams] | None = None, *,
                  prompt_token_ids: AbcSequence[AbcSequence[int]] | None = None,
-                 use_tqdm: bool = False) -> list[RequestOutput]:
+                 use_tqdm: bool = True) -> list[RequestOutput]:
         """One completion per prompt, in input order
         (interface of reference: src/tokamak/engine/llm.py:265-334)."""
         if (prompts is None) == (prompt_token_ids is None):

@@ -102,23 +102,52 @@ class LayeredModel:
         if self.plan.tie_word_embeddings:
             self.head.tie(self.embedding)
 
+    # -- what the parts ask of a step ------------------------------------------
+    def step_planners(self) -> list:
+        """The parts' planners of work lists, one per name, in the order first met."""
+        found: dict[str, object] = {}
+        for part in self._all_parts():
+            planner = part.step_planner()
+            if planner is not None:
+                if not planner.name:
+                    raise ValueError(f"{type(part).__name__}'s step planner has no name")
+                found.setdefault(planner.name, planner)
+        return list(found.values())
+
+    def check_page_size(self, page_size: int) -> None:
+        for part in self._all_parts():
+            part.check_page_size(page_size)
+
     # -- cache ---------------------------------------------------------------
-    def _mixer_of(self, call):
-        return self.blocks[call.layer].mixer
+    def _mixers_of(self, call):
+        """(mixer, cache slot) pairs of a layer call."""
+        mixers = list(self.blocks[call.layer].mixers.values())
+        if mixers and len(call.slots) != len(mixers):
+            raise ValueError(f"layer {call.layer} has {len(mixers)} mixer(s) but its call brings "
+                             f"{len(call.slots)} cache slot(s)")
+        return list(zip(mixers, call.slots))
+
+    def _store_of(self, call, storage):
+        """What the block of a call receives as ``store``: its mixer's slot, or with several
+        mixers a dict of slots by their roles."""
+        block = self.blocks[call.layer]
+        if len(block.mixers) <= 1:
+            return storage.slot(call.slots[0])
+        return {role: storage.slot(slot) for role, slot in zip(block.mixers, call.slots)}
 
     def cache_layout(self) -> tuple[list[CacheGroupSpec], dict[int, SlotLayout]]:
         """Cache groups (slots that share a retention rule) and each slot's layout."""
         requests: dict[int, CacheRequest] = {}
         for call in self.plan.order:
-            mixer = self._mixer_of(call)
-            if not call.writes_cache or mixer is None:
+            if not call.writes_cache:
                 continue
-            req = mixer.cache_request()
-            if req is None:
-                continue
-            if call.cache in requests and requests[call.cache] != req:
-                raise ValueError(f"cache slot {call.cache} is written with two different layouts")
-            requests[call.cache] = req
+            for mixer, slot in self._mixers_of(call):
+                req = mixer.cache_request()
+                if req is None:
+                    continue
+                if slot in requests and requests[slot] != req:
+                    raise ValueError(f"cache slot {slot} is written with two different layouts")
+                requests[slot] = req
         windows: list[int | None] = []
         for req in requests.values():
             if req.window not in windows:
@@ -139,12 +168,12 @@ class LayeredModel:
         """Cache slot -> arrays of the fixed-size per-request state its mixer keeps."""
         out: dict[int, dict[str, StateArray]] = {}
         for call in self.plan.order:
-            mixer = self._mixer_of(call)
-            if mixer is None or not call.writes_cache:
+            if not call.writes_cache:
                 continue
-            request = mixer.state_request()
-            if request:
-                out[call.cache] = dict(request)
+            for mixer, slot in self._mixers_of(call):
+                request = mixer.state_request()
+                if request:
+                    out[slot] = dict(request)
         return out
 
     # -- compute -------------------------------------------------------------
@@ -156,7 +185,7 @@ class LayeredModel:
         recordings: dict[tuple, layer_replay.LayerRecording | None] = {}
         for at, call in enumerate(order):
             block = self.blocks[call.layer]
-            store = storage.slot(call.cache)
+            store = self._store_of(call, storage)
             kwargs = {}
             if block.fuses_residual:
                 # the norm that reads the stream after this block: its last product may prepare for it
@@ -168,11 +197,12 @@ class LayeredModel:
                 continue
             then = kwargs.get("then")
             held = self._own_tensors.get((call.layer, call.cache))
-            if held is None or held[0] is not store:      # (another cache storage: its arrays lie elsewhere)
-                held = self._own_tensors[(call.layer, call.cache)] = (store, layer_replay.own_tensors(block, store))
+            if held is None or held[0] is not storage:      # (another cache storage: its arrays lie elsewhere)
+                held = self._own_tensors[(call.layer, call.cache)] = (storage, layer_replay.own_tensors(block, store))
             own = held[1]
             tensors = layer_replay.call_tensors(own, pending, then)
-            key = (self._layer_kind[call.layer], call.writes_cache, store.group, type(then), layer_replay.pending_kind(pending))
+            key = (self._layer_kind[call.layer], call.writes_cache, layer_replay.store_groups(store), type(then),
+                   layer_replay.pending_kind(pending))
             if key in recordings:
                 recorded = recordings[key]
                 if recorded is not None:

@@ -18,7 +18,7 @@ from tokamak_amd.cache.manager import CacheManager, OutOfSlotsError
 from tokamak_amd.cache.pages import OutOfPagesError
 from tokamak_amd.config.registry import load_model_description
 from tokamak_amd.engine.batch import StepBatch, StepSpan, batch_from_device, pack_batch
-from tokamak_amd.engine.decode_graph import DecodeGraph, pow2_at_least, quarter_octave_at_least
+from tokamak_amd.engine.decode_graph import DecodeGraph, pow2_at_least
 from tokamak_amd.engine.model import LayeredModel
 from tokamak_amd.engine.storage import CacheStorage
 from tokamak_amd.kernels import ops
@@ -77,11 +77,13 @@ class ModelRunner:
         self.device = torch.device(device)
         if self.device.type != "cuda" or not torch.cuda.is_available():
             raise RuntimeError("tokamak_amd runs on a GPU only; no GPU is visible")
-        if page_size < 8 or page_size % 8:
-            raise ValueError(f"page_size must be a multiple of 8, got {page_size}")
+        if page_size < 1:
+            raise ValueError(f"page_size must be >= 1, got {page_size}")
         self.plan = plan
         self.page_size = page_size
         self.model = LayeredModel(plan, dtype=self.dtype, device=self.device)
+        self.model.check_page_size(page_size)      # what the parts' kernels take
+        self._planners = self.model.step_planners()
         self.num_tensors = load_weights(self.model, source, dtype=self.dtype, device=self.device)
         groups, layouts = self.model.cache_layout()
         self.num_groups = len(groups)
@@ -228,7 +230,7 @@ class ModelRunner:
 
     def prepare(self, entries: list[StepEntry]) -> StepBatch:
         """Reserve what the entries need and build the step's descriptor."""
-        packed = pack_batch(self._spans(entries), self.num_groups)
+        packed = pack_batch(self._spans(entries), self.num_groups, self._planners)
         host = torch.from_numpy(packed.buf)
         batch = batch_from_device(packed, host.pin_memory().to(self.device, non_blocking=True))
         self._feed(batch)
@@ -241,10 +243,9 @@ class ModelRunner:
         for s in spans:
             s.want = [0]            # the captured step computes every row's logits
         widths = [pow2_at_least(max(len(s.tables[g]) for s in spans), 16) for g in range(self.num_groups)]
-        packed = pack_batch(spans, self.num_groups, fixed_widths=widths)
-        # the longest context fixes how the attention kernel splits the keys: bucketed, four an octave
-        packed.max_decode_len = quarter_octave_at_least(packed.max_decode_len, 256)
-        key = (len(spans), tuple(widths), packed.max_decode_len)
+        # the parts' facts of the step (rounded as their planners ask) are part of the shape
+        packed = pack_batch(spans, self.num_groups, self._planners, fixed_widths=widths, bucket=True)
+        key = (len(spans), tuple(widths), packed.shape_key())
         graph = self._graphs.pop(key, None)
         if graph is None:
             # a new shape: this step runs eagerly, once, and is recorded for the next ones

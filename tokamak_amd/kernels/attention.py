@@ -1,10 +1,15 @@
-"""Dispatch of paged attention to the kernel that fits the shape."""
+"""Dispatch of paged attention to the kernel that fits the shape, and the work lists
+those kernels read: how a step's spans are cut into single tokens and tiles."""
 
 from __future__ import annotations
 
 import torch
 
 from tokamak_amd.kernels import ops
+from tokamak_amd.engine.batch import StepPlanner
+
+TILE_TOKENS = 16   # tokens per attention tile of a prompt portion (csrc/attention_generic.hip: kTileTokens)
+WIDE_TOKENS = 32   # and per tile of the wide matrix-core kernel
 
 MFMA_HEAD_DIMS = (64, 128)
 DECODE_WAVES = 16           # waves of a decode block (csrc/attention_mfma.hip: kDecodeWaves)
@@ -17,6 +22,91 @@ DENSE_TILES_FROM = 2048         # every tiled span starts at least this deep: th
 WIDE_FROM_KEYS = 4096           # longest context from which the 32-token tiles of the wide kernel pay (+15-20 %;
                                 # for shorter walks the narrow one's smaller tiles balance better)
 WIDE_FROM_TOKENS = 20           # ... if a 32-token tile holds at least this many tokens on average
+
+
+def quarter_octave_at_least(n: int, floor: int) -> int:
+    """The smallest of floor, 1.25 floor, 1.5 floor, 1.75 floor, 2 floor, 2.5 floor, ...
+    that is >= n: four buckets an octave, so a bucket overshoots by a quarter at most."""
+    v = floor
+    while 2 * v < n:
+        v *= 2
+    if n <= v:
+        return v
+    step = v // 4
+    return v + -(-(n - v) // step) * step
+
+
+class AttentionWork(StepPlanner):
+    """The attention kernels' cut of a step: spans of one token run alone (``single``: their
+    token rows), longer spans are cut into tiles of up to 16 consecutive tokens
+    (``tile_first``, ``tile_count``) and, for the wide kernel, of up to 32 (``wide_first``,
+    ``wide_count``).  Facts: how many of each, the tokens in tiled spans, the longest
+    context among the single tokens (it fixes how their keys are split), the longest
+    among the tiled spans, and the shortest cached length among them."""
+
+    name = "attention"
+
+    def lists(self, q_lens, ctx_lens):
+        single, tiles, wide = [], [], []
+        at = 0
+        for q in q_lens:
+            if q == 1:
+                single.append(at)
+            else:
+                tiles.extend((at + t, min(TILE_TOKENS, q - t)) for t in range(0, q, TILE_TOKENS))
+                wide.extend((at + t, min(WIDE_TOKENS, q - t)) for t in range(0, q, WIDE_TOKENS))
+            at += q
+        arrays = {"single": single, "tile_first": [t[0] for t in tiles], "tile_count": [t[1] for t in tiles],
+                  "wide_first": [t[0] for t in wide], "wide_count": [t[1] for t in wide]}
+        tiled = [(q, c) for q, c in zip(q_lens, ctx_lens) if q > 1]
+        facts = {
+            "num_single": len(single), "num_tiles": len(tiles), "num_wide": len(wide),
+            "num_tile_tokens": sum(q for q, _ in tiled),
+            "max_single_len": max((c + 1 for q, c in zip(q_lens, ctx_lens) if q == 1), default=0),
+            "max_tile_len": max((c + q for q, c in tiled), default=0),
+            "min_tile_ctx": min((c for _, c in tiled), default=0),
+        }
+        return arrays, facts
+
+    def bucket(self, facts):
+        # the longest context fixes how the decode kernel splits the keys: four buckets an octave
+        facts["max_single_len"] = quarter_octave_at_least(facts["max_single_len"], 256)
+        return facts
+
+
+ATTENTION_WORK = AttentionWork()
+
+
+class _Work:
+    """The attention planner's lists and facts of a step, by attribute."""
+
+    def __init__(self, batch) -> None:
+        lists, facts = batch.lists, batch.facts
+        try:
+            self.single = lists["attention.single"]
+            self.tile_first, self.tile_count = lists["attention.tile_first"], lists["attention.tile_count"]
+            self.wide_first, self.wide_count = lists["attention.wide_first"], lists["attention.wide_count"]
+            self.num_single, self.num_tiles = facts["attention.num_single"], facts["attention.num_tiles"]
+            self.num_wide, self.num_tile_tokens = facts["attention.num_wide"], facts["attention.num_tile_tokens"]
+            self.max_single_len, self.max_tile_len = facts["attention.max_single_len"], facts["attention.max_tile_len"]
+            self.min_tile_ctx = facts["attention.min_tile_ctx"]
+        except KeyError as missing:
+            raise ops.KernelError(f"the step's descriptor lacks {missing}: it was packed without the attention "
+                                  f"part's planner (kernels.attention.ATTENTION_WORK)") from None
+
+
+def work_of(batch) -> _Work:
+    work = batch.memo.get("attention.work")
+    if work is None:
+        work = batch.memo["attention.work"] = _Work(batch)
+    return work
+
+
+def check_page_size(page_size: int) -> None:
+    """Pages hold a multiple of 8 tokens: the value layout groups tokens in quads of four,
+    the key layout in pieces of 8 numbers, and the generic kernel walks pages 8 keys at a time."""
+    if page_size < 8 or page_size % 8:
+        raise ValueError(f"page_size must be a multiple of 8 for the attention kernels, got {page_size}")
 
 
 def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
@@ -66,7 +156,8 @@ def tile_split(num_tiles: int, blocks_per_tile: int, max_len: int) -> tuple[int,
 
 def fused_decode_fits(dtype, head_dim, page_size, group, window, rotary_dim, batch) -> bool:
     """A step of decode tokens only, at shapes the one-kernel form takes."""
-    return (batch.num_tiles == 0 and batch.num_decode == batch.num_tokens and batch.num_decode > 0
+    work = work_of(batch)
+    return (work.num_tiles == 0 and work.num_single == batch.num_tokens and work.num_single > 0
             and mfma_fits(dtype, head_dim, page_size, group, window) and group <= ops.FUSED_DECODE_MAX_GROUP
             and rotary_dim in (0, head_dim))
 
@@ -75,14 +166,15 @@ def decode_attention_fused(qkv, q_weight, k_weight, cos, sin, k_cache, v_cache, 
                            num_heads, num_kv_heads, head_dim, rotary_dim, page_size, eps, scale, store) -> bool:
     """q/k norm, rotation, cache write and attention of a decode-only step in one kernel
     (plus the merge of the splits, if a token's keys are split)."""
-    split, nsplit = decode_split(batch.num_decode, num_kv_heads, batch.max_decode_len)
+    work = work_of(batch)
+    split, nsplit = decode_split(work.num_single, num_kv_heads, work.max_single_len)
     if ops._profile is not None:
         keys = sum(c + 1 for c in batch.ctx_lens)
-        ops._note(f"decode {batch.num_decode} tokens, fused", keys * 2 * num_kv_heads * head_dim * 2,
+        ops._note(f"decode {work.num_single} tokens, fused", keys * 2 * num_kv_heads * head_dim * 2,
                   keys * 4.0 * num_heads * head_dim)
     return ops.attention_decode_fused(
         qkv, q_weight, k_weight, cos, sin, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token,
-        batch.decode_tokens, batch.num_decode, out, num_heads=num_heads, num_kv_heads=num_kv_heads,
+        work.single, work.num_single, out, num_heads=num_heads, num_kv_heads=num_kv_heads,
         head_dim=head_dim, rotary_dim=rotary_dim, page_size=page_size, eps=eps, scale=scale, store=store,
         split_keys=split, num_splits=nsplit)
 
@@ -95,8 +187,10 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     bfloat16 with head size 64 or 128: the MFMA kernel, once over the single
     (decode) tokens with their context split, once over 16-token tiles of the
     prompt portions (their keys split too when the tiles are few and the context
-    long).  Everything else: the generic float32-arithmetic kernel.
+    long).  Everything else, and whatever the MFMA library does not instantiate:
+    the generic float32-arithmetic kernel.
     """
+    work = work_of(batch)
     profiling = ops._profile is not None
     if profiling:
         # keys each query sees; the cache bytes of a request are read once per kv head
@@ -106,35 +200,10 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
         kv_token_bytes = 2 * num_kv_heads * head_dim * q.element_size()
         flops_per_pair = 4.0 * num_heads * head_dim
     if mfma_fits(q.dtype, head_dim, page_size, num_heads // num_kv_heads, window):
-        common = dict(num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
-                      page_size=page_size, scale=scale)
-        if batch.num_decode:
-            split, nsplit = decode_split(batch.num_decode, num_kv_heads, batch.max_decode_len)
-            if profiling:
-                ops._note(f"decode {batch.num_decode} tokens", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
-            ops.attention_mfma("heads", q, k_cache, v_cache, block_tables, batch.positions,
-                               batch.req_of_token, batch.decode_tokens, None, batch.num_decode, out,
-                               split_keys=split, num_splits=nsplit, **common)
-        if batch.num_tiles:
-            group = num_heads // num_kv_heads
-            per_tile = num_kv_heads * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
-            split, nsplit = tile_split(batch.num_tiles, per_tile, batch.max_tile_len)
-            if (nsplit == 1 and batch.max_tile_len >= WIDE_FROM_KEYS
-                    and batch.num_tile_tokens >= WIDE_FROM_TOKENS * batch.num_wide):
-                # long walks over the keys, tiles of 32 tokens mostly full: the wide kernel
-                if profiling:
-                    ops._note(f"portions {batch.num_wide} wide tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
-                ops.attention_mfma("tokens_wide", q, k_cache, v_cache, block_tables, batch.positions,
-                                   batch.req_of_token, batch.wide_first, batch.wide_count, batch.num_wide,
-                                   out, **common)
-                return
-            dense = nsplit == 1 and batch.min_tile_ctx >= DENSE_TILES_FROM
-            if profiling:
-                ops._note(f"portions {batch.num_tiles} tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
-            ops.attention_mfma("tokens_dense" if dense else "tokens", q, k_cache, v_cache, block_tables, batch.positions,
-                               batch.req_of_token, batch.tile_first, batch.tile_count, batch.num_tiles,
-                               out, split_keys=split, num_splits=nsplit, **common)
-        return
+        if _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, num_heads=num_heads,
+                                 num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size, scale=scale,
+                                 note=(decode_keys, tile_keys, tile_pairs, kv_token_bytes, flops_per_pair) if profiling else None):
+            return
     if profiling:
         ops._note(f"{batch.num_tokens} tokens", (decode_keys + tile_keys) * kv_token_bytes,
                   (decode_keys + tile_pairs) * flops_per_pair)
@@ -142,4 +211,42 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
         q, k_cache, v_cache, block_tables, batch.positions, batch.req_of_token, out,
         num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
         scale=scale, window=window,
-        tiles=(batch.tile_first, batch.tile_count, batch.num_tiles, batch.decode_tokens, batch.num_decode))
+        tiles=(work.tile_first, work.tile_count, work.num_tiles, work.single, work.num_single))
+
+
+def _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, *, num_heads, num_kv_heads,
+                          head_dim, page_size, scale, note) -> bool:
+    """The matrix-core kernels over the step's single tokens and tiles.  False if the
+    library has no instance for the shape: nothing of ``out`` counts then, and the caller
+    runs the generic kernel over the whole step."""
+    common = dict(num_heads=num_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
+                  page_size=page_size, scale=scale)
+    if note is not None:
+        decode_keys, tile_keys, tile_pairs, kv_token_bytes, flops_per_pair = note
+    if work.num_single:
+        split, nsplit = decode_split(work.num_single, num_kv_heads, work.max_single_len)
+        if note is not None:
+            ops._note(f"decode {work.num_single} tokens", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
+        if not ops.attention_mfma("heads", q, k_cache, v_cache, block_tables, batch.positions,
+                                  batch.req_of_token, work.single, None, work.num_single, out,
+                                  split_keys=split, num_splits=nsplit, **common):
+            return False
+    if work.num_tiles:
+        group = num_heads // num_kv_heads
+        per_tile = num_kv_heads * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
+        split, nsplit = tile_split(work.num_tiles, per_tile, work.max_tile_len)
+        if (nsplit == 1 and work.max_tile_len >= WIDE_FROM_KEYS
+                and work.num_tile_tokens >= WIDE_FROM_TOKENS * work.num_wide):
+            # long walks over the keys, tiles of 32 tokens mostly full: the wide kernel
+            if note is not None:
+                ops._note(f"portions {work.num_wide} wide tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
+            return ops.attention_mfma("tokens_wide", q, k_cache, v_cache, block_tables, batch.positions,
+                                      batch.req_of_token, work.wide_first, work.wide_count, work.num_wide,
+                                      out, **common)
+        dense = nsplit == 1 and work.min_tile_ctx >= DENSE_TILES_FROM
+        if note is not None:
+            ops._note(f"portions {work.num_tiles} tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
+        return ops.attention_mfma("tokens_dense" if dense else "tokens", q, k_cache, v_cache, block_tables, batch.positions,
+                                  batch.req_of_token, work.tile_first, work.tile_count, work.num_tiles,
+                                  out, split_keys=split, num_splits=nsplit, **common)
+    return True

@@ -6,7 +6,8 @@ import torch
 
 from tokamak_amd.config.registry import register_part
 from tokamak_amd.kernels import ops
-from tokamak_amd.kernels.attention import decode_attention_fused, fused_decode_fits, paged_attention
+from tokamak_amd.kernels.attention import (ATTENTION_WORK, check_page_size, decode_attention_fused, fused_decode_fits,
+                                            paged_attention)
 from tokamak_amd.kernels.linear import linear
 from tokamak_amd.parts.base import CacheRequest, Fetch, Mixer, PositionData
 from tokamak_amd.weights.spec import TensorSpec
@@ -69,6 +70,16 @@ class GQAAttention(Mixer):
     def cache_request(self) -> CacheRequest:
         width = self.num_kv_heads * self.head_dim
         return CacheRequest.of(window=self.window, k=width, v=width)
+
+    def step_planner(self):
+        return ATTENTION_WORK
+
+    def check_page_size(self, page_size: int) -> None:
+        check_page_size(page_size)
+
+    def pair_flops(self) -> float:
+        # q.k and p.v: two multiply-adds per head and head element
+        return 4.0 * self.num_heads * self.head_dim
 
     def forward(self, h, batch, store, writes_cache: bool = True,
                 position: PositionData | None = None, add_into=None):

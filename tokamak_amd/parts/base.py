@@ -22,6 +22,10 @@ prefix, and everything about the running batch arrives in the ``StepBatch``.
 * ``FeedForward.forward(h, batch)``: token-wise map [N, H] -> [N, H].
 * ``Block.forward(resid, pending, ...)``: the arrangement of a layer's parts,
   which it receives as a dict by role.
+
+A part whose kernels want the step cut into work of their own shape (tiles of a
+portion's tokens, chunks of a scan) declares a ``StepPlanner``; what page sizes its
+kernels take it says in ``check_page_size``.  The engine asks; it knows neither.
 """
 
 from __future__ import annotations
@@ -31,6 +35,7 @@ from typing import Callable
 
 import torch
 
+from tokamak_amd.engine.batch import StepPlanner  # noqa: F401  (part of the parts' interface)
 from tokamak_amd.weights.spec import TensorSpec
 
 Fetch = Callable[[str], "torch.Tensor | None"]
@@ -72,6 +77,14 @@ class Part:
 
     def bind(self, prefix: str, fetch: Fetch) -> None:
         pass
+
+    def step_planner(self) -> StepPlanner | None:
+        """The planner of the work lists this part's kernels read, or None."""
+        return None
+
+    def check_page_size(self, page_size: int) -> None:
+        """Raise ``ValueError`` if the part's kernels cannot work with cache pages of
+        ``page_size`` tokens."""
 
 
 @dataclass(frozen=True)
@@ -134,6 +147,10 @@ class Embedding(Part):
     def forward(self, batch) -> torch.Tensor:
         raise NotImplementedError
 
+    def tied_matrix(self) -> torch.Tensor:
+        """The [vocab, dim] matrix a head shares with this embedding when the two are tied."""
+        raise NotImplementedError(f"{type(self).__name__} has no matrix to tie a head to")
+
 
 class Head(Part):
     def forward(self, h: torch.Tensor) -> torch.Tensor:
@@ -165,6 +182,12 @@ class Mixer(Part):
         a request is admitted."""
         return None
 
+    def pair_flops(self) -> float:
+        """Floating-point operations per (query token, visible earlier token) pair of one
+        call, for the measurement's count of a step's work; 0 for a mixer whose work does
+        not grow with the context."""
+        return 0.0
+
     def forward(self, h: torch.Tensor, batch, store, writes_cache: bool = True,
                 position: PositionData | None = None) -> torch.Tensor:
         raise NotImplementedError
@@ -179,8 +202,11 @@ class Block:
     """Arrangement of one layer's parts.
 
     ``roles``: names of the parts it needs; ``optional``: of those it can do
-    without.  ``parts`` holds the built parts by role.  At most one
-    part of a block is a mixer: it owns the cache slot of the layer call.
+    without.  ``parts`` holds the built parts by role.  ``mixers`` holds those that are
+    mixers, by role, in the order the plan names them: a layer call brings one cache slot
+    for each.  With one mixer (or none) ``forward`` receives that slot's ``SlotStore`` as
+    ``store`` and ``mixer`` names it; with several, ``store`` is a dict of ``SlotStore`` by
+    the mixers' roles.
     """
 
     roles: tuple[str, ...] = ()
@@ -195,11 +221,9 @@ class Block:
         if missing or unknown:
             raise ValueError(f"{type(self).__name__} needs parts {sorted(self.roles)} "
                              f"(optional: {sorted(self.optional)}); missing {missing}, unknown {unknown}")
-        mixers = [p for p in parts.values() if isinstance(p, Mixer)]
-        if len(mixers) > 1:
-            raise ValueError(f"{type(self).__name__}: a layer has one cache slot, so at most one mixer")
         self.parts = dict(parts)
-        self.mixer: Mixer | None = mixers[0] if mixers else None
+        self.mixers: dict[str, Mixer] = {role: p for role, p in parts.items() if isinstance(p, Mixer)}
+        self.mixer: Mixer | None = next(iter(self.mixers.values())) if len(self.mixers) == 1 else None
         # a block's launches are replayed only if the block itself says so and all its parts do
         self.replayable = bool(type(self).replays_parts) and all(p.replayable for p in parts.values())
 

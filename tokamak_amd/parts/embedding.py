@@ -28,6 +28,9 @@ class TokenEmbedding(Embedding):
     def bind(self, prefix: str, fetch: Fetch) -> None:
         self.weight = fetch(prefix + "weight")
 
+    def tied_matrix(self) -> torch.Tensor:
+        return self.weight
+
     def forward(self, batch) -> torch.Tensor:
         resid = torch.empty((batch.num_tokens, self.dim), dtype=torch.float32, device=self.device)
         ops.embed_gather(self.weight, batch.token_ids, resid)
@@ -54,8 +57,12 @@ class LinearHead(Head):
         if not self.tied:
             self.weight = fetch(prefix + "weight")
 
-    def tie(self, embedding: TokenEmbedding) -> None:
-        self.weight = embedding.weight
+    def tie(self, embedding: Embedding) -> None:
+        weight = embedding.tied_matrix()
+        if tuple(weight.shape) != (self.vocab_size, self.dim):
+            raise ValueError(f"a tied head of {(self.vocab_size, self.dim)} cannot share an embedding "
+                             f"matrix of {tuple(weight.shape)}")
+        self.weight = weight
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return linear(h, self.weight, out_dtype=torch.float32)

@@ -46,11 +46,7 @@ def validate(expected: Mapping[str, TensorSpec], found: Mapping[str, tuple]) -> 
 
 
 def target_dtype(spec: TensorSpec, stored: torch.dtype, compute_dtype: torch.dtype) -> torch.dtype:
-    if spec.role == "table":
-        return torch.int32
-    if spec.role == "vector":
-        return torch.float32
-    return compute_dtype
+    return {"int32": torch.int32, "float32": torch.float32, "stored": stored, "compute": compute_dtype}[spec.holding]
 
 
 def load_weights(model, source, *, dtype: torch.dtype, device: str | torch.device) -> int:
