@@ -103,6 +103,15 @@ def measure_peaks() -> dict:
 # ---------------------------------------------------------------------------
 # the model and what a step has to move and compute, from the plan
 # ---------------------------------------------------------------------------
+def make_llm(cfg, dtype, pool_tokens, max_requests, max_seq_len, seed=0):
+    """The engine's entry point over seeded random weights of ``cfg``'s shape, drawn on the GPU."""
+    from tokamak_amd import LLM
+
+    return LLM(cfg, seed=seed, random_weights_on_gpu=True, dtype=dtype, block_size=PAGE_SIZE,
+               kv_pool_tokens=pool_tokens, max_batch_size=max_requests, max_seq_len=max_seq_len,
+               max_num_batched_tokens=PREFILL_TOKENS)
+
+
 def make_runner(arch, cfg, dtype, pool_tokens, max_requests, seed=0):
     import torch
 
@@ -198,54 +207,51 @@ def time_prefill(runner, vocab, repeats=5):
     return statistics.median(times[2:])
 
 
-def decode_pass(runner, vocab, batch, prompt_tokens, steps, seed):
+def decode_pass(llm, vocab, batch, prompt_tokens, steps, seed):
     """``batch`` fresh requests with ``prompt_tokens``-token prompts, then ``steps`` greedy
-    decode steps of the whole batch; seconds for those steps."""
+    decode steps of the whole batch; seconds for those steps.
+
+    The timed steps are run by the generation loop itself (``LLM.run``: the scheduler plans
+    every step, each is launched before the tokens of the step before it are read and takes
+    them from the sampler's output on the GPU, and the host reads every step's tokens one
+    step late).  Before that every prompt runs alone, in portions, and its first token is
+    read at once, so that all requests enter the timed steps with the same context."""
     import torch
 
-    from tokamak_amd.engine.runner import StepEntry
-    from tokamak_amd.sampling.sampler import greedy_tokens
+    from tokamak_amd import SamplingParams
+    from tokamak_amd.engine.scheduler import Scheduler, Span, StepPlan
 
-    last = []
+    params = SamplingParams(temperature=0.0, max_new_tokens=steps + 1, ignore_eos=True)
+    scheduler = Scheduler(llm.runner.manager, batch, max(batch, llm.max_num_batched_tokens))
+    requests = []
     for r in range(batch):
-        logits = fill(runner, r, random_prompt(vocab, prompt_tokens, seed * 1000 + r))
-        last.append(int(greedy_tokens(logits).item()))
-    # The generation loop of LLM.generate: every step is launched before the tokens of the
-    # step before it are read (it takes them from the sampler's output on the GPU), and the
-    # host reads every step's tokens, one step late.
-    pinned = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
-    copied = [torch.cuda.Event(), torch.cuda.Event()]
-    generated = []
+        request = llm.new_request(r, random_prompt(vocab, prompt_tokens, seed * 1000 + r), params)
+        for at in range(0, prompt_tokens, PREFILL_TOKENS):
+            n = min(PREFILL_TOKENS, prompt_tokens - at)
+            flight = llm.launch(StepPlan([Span(request, at, n, at + n == prompt_tokens)]))
+            if flight is not None:
+                llm.read(flight)
+        scheduler.running.append(request)
+        requests.append(request)
+    assert all(r.num_generated == 1 and r.decoding for r in requests)
+    before = llm.num_steps
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(steps):
-        if i == 0:
-            entries = [StepEntry(r, [last[r]], [0]) for r in range(batch)]
-        else:
-            entries = [StepEntry(r, [0], [0], feed=r) for r in range(batch)]
-        logits = runner.step(entries)
-        drawn = greedy_tokens(logits, out=runner.sampled)
-        pinned[i % 2].copy_(drawn, non_blocking=True)
-        copied[i % 2].record()
-        if i > 0:
-            copied[(i - 1) % 2].synchronize()
-            generated.append(pinned[(i - 1) % 2].tolist())
-    copied[(steps - 1) % 2].synchronize()
-    generated.append(pinned[(steps - 1) % 2].tolist())
+    llm.run(scheduler)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    assert len(generated) == steps and all(len(g) == batch for g in generated)
-    for r in range(batch):
-        runner.end(r)
+    assert llm.num_steps - before == steps, f"{llm.num_steps - before} steps ran, {steps} were to be timed"
+    assert all(r.finished and r.num_generated == steps + 1 for r in requests)
+    llm.runner.end_all()
     return elapsed
 
 
-def time_decode(runner, vocab, batch, prompt_tokens, steps, warmup, repeats):
+def time_decode(llm, vocab, batch, prompt_tokens, steps, warmup, repeats):
     """Median seconds per step over ``repeats`` timed passes, after one untimed pass of
     ``warmup`` steps; and every pass's figure."""
     if warmup > 0:
-        decode_pass(runner, vocab, batch, prompt_tokens, warmup, seed=0)
-    runs = [decode_pass(runner, vocab, batch, prompt_tokens, steps, seed=1 + i) / steps for i in range(repeats)]
+        decode_pass(llm, vocab, batch, prompt_tokens, warmup, seed=0)
+    runs = [decode_pass(llm, vocab, batch, prompt_tokens, steps, seed=1 + i) / steps for i in range(repeats)]
     return statistics.median(runs), runs
 
 
@@ -630,18 +636,20 @@ def main() -> int:
     peaks = None if args.no_peaks else measure_peaks()
     ops.set_library_tuning(not args.no_tune)
     pool = max_batch * (-(-(final_context + 1) // PAGE_SIZE) * PAGE_SIZE + PAGE_SIZE)
-    runner = make_runner(arch, cfg, args.dtype, max(pool, PREFILL_TOKENS + PAGE_SIZE), max_batch)
+    longest = max(final_context + 1, PREFILL_TOKENS + 1)
+    llm = make_llm(cfg, args.dtype, max(pool, PREFILL_TOKENS + PAGE_SIZE, longest), max_batch, longest)
+    runner = llm.runner
     cost = StepCost(runner)
     vocab = runner.plan.vocab_size
 
     prefill_s = time_prefill(runner, vocab) if args.phase in ("all", "prefill") else None
     step_s = runs = None
     if args.phase in ("all", "decode"):
-        step_s, runs = time_decode(runner, vocab, args.batch, prompt_tokens, args.steps, args.warmup, args.repeats)
+        step_s, runs = time_decode(llm, vocab, args.batch, prompt_tokens, args.steps, args.warmup, args.repeats)
     points = {}
     if want_points:
         for b in (1, 64):
-            s, _ = time_decode(runner, vocab, b, prompt_tokens, args.steps, min(args.warmup, 4), args.repeats)
+            s, _ = time_decode(llm, vocab, b, prompt_tokens, args.steps, min(args.warmup, 4), args.repeats)
             keys = prompt_tokens + (args.steps + 1) / 2.0
             points[f"decode_b{b}"] = round(b / s, 1)
             points[f"decode_b{b}_hbm_frac"] = round(cost.decode_bytes(b, keys) / s / HBM_PEAK, 4)

@@ -187,20 +187,12 @@ class LLM:
                 raise ValueError(f"Got {len(per_request)} SamplingParams for {len(id_lists)} prompts")
 
         now = time.perf_counter()
-        requests = []
-        for rid, (ids, params) in enumerate(zip(id_lists, per_request)):
-            seed = params.seed if params.seed is not None else random.getrandbits(62)
-            request = Request.from_prompt(rid, ids, params, seed)
-            request.arrived_at = now
-            self._check_request(request)
-            requests.append(request)
-
+        requests = [self.new_request(rid, ids, params, now)
+                    for rid, (ids, params) in enumerate(zip(id_lists, per_request))]
         scheduler = Scheduler(self.runner.manager, self.max_batch_size, self.max_num_batched_tokens,
                               self.prefill_chunk)
         for request in requests:
             scheduler.submit(request)
-        for request in requests:
-            request.context_limit = self._context_limit(request)
         # a bar over finished requests, as the reference shows (src/tokamak/engine/llm.py:299)
         self._progress = None
         if use_tqdm:
@@ -210,21 +202,7 @@ class LLM:
             except ImportError:
                 pass
         try:
-            # One step ahead: a step is planned and launched while the one before it runs; the
-            # tokens that one sampled are read (and stop rules applied) meanwhile.  A decoding
-            # request's next step takes its token from the sampler's output on the GPU.
-            in_flight = None
-            while scheduler.busy or in_flight is not None:
-                plan = scheduler.plan() if scheduler.busy else None
-                launched = self._launch(plan) if plan is not None else None
-                if in_flight is not None:
-                    self._read(in_flight)
-                elif plan is None or not plan.spans:
-                    raise RuntimeError("the scheduler has unfinished requests but plans no step")
-                in_flight = launched
-                if in_flight is not None and not self.steps_ahead:
-                    self._read(in_flight)
-                    in_flight = None
+            self.run(scheduler)
         finally:
             if self._progress is not None:
                 self.last_progress = f"{self._progress.n}/{self._progress.total}"
@@ -236,7 +214,38 @@ class LLM:
                 self.runner.manager.free(request.rid)
         return [self._output(request, text) for request, text in zip(requests, texts)]
 
-    def _launch(self, plan: StepPlan) -> _InFlight | None:
+    def new_request(self, rid: int, ids: list[int], params: SamplingParams, now: float | None = None) -> Request:
+        """A checked request for ``ids``, with its seed and its limit of tokens."""
+        seed = params.seed if params.seed is not None else random.getrandbits(62)
+        request = Request.from_prompt(rid, ids, params, seed)
+        request.arrived_at = time.perf_counter() if now is None else now
+        self._check_request(request)
+        request.context_limit = self._context_limit(request)
+        return request
+
+    def run(self, scheduler: Scheduler) -> None:
+        """The step loop: until the scheduler has nothing left, plan a step, launch it, and
+        read the tokens of the step before it.
+
+        One step ahead: a step is planned and launched while the one before it runs; the
+        tokens that one sampled are read (and stop rules applied) meanwhile.  A decoding
+        request's next step takes its token from the sampler's output on the GPU.  With
+        ``steps_ahead`` off every step's tokens are read before the next is planned.
+        ``generate`` runs this loop, and so does the benchmark's timed decoding."""
+        in_flight = None
+        while scheduler.busy or in_flight is not None:
+            plan = scheduler.plan() if scheduler.busy else None
+            launched = self.launch(plan) if plan is not None else None
+            if in_flight is not None:
+                self.read(in_flight)
+            elif plan is None or not plan.spans:
+                raise RuntimeError("the scheduler has unfinished requests but plans no step")
+            in_flight = launched
+            if in_flight is not None and not self.steps_ahead:
+                self.read(in_flight)
+                in_flight = None
+
+    def launch(self, plan: StepPlan) -> _InFlight | None:
         """Run the plan's step and draw its tokens, all without waiting for the GPU; None
         if the step samples nothing (or the plan is empty)."""
         for victim in plan.evicted:
@@ -274,7 +283,7 @@ class LLM:
         self._copied[turn].record()
         return _InFlight(sampling, host, self._copied[turn])
 
-    def _read(self, step: _InFlight) -> None:
+    def read(self, step: _InFlight) -> None:
         """Wait for a launched step's tokens and give them to their requests."""
         step.copied.synchronize()
         stamp = time.perf_counter()
