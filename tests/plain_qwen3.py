@@ -93,7 +93,8 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
     return x * cos + rotate_half(x) * sin
 
 
-def causal_gqa_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float) -> torch.Tensor:
+def causal_gqa_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+                         query_block: int | None = None) -> torch.Tensor:
     """Scores, mask, softmax, weighted values.
 
     q [T, nh, hd]; k, v [T, nkv, hd].  Query head a uses kv head a // G
@@ -102,24 +103,32 @@ def causal_gqa_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scal
     (src/tokamak/kernels/paged_attention.py:277), a query at position t sees
     positions c <= t (src/tokamak/model/step_context.py:93-96), explicit softmax
     as in tests/unit/test_paged_attention_kernel.py:42-50.
+
+    ``query_block``: for sequences whose [T, T] score matrix would not fit in memory, the
+    same arithmetic for ``query_block`` queries at a time against the keys up to the
+    block's last query (the keys behind it are masked anyway).
     """
     T, nh, hd = q.shape
     nkv = k.shape[1]
     group = nh // nkv
     out = torch.empty_like(q)
-    visible = torch.arange(T)[None, :] <= torch.arange(T)[:, None]
-    for a in range(nh):
-        kv = a // group
-        scores = (q[:, a, :] @ k[:, kv, :].T) * scale
-        scores = scores.masked_fill(~visible, float("-inf"))
-        scores = scores - scores.max(dim=-1, keepdim=True).values
-        probs = scores.exp()
-        probs = probs / probs.sum(dim=-1, keepdim=True)
-        out[:, a, :] = probs @ v[:, kv, :]
+    block = T if query_block is None else query_block
+    for first in range(0, T, block):
+        last = min(T, first + block)
+        visible = torch.arange(last)[None, :] <= torch.arange(first, last)[:, None]
+        for a in range(nh):
+            kv = a // group
+            scores = (q[first:last, a, :] @ k[:last, kv, :].T) * scale
+            scores = scores.masked_fill(~visible, float("-inf"))
+            scores = scores - scores.max(dim=-1, keepdim=True).values
+            probs = scores.exp()
+            probs = probs / probs.sum(dim=-1, keepdim=True)
+            out[first:last, a, :] = probs @ v[:last, kv, :]
     return out
 
 
-def attention_block(h: torch.Tensor, w: dict, prefix: str, s: dict, positions: torch.Tensor) -> torch.Tensor:
+def attention_block(h: torch.Tensor, w: dict, prefix: str, s: dict, positions: torch.Tensor,
+                    query_block: int | None = None) -> torch.Tensor:
     """src/tokamak/model/transformer.py:65-86: project, per-head q/k norm, rope, attend, o_proj."""
     T = h.shape[0]
     q = (h @ w[prefix + "q_proj.weight"].T).view(T, s["nh"], s["hd"])
@@ -131,7 +140,7 @@ def attention_block(h: torch.Tensor, w: dict, prefix: str, s: dict, positions: t
     cos, sin = rope_tables(positions, s["hd"], s["theta"])
     q = apply_rope(q, cos, sin)
     k = apply_rope(k, cos, sin)
-    o = causal_gqa_attention(q, k, v, s["hd"] ** -0.5)
+    o = causal_gqa_attention(q, k, v, s["hd"] ** -0.5, query_block)
     return o.reshape(T, s["nh"] * s["hd"]) @ w[prefix + "o_proj.weight"].T
 
 
@@ -147,33 +156,36 @@ def swiglu(h: torch.Tensor, w: dict, prefix: str) -> torch.Tensor:
     return (silu(gate) * up) @ w[prefix + "down_proj.weight"].T
 
 
-def decoder_layer(x: torch.Tensor, w: dict, i: int, s: dict, positions: torch.Tensor) -> torch.Tensor:
+def decoder_layer(x: torch.Tensor, w: dict, i: int, s: dict, positions: torch.Tensor,
+                  query_block: int | None = None) -> torch.Tensor:
     """src/tokamak/model/transformer.py:107-108: pre-norm residual block."""
     p = f"model.layers.{i}."
-    x = x + attention_block(rmsnorm(x, w[p + "input_layernorm.weight"], s["eps"]), w, p + "self_attn.", s, positions)
+    x = x + attention_block(rmsnorm(x, w[p + "input_layernorm.weight"], s["eps"]), w, p + "self_attn.", s, positions,
+                            query_block)
     x = x + swiglu(rmsnorm(x, w[p + "post_attention_layernorm.weight"], s["eps"]), w, p + "mlp.")
     return x
 
 
-def hidden_states(token_ids, cfg: dict, w: dict, start_position: int = 0) -> torch.Tensor:
+def hidden_states(token_ids, cfg: dict, w: dict, start_position: int = 0,
+                  query_block: int | None = None) -> torch.Tensor:
     """src/tokamak/model/transformer.py:138-144: embed, L layers, final norm."""
     s = sizes(cfg)
     ids = torch.as_tensor(token_ids, dtype=torch.long)
     positions = torch.arange(len(ids)) + start_position
     x = w["model.embed_tokens.weight"][ids]  # plain row gather (transformer.py:140)
     for i in range(s["L"]):
-        x = decoder_layer(x, w, i, s, positions)
+        x = decoder_layer(x, w, i, s, positions, query_block)
     return rmsnorm(x, w["model.norm.weight"], s["eps"])
 
 
-def logits(token_ids, cfg: dict, w: dict, start_position: int = 0) -> torch.Tensor:
+def logits(token_ids, cfg: dict, w: dict, start_position: int = 0, query_block: int | None = None) -> torch.Tensor:
     """Logits [T, V] at every position (src/tokamak/model/transformer.py:173-176).
 
     A tied model projects with the embedding matrix itself (transformer.py:155-156).
     """
     s = sizes(cfg)
     head = w["model.embed_tokens.weight"] if s["tied"] else w["lm_head.weight"]
-    return (hidden_states(token_ids, cfg, w, start_position) @ head.T).to(torch.float32)
+    return (hidden_states(token_ids, cfg, w, start_position, query_block) @ head.T).to(torch.float32)
 
 
 def greedy(token_ids, num_new: int, cfg: dict, w: dict) -> list[int]:

@@ -310,3 +310,34 @@ def test_sampler_vectors():
     assert int(p.argmax()) == int(logits.argmax()) and p.max() == 1.0
     p = plain.sampling_probs(logits, 0.5, 0, 1.0)
     torch.testing.assert_close(p, torch.softmax(logits.double() / 0.5, -1))
+
+
+def test_the_kernel_tests_own_helpers_agree_with_each_other():
+    """The page packing without a loop equals the token-by-token one (written from the
+    documented layout), and the blocked float64 attention equals the query-by-query one."""
+    from kernel_util import pack_pages, pack_pages_whole, reference_attention, reference_attention_blocked
+
+    g = torch.Generator().manual_seed(3)
+    T, nkv, hd, ps = 77, 2, 32, 16
+    k, v = torch.randn(T, nkv, hd, generator=g), torch.randn(T, nkv, hd, generator=g)
+    table = [4, 0, 6, 2, 5]
+    a = [torch.zeros(8, nkv * hd * ps) for _ in range(2)]
+    b = [torch.zeros(8, nkv * hd * ps) for _ in range(2)]
+    pack_pages(a[0], a[1], k, v, table, ps)
+    pack_pages_whole(b[0], b[1], k, v, table, ps)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    q = torch.randn(9, 4, hd, generator=g)
+    positions = [3, 20, 21, 40, 41, 42, 60, 75, 76]
+    one = reference_attention(q, k, v, positions, 0.3)
+    two = reference_attention_blocked(q, k, v, positions, 0.3, block=4)
+    torch.testing.assert_close(one, two, rtol=1e-12, atol=1e-12)
+
+
+def test_attention_in_blocks_of_queries_is_the_same_arithmetic(tmp_path):
+    """``query_block`` only bounds memory for long sequences: the same logits."""
+    folder = make_folder(tmp_path, "B")
+    cfg, w = plain.read_folder(folder)
+    ids = torch.randint(0, cfg["vocab_size"], (45,), generator=torch.Generator().manual_seed(1)).tolist()
+    whole = plain.logits(ids, cfg, w)
+    for block in (1, 7, 16, 45, 100):
+        torch.testing.assert_close(plain.logits(ids, cfg, w, query_block=block), whole, rtol=0, atol=2e-6)
