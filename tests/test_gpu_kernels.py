@@ -144,35 +144,41 @@ def test_many_tiles_over_long_contexts_use_the_four_wave_kernel():
         torch.testing.assert_close(g, w, **TOL[torch.bfloat16])
 
 
-@pytest.mark.parametrize("nh, nkv, hd, ps", [(8, 2, 128, 16), (6, 3, 64, 32), (3, 1, 128, 16), (32, 8, 128, 16), (4, 4, 64, 64)])
-def test_wide_tiles_for_long_walks(nh, nkv, hd, ps, monkeypatch):
-    """Portions cut into tiles of 32 tokens, the 32x32 matrix-core form: taken (checked by
-    its conditions, here with the threshold on the context lowered) when tiles are mostly
+@pytest.mark.parametrize("nh, nkv, hd, ps", [(8, 2, 128, 16), (6, 3, 64, 32), (3, 1, 128, 16), (32, 8, 128, 16), (4, 4, 64, 64),
+                                             (5, 1, 128, 16), (12, 2, 64, 16), (7, 1, 128, 32), (16, 2, 128, 16), (20, 2, 64, 16),
+                                             (6, 1, 128, 16), (9, 1, 64, 16)])
+def test_tiles_of_32_tokens_for_long_walks(nh, nkv, hd, ps, monkeypatch):
+    """Portions cut into tiles of 32 tokens, the 32x32 matrix-core forms: taken (checked by
+    their conditions, here with the thresholds on the context lowered) when tiles are mostly
     full; portions that start at zero, in the middle of a page, end inside a tile, a
-    one-token tail tile, and a decode token beside them."""
+    one-token tail tile, and a decode token beside them.  Groups of three query heads and
+    more take the group form (a block of all the group's heads, up to eight, and shares of
+    the keys that are merged in the block), smaller ones the wide form."""
     from tokamak_amd.kernels import attention
 
     monkeypatch.setattr(attention, "WIDE_FROM_KEYS", 64)
-    requests = [(0, 200), (37, 150), (900, 33), (5, 32), (300, 1)]
+    monkeypatch.setattr(attention, "GROUP_FROM_KEYS", 64)
+    requests = [(0, 200), (37, 150), (900, 33), (5, 32), (300, 1), (0, 450)]
     tiles = [q for _, q in requests if q > 1]
     assert sum(tiles) >= attention.WIDE_FROM_TOKENS * sum(-(-q // 32) for q in tiles)
     launched = []
     real = attention.ops.attention_mfma
     monkeypatch.setattr(attention.ops, "attention_mfma", lambda mode, *a, **k: (launched.append(mode), real(mode, *a, **k))[1])
     got, want = run_attention(torch.bfloat16, nh, nkv, hd, ps, requests, seed=21)
-    assert launched == ["heads", "tokens_wide"]
+    assert launched == ["heads", "tokens_group" if nh // nkv >= 3 else "tokens_wide"]
     for g, w in zip(got, want):
         assert torch.isfinite(g).all(), "a page that the request does not own, or a slot past its end, was read"
         torch.testing.assert_close(g, w, **TOL[torch.bfloat16])
 
 
-def test_wide_tiles_find_a_far_key_and_respect_the_causal_edge():
-    """The wide form on inputs made to show faults: one key far back dominates one query's
+@pytest.mark.parametrize("nh, nkv", [(8, 2), (4, 2), (5, 1)])
+def test_tiles_of_32_tokens_find_a_far_key_and_respect_the_causal_edge(nh, nkv):
+    """The group form (and for groups of two the wide form) on inputs made to show faults: one key far back dominates one query's
     softmax (its value must come out), and the key right after a query's position is made
     enormous (reading it would show)."""
     from tokamak_amd.kernels import attention
 
-    hd, nh, nkv = 128, 8, 2
+    hd = 128
     seen = {}
 
     def boost(q, k, v, ctx, qlen):

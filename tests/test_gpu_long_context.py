@@ -109,13 +109,23 @@ def test_a_short_portion_over_the_longest_context(dtype, keys, monkeypatch):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("keys", [32768, 40960])
 def test_a_long_portion_over_the_longest_context(dtype, keys, monkeypatch):
-    """2,048 tokens at the end of ``keys``: the wide matrix-core form at its real threshold."""
+    """2,048 tokens at the end of ``keys``: the group form (tiles of 32 tokens, a block a CU) at
+    its real threshold."""
     ctx = keys - 2048
     targets = [(0, 0), (31, 63), (32, 64), (1000, ctx - 1), (1500, ctx + 1499), (2047, ctx // 3), (777, 4095), (778, 4096)]
     launched = run(dtype, 8, 2, ctx, 2048, seed=keys + 2, targets=targets,
                    monkeypatch=monkeypatch if dtype == torch.bfloat16 else None)
     if dtype == torch.bfloat16:
-        assert launched == [("tokens_wide", 1)]
+        assert launched == [("tokens_group", 1)]
+
+
+@pytest.mark.parametrize("keys", [32768, 40960])
+def test_a_long_portion_of_pairs_of_heads_over_the_longest_context(keys, monkeypatch):
+    """The same with two query heads a kv head: the wide form."""
+    ctx = keys - 2048
+    targets = [(0, 0), (31, 63), (32, 64), (1000, ctx - 1), (1500, ctx + 1499), (2047, ctx // 3)]
+    launched = run(torch.bfloat16, 8, 4, ctx, 2048, seed=keys + 4, targets=targets, monkeypatch=monkeypatch)
+    assert launched == [("tokens_wide", 1)]
 
 
 @pytest.mark.parametrize("keys", [32768, 40960])

@@ -897,6 +897,333 @@ void attention_prefill_wide_kernel(
 #undef TK_FETCH
 #undef TK_PAGES
 
+// ---------------------------------------------------------------------------
+// Prompt portions, group form: the wide form's products (tiles of up to 32 tokens,
+// v_mfma_f32_32x32x16_bf16) in a block that holds a whole CU: GB query heads of one kv
+// head times S shares of the keys, one wave each (GB * S <= 8 waves, two a SIMD with the
+// registers the wide form needs).  A stage is 64 * S keys; wave (head hw, share sp) takes
+// the stage's keys 64 sp .. 64 sp + 63, and the shares of a head are merged through LDS
+// when the tile's keys are done.  Against the wide form with its two independent blocks a
+// CU: every kv head's keys and values are copied into LDS once for all its query heads
+// (any group size, also 3, 5, 7), and a tile's walk over the keys is S times shorter, so
+// that a prompt from position zero, whose tiles differ in length from 32 keys to the whole
+// prompt, leaves no CU with one long tile at a quarter of its waves: tiles are started
+// longest first, twice as many as there are CUs, and the short ones fill in behind.
+// ---------------------------------------------------------------------------
+template <int HD, int GB, int S>
+__global__ __launch_bounds__(GB * S * 64)
+void attention_prefill_group_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int max_pages,
+    const int* __restrict__ positions, const int* __restrict__ req_of_token,
+    const int* __restrict__ item_token, const int* __restrict__ item_count,
+    bf16_t* __restrict__ out, int num_items, int nh, int nkv, int ps, float scale_log2) {
+  constexpr int KST = HD / 16;  // 16-wide steps over the head dim (QK^T)
+  constexpr int DB = HD / 32;   // 32-wide blocks of the head dim (PV outputs)
+  constexpr int DBL = HD / 16;  // 16-dim blocks of a V page
+  constexpr int THREADS = GB * S * 64;
+  constexpr int STAGE = 64 * S;             // keys a stage
+  constexpr int GROUP_PIECES = 2 * HD;      // 16-byte pieces of K (and of V) per 16-key group
+  constexpr int SUB_PIECES = 4 * GROUP_PIECES;  // per 64 keys
+  constexpr int PIECES = S * SUB_PIECES;    // per stage
+  constexpr int PPT = (PIECES + THREADS - 1) / THREADS;
+  constexpr bool EVEN = PIECES % THREADS == 0;
+  constexpr int ACC = DB * 16;              // accumulator floats a lane
+  static_assert(GROUP_PIECES % 64 == 0, "a wave's pieces of one load lie in one 16-key group");
+  // two stages in LDS where they fit: the next stage is written while this one is multiplied,
+  // and one barrier a stage is enough
+  constexpr int NB = (2 * PIECES * 32 <= 160 * 1024) ? 2 : 1;
+  constexpr int BUF = 2 * PIECES * 8;       // elements of a stage's K and V
+  extern __shared__ __attribute__((aligned(16))) bf16_t smem_group[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, g = lane >> 5;
+  const int hw = wave % GB, sp = wave / GB;
+  const int G = nh / nkv;
+  const int nblk = (G + GB - 1) / GB;
+  const int kvh = blockIdx.x / nblk;
+  const int hin = (blockIdx.x % nblk) * GB + hw;
+  const bool computes = hin < G;
+  const int head = kvh * G + (computes ? hin : 0);
+  const int item = num_items - 1 - blockIdx.y;  // later tiles have more keys: start them first
+
+  const int n0 = item_token[item];
+  const int count = item_count[item];
+  const int pos0 = positions[n0];
+  const int last_pos = pos0 + count - 1;
+  const int last_key = last_pos;
+  const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
+  const size_t page_elems = (size_t)nkv * HD * ps;
+  const size_t head_off = (size_t)kvh * HD * ps;
+  const int c_pos = pos0 + col;
+  const bool c_valid = col < count;
+
+  // Q as B operand: lane (query col, g) holds Q[col][16c + 8g .. +8]
+  bf16x8 qreg[KST];
+  {
+    const bf16_t* qp = q + ((size_t)(n0 + (c_valid ? col : 0)) * nh + head) * HD + g * 8;
+#pragma unroll
+    for (int c = 0; c < KST; ++c) {
+      Frag8 f;
+      f.u = *reinterpret_cast<const uint4*>(qp + c * 16);
+      if (!c_valid) f.u = make_uint4(0, 0, 0, 0);
+      qreg[c] = f.v;
+    }
+  }
+
+  float m_run = -INFINITY, l_run = 0.f;
+  float16v acc[DB];  // acc[db][4i + j] = O^T[dim 32 db + 8i + 4g + j][col]
+#pragma unroll
+  for (int d = 0; d < DB; ++d)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[d][e] = 0.f;
+
+  // Piece p = i * THREADS + tid of a stage: share p / SUB_PIECES, and within the share's 64
+  // keys as the wide form has it.
+  u32x4 kpre[PPT], vpre[PPT];
+  const int ps_shift = __ffs(ps) - 1;  // page sizes are powers of two here
+  int grp[PPT];                        // 16-key group within the stage; wave-uniform
+  unsigned k_in[PPT], v_in[PPT];       // byte offset inside the page's head, for key 0 of a group
+  int v_quad[PPT];
+  unsigned v_lds[PPT][2];              // element offsets in vs of the piece's two dims
+  bool piece[PPT];                     // wave-uniform: the piece exists
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    const int pa = i * THREADS + tid;
+    piece[i] = EVEN || pa < PIECES;
+    const int share = pa / SUB_PIECES, p = pa % SUB_PIECES;
+    grp[i] = __builtin_amdgcn_readfirstlane(piece[i] ? share * 4 + p / GROUP_PIECES : 0);
+    k_in[i] = (unsigned)((((p / 16) % (HD / 8)) * ps + (p % 16)) * 8) * 2u;
+    const int d = (p / 32) % DBL, quad = (p % 32) / 8, dp = p % 8;
+    v_in[i] = (unsigned)(d * (ps >> 2) * 64 + (p % 32) * 8) * 2u;
+    v_quad[i] = quad;
+    // vs, per share: [group j][g = quad & 1][dim][quad >> 1][4 keys]
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+      v_lds[i][half] = (unsigned)(share * SUB_PIECES * 8) +
+          (unsigned)(((((p / GROUP_PIECES) * 2 + (quad & 1)) * HD + d * 16 + 2 * dp + half) * 2 + (quad >> 1)) * 4);
+  }
+  int page_next[PPT];
+#define TK_GPAGES(S0)                                                              \
+  if ((S0) <= last_key) {                                                          \
+    _Pragma("unroll") for (int i = 0; i < PPT; ++i) {                              \
+      const int c0 = ((S0) + grp[i] * 16 <= last_pos) ? (S0) + grp[i] * 16 : (S0); \
+      page_next[i] = table[c0 >> ps_shift];                                        \
+    }                                                                              \
+  }
+#define TK_GFETCH(S0)                                                                              \
+  {                                                                                                \
+    _Pragma("unroll") for (int i = 0; i < PPT; ++i) if (piece[i]) {                                \
+      const int c0 = ((S0) + grp[i] * 16 <= last_pos) ? (S0) + grp[i] * 16 : (S0);                 \
+      const size_t pg = (size_t)__builtin_amdgcn_readfirstlane(page_next[i]) * page_elems + head_off; \
+      const int off = c0 & (ps - 1);                                                               \
+      const char* kp = reinterpret_cast<const char*>(k_cache + pg + (size_t)off * 8);              \
+      const char* vp = reinterpret_cast<const char*>(v_cache + pg + (size_t)(off >> 2) * 64);      \
+      kpre[i] = *reinterpret_cast<const u32x4*>(kp + k_in[i]);                                     \
+      vpre[i] = *reinterpret_cast<const u32x4*>(vp + v_in[i]);                                     \
+    }                                                                                              \
+    TK_GPAGES((S0) + STAGE)                                                                        \
+  }
+
+  // keys past the request's end may hold anything (their probability is zero, but 0 * NaN
+  // is NaN): their values are zeroed on the way into LDS
+#define TK_GSTORE(S0, KS, VS)                                                                        \
+  {                                                                                                  \
+    if ((S0) + STAGE - 1 > last_pos) {                                                               \
+      _Pragma("unroll") for (int i = 0; i < PPT; ++i) {                                              \
+        const int k0 = (S0) + grp[i] * 16 + v_quad[i] * 4;                                           \
+        const unsigned m01 = (k0 + 0 > last_pos ? 0u : 0x0000ffffu) | (k0 + 1 > last_pos ? 0u : 0xffff0000u); \
+        const unsigned m23 = (k0 + 2 > last_pos ? 0u : 0x0000ffffu) | (k0 + 3 > last_pos ? 0u : 0xffff0000u); \
+        vpre[i] &= u32x4{m01, m23, m01, m23};                                                        \
+      }                                                                                              \
+    }                                                                                                \
+    _Pragma("unroll") for (int i = 0; i < PPT; ++i) if (piece[i]) {                                  \
+      *reinterpret_cast<u32x4*>((KS) + (size_t)(i * THREADS + tid) * 8) = kpre[i];                   \
+      *reinterpret_cast<uint2*>((VS) + v_lds[i][0]) = make_uint2(vpre[i][0], vpre[i][1]);            \
+      *reinterpret_cast<uint2*>((VS) + v_lds[i][1]) = make_uint2(vpre[i][2], vpre[i][3]);            \
+    }                                                                                                \
+  }
+  TK_GPAGES(0)
+  TK_GFETCH(0)
+  if (NB == 2) {
+    TK_GSTORE(0, smem_group, smem_group + PIECES * 8)
+    if (STAGE <= last_key) TK_GFETCH(STAGE)
+    __syncthreads();
+  }
+  for (int s0 = 0; s0 <= last_key; s0 += STAGE) {
+    bf16_t* ks = smem_group;
+    if (NB == 2) {
+      // this stage lies in buffer (s0 / STAGE) & 1; the next one, on its way in registers since
+      // the stage before, goes into the other buffer, which every wave has left behind
+      const int b = (s0 / STAGE) & 1;
+      ks = smem_group + (size_t)b * BUF;
+      if (s0 + STAGE <= last_key) {
+        bf16_t* kn = smem_group + (size_t)(b ^ 1) * BUF;
+        TK_GSTORE(s0 + STAGE, kn, kn + PIECES * 8)
+        if (s0 + 2 * STAGE <= last_key) TK_GFETCH(s0 + 2 * STAGE)
+      }
+    } else {
+      __syncthreads();  // every wave has read the previous stage
+      TK_GSTORE(s0, ks, ks + PIECES * 8)
+      __syncthreads();
+      if (s0 + STAGE <= last_key) TK_GFETCH(s0 + STAGE)
+    }
+    const bf16_t* const ksw = ks + (size_t)sp * SUB_PIECES * 8;  // this wave's share of the stage
+    const bf16_t* const vsw = ksw + PIECES * 8;
+    const int w0 = s0 + 64 * sp;  // this wave's 64 keys of the stage
+    if (computes && w0 <= last_key) {
+
+    // S^T for two blocks of 32 keys: sc[kb][4i + j] = score of key w0 + 32 kb + 8i + 4g + j.
+    // A block's operands are asked for together, and the second block's while the first
+    // block's products run: a wave that waits for each operand in turn spends its time on
+    // round trips to LDS (some hundred clocks each), not on the products.
+    float16v sc[2];
+    {
+      Frag8 kf[2][KST];  // K[key 32 kb + col][16c + 8g .. +8]: piece (group 2kb + col/16, chunk 2c + g, key col%16)
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sc[kb][e] = 0.f;
+#pragma unroll
+        for (int c = 0; c < KST; ++c)
+          kf[kb][c].u = *reinterpret_cast<const uint4*>(
+              ksw + ((size_t)((2 * kb + (col >> 4)) * (HD / 8) + 2 * c + g) * 16 + (col & 15)) * 8);
+      }
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int c = 0; c < KST; ++c)
+          sc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kb][c].v, qreg[c], sc[kb], 0, 0, 0);
+      // the order asked of the scheduler: the first block's reads; a product and a read of the
+      // second block in turn; the second block's products
+      __builtin_amdgcn_sched_group_barrier(0x100, KST, 0);
+#pragma unroll
+      for (int c = 0; c < KST; ++c) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, KST, 0);
+    }
+    if (w0 + 63 > pos0) {  // some key of these is hidden from some query, or is past the end
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = w0 + 32 * kb + 8 * (e >> 2) + 4 * g + (e & 3);
+          if (key > c_pos || key > last_pos) sc[kb][e] = -INFINITY;
+        }
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) tmax = fmaxf(tmax, sc[kb][e]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    // the running maximum is kept in units of log2: m = max(score) * scale * log2(e)
+    const float m_new = fmaxf(m_run, tmax * scale_log2);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);
+    m_run = m_new;
+    float psum = 0.f;
+    Frag8 pb[2][2];  // pb[kb][h]: the sixteen keys 32 kb + 16 h .. of this lane's half
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        float pr[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pr[e] = fast_exp2(fmaf(sc[kb][8 * h + e], scale_log2, -m_safe));
+          psum += pr[e];
+        }
+        pb[kb][h].u = make_uint4(pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3]), pack_bf16x2(pr[4], pr[5]),
+                                 pack_bf16x2(pr[6], pr[7]));
+      }
+    l_run = l_run * alpha + psum;
+    // the accumulators need rescaling only when some query's maximum moved
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+      for (int d = 0; d < DB; ++d) acc[d] *= alpha;
+    }
+    {
+      // O^T += V^T P^T, a 32-dim block of the output at a time; operands asked for a block ahead
+      Frag8 vf[DB][4];  // V^T[dim 32 d + col][the lane half's eight keys of group 2 kb + h]
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int kh = 0; kh < 4; ++kh)
+          vf[d][kh].u = *reinterpret_cast<const uint4*>(vsw + ((size_t)(kh * 2 + g) * HD + 32 * d + col) * 8);
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int kh = 0; kh < 4; ++kh)
+          acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[d][kh].v, pb[kh >> 1][kh & 1].v, acc[d], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+      for (int i = 0; i < 4 * DB - 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+    }
+    }  // computes
+    if (NB == 2) __syncthreads();  // the next stage is written, and every wave has read this one
+  }
+#undef TK_GSTORE
+#undef TK_GFETCH
+#undef TK_GPAGES
+
+  if (S > 1) {
+    // the shares of a head meet in LDS: share sp > 0 leaves its (acc, m, l), share 0 adds them
+    // in share order.  Per (share - 1, head): ACC rows of 64 lanes, then m and l.
+    float* const ms = reinterpret_cast<float*>(smem_group);
+    constexpr int PER = (ACC + 2) * 64;
+    __syncthreads();  // every wave has read the last stage
+    if (sp > 0) {
+      float* mine = ms + (size_t)((sp - 1) * GB + hw) * PER;
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mine[(d * 16 + e) * 64 + lane] = acc[d][e];
+      mine[ACC * 64 + lane] = m_run;
+      mine[(ACC + 1) * 64 + lane] = l_run;
+    }
+    __syncthreads();
+    if (sp > 0) return;
+#pragma unroll
+    for (int s = 1; s < S; ++s) {
+      const float* theirs = ms + (size_t)((s - 1) * GB + hw) * PER;
+      const float m2 = theirs[ACC * 64 + lane], l2 = theirs[(ACC + 1) * 64 + lane];
+      const float m_new = fmaxf(m_run, m2);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float a1 = fast_exp2(m_run - m_safe), a2 = fast_exp2(m2 - m_safe);
+      m_run = m_new;
+      l_run = l_run * a1 + l2 * a2;
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[d][e] = acc[d][e] * a1 + theirs[(d * 16 + e) * 64 + lane] * a2;
+    }
+  }
+
+  float l = l_run;
+  l += __shfl_xor(l, 32, kWave);
+  if (c_valid && computes) {
+    const float inv = 1.f / l;
+    bf16_t* op = out + ((size_t)(n0 + col) * nh + head) * HD + g * 4;
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint2 o;
+        o.x = pack_bf16x2(acc[d][4 * i] * inv, acc[d][4 * i + 1] * inv);
+        o.y = pack_bf16x2(acc[d][4 * i + 2] * inv, acc[d][4 * i + 3] * inv);
+        *reinterpret_cast<uint2*>(op + 32 * d + 8 * i) = o;
+      }
+  }
+}
+
+
 template <int HD, int HPB, int OCC>
 static int launch_prefill(const void* q, const void* k_cache, const void* v_cache,
                           const int* block_tables, int max_pages, const int* positions,
@@ -930,6 +1257,66 @@ static int launch_prefill_wide(const void* q, const void* k_cache, const void* v
       positions, req_of_token, item_token, item_count, (bf16_t*)out, num_items, nh, nkv, ps,
       scale * 1.4426950408889634f);
   return launch_status();
+}
+
+template <int HD, int GB, int S>
+static int launch_prefill_group(const void* q, const void* k_cache, const void* v_cache,
+                                const int* block_tables, int max_pages, const int* positions,
+                                const int* req_of_token, const int* item_token, const int* item_count,
+                                int num_items, void* out, int nh, int nkv, int ps, float scale,
+                                hipStream_t stream) {
+  const int G = nh / nkv;
+  constexpr size_t one_stage = (size_t)S * 8 * HD * 16 * 2;                       // K and V of a stage
+  constexpr size_t stage_bytes = 2 * one_stage <= 160 * 1024 ? 2 * one_stage : one_stage;  // two where they fit
+  constexpr size_t merge_bytes = (size_t)(S - 1) * GB * ((HD / 2 + 2) * 64) * 4;  // the shares' results
+  constexpr size_t lds = stage_bytes > merge_bytes ? stage_bytes : merge_bytes;
+  static_assert(lds <= 160 * 1024, "a stage must fit the CU's LDS");
+  if (lds > 48 * 1024) {
+    static bool raised = false;  // per template instance
+    if (!raised) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_group_kernel<HD, GB, S>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return -2;
+      }
+      raised = true;
+    }
+  }
+  dim3 grid(nkv * ((G + GB - 1) / GB), num_items);
+  attention_prefill_group_kernel<HD, GB, S><<<grid, GB * S * 64, lds, stream>>>(
+      (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_pages,
+      positions, req_of_token, item_token, item_count, (bf16_t*)out, num_items, nh, nkv, ps,
+      scale * 1.4426950408889634f);
+  return launch_status();
+}
+
+// Heads of a kv head's group that share a block of the group form, and the shares of the
+// keys beside them: as many waves as fit two a SIMD (eight), all heads of the group in one
+// block where that is possible.
+template <int HD>
+static int launch_prefill_group_any(const void* q, const void* k_cache, const void* v_cache,
+                                    const int* block_tables, int max_pages, const int* positions,
+                                    const int* req_of_token, const int* item_token, const int* item_count,
+                                    int num_items, void* out, int nh, int nkv, int ps, float scale,
+                                    hipStream_t stream) {
+#define TK_GARGS                                                                                  \
+  q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
+      num_items, out, nh, nkv, ps, scale, stream
+  const int G = nh / nkv;
+  const int nblk = (G + 7) / 8;
+  const int gb = (G + nblk - 1) / nblk;  // heads a block: G itself up to 8, else an even share
+  switch (gb) {
+    case 1: return launch_prefill_group<HD, 1, 4>(TK_GARGS);
+    case 2: return launch_prefill_group<HD, 2, 4>(TK_GARGS);
+    case 3: return launch_prefill_group<HD, 3, 2>(TK_GARGS);
+    case 4: return launch_prefill_group<HD, 4, 2>(TK_GARGS);
+    case 5: return launch_prefill_group<HD, 5, 1>(TK_GARGS);
+    case 6: return launch_prefill_group<HD, 6, 1>(TK_GARGS);
+    case 7: return launch_prefill_group<HD, 7, 1>(TK_GARGS);
+    case 8: return launch_prefill_group<HD, 8, 1>(TK_GARGS);
+  }
+#undef TK_GARGS
+  return -2;
 }
 
 template <int HD, bool FUSED>
@@ -973,6 +1360,7 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
 //         is a multiple of 64 and the partial buffers hold 16 rows per item)
 // mode 2: tokens, every tile over a long context (same results; the kernel built for four waves a SIMD)
 // mode 3: tokens, wide form (item = up to 32 consecutive tokens of one request; nsplit must be 1)
+// mode 4: tokens, group form (items as in mode 3; any group size; a block holds a CU)
 // Returns -2 if this shape is not instantiated (the caller uses the generic kernel).
 TK_API int tk_attention_decode_waves() { return kDecodeWaves; }
 
@@ -983,7 +1371,7 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
                              int split_keys, int nh, int nkv, int hd, int ps, float scale,
                              hipStream_t stream) {
   if (num_items <= 0) return 0;
-  if (mode < 0 || mode > 3) return -1;
+  if (mode < 0 || mode > 4) return -1;
   if (nkv <= 0 || nh % nkv != 0 || ps < 16 || (ps & (ps - 1)) != 0 || split_keys % 16 != 0 || nsplit < 1) return -1;
   if (num_items > 65535 || nh > 65535) return -1;
   const int G = nh / nkv;
@@ -996,20 +1384,29 @@ TK_API int tk_attention_mfma(int mode, const void* q, const void* k_cache, const
     if (hd == 64) return launch<64, false>(TK_ARGS);
     return -2;
   }
+  if (mode == 4) {
+    if (nsplit != 1) return -1;
+    if (hd == 128) return launch_prefill_group_any<128>(q, k_cache, v_cache, block_tables, max_pages, positions,
+                                                        req_of_token, item_token, item_count, num_items, out, nh,
+                                                        nkv, ps, scale, stream);
+    if (hd == 64) return launch_prefill_group_any<64>(q, k_cache, v_cache, block_tables, max_pages, positions,
+                                                      req_of_token, item_token, item_count, num_items, out, nh,
+                                                      nkv, ps, scale, stream);
+    return -2;
+  }
   const int hpb = (G % 4 == 0) ? 4 : (G % 2 == 0) ? 2 : 1;
   if (mode == 3) {
     if (nsplit != 1) return -1;
 #define TK_WARGS                                                                                  \
   q, k_cache, v_cache, block_tables, max_pages, positions, req_of_token, item_token, item_count, \
       num_items, out, nh, nkv, ps, scale, stream
+    // (groups of three heads and more take the group form; blocks of two heads or one here)
     if (hd == 128) {
-      if (hpb == 4) return launch_prefill_wide<128, 4>(TK_WARGS);
-      if (hpb == 2) return launch_prefill_wide<128, 2>(TK_WARGS);
+      if (G % 2 == 0) return launch_prefill_wide<128, 2>(TK_WARGS);
       return launch_prefill_wide<128, 1>(TK_WARGS);
     }
     if (hd == 64) {
-      if (hpb == 4) return launch_prefill_wide<64, 4>(TK_WARGS);
-      if (hpb == 2) return launch_prefill_wide<64, 2>(TK_WARGS);
+      if (G % 2 == 0) return launch_prefill_wide<64, 2>(TK_WARGS);
       return launch_prefill_wide<64, 1>(TK_WARGS);
     }
 #undef TK_WARGS

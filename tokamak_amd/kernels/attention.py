@@ -22,6 +22,8 @@ DENSE_TILES_FROM = 2048         # every tiled span starts at least this deep: th
 WIDE_FROM_KEYS = 4096           # longest context from which the 32-token tiles of the wide kernel pay (+15-20 %;
                                 # for shorter walks the narrow one's smaller tiles balance better)
 WIDE_FROM_TOKENS = 20           # ... if a 32-token tile holds at least this many tokens on average
+GROUP_FROM_KEYS = 1024          # longest context from which the group form (a block a CU, all heads of a kv head) pays ...
+GROUP_FROM_HEADS = 3            # ... for groups of at least this many query heads a kv head (fewer: too few waves a block)
 
 
 def quarter_octave_at_least(n: int, floor: int) -> int:
@@ -184,11 +186,13 @@ def paged_attention(q, k_cache, v_cache, block_tables, batch, out, *, num_heads,
     """out[n] = softmax(q[n] . K[0..pos_n] * scale) V, per head, over the pages
     of each token's request.
 
-    bfloat16 with head size 64 or 128: the MFMA kernel, once over the single
-    (decode) tokens with their context split, once over 16-token tiles of the
-    prompt portions (their keys split too when the tiles are few and the context
-    long).  Everything else, and whatever the MFMA library does not instantiate:
-    the generic float32-arithmetic kernel.
+    bfloat16 with head size 64 or 128: the MFMA kernels, once over the single
+    (decode) tokens with their context split, once over the tiles of the prompt
+    portions: tiles of 32 tokens in the group form (a block a CU: all query heads
+    of a kv head and shares of the keys) when the tiles are mostly full and walk
+    a thousand keys or more; tiles of 16 otherwise, their keys split over blocks
+    when the tiles are few and the context long.  Everything else, and whatever
+    the MFMA library does not instantiate: the generic float32-arithmetic kernel.
     """
     work = work_of(batch)
     profiling = ops._profile is not None
@@ -235,6 +239,14 @@ def _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, *
         group = num_heads // num_kv_heads
         per_tile = num_kv_heads * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
         split, nsplit = tile_split(work.num_tiles, per_tile, work.max_tile_len)
+        if (nsplit == 1 and work.max_tile_len >= GROUP_FROM_KEYS and group >= GROUP_FROM_HEADS
+                and work.num_tile_tokens >= WIDE_FROM_TOKENS * work.num_wide):
+            # tiles of 32 tokens mostly full: the group form, whose blocks hold a CU each
+            if note is not None:
+                ops._note(f"portions {work.num_wide} wide tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
+            return ops.attention_mfma("tokens_group", q, k_cache, v_cache, block_tables, batch.positions,
+                                      batch.req_of_token, work.wide_first, work.wide_count, work.num_wide,
+                                      out, **common)
         if (nsplit == 1 and work.max_tile_len >= WIDE_FROM_KEYS
                 and work.num_tile_tokens >= WIDE_FROM_TOKENS * work.num_wide):
             # long walks over the keys, tiles of 32 tokens mostly full: the wide kernel

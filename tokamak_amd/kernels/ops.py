@@ -709,7 +709,9 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     """bf16 attention on the matrix cores.  ``mode`` "heads": every item is one
     decode token; "tokens": every item is up to 16 consecutive tokens of one
     request ("tokens_dense": the same, with the kernel variant for tiles that all
-    walk a long context; "tokens_wide": items of up to 32 tokens, the 32x32 MFMA form).  With ``num_splits`` > 1 the keys of an item are cut into pieces of
+    walk a long context; "tokens_wide": items of up to 32 tokens, the 32x32 MFMA form;
+    "tokens_group": the same items, a block of up to eight waves holding all query heads of
+    a kv head and shares of the keys, any group size).  With ``num_splits`` > 1 the keys of an item are cut into pieces of
     ``split_keys`` (a multiple of 16; of 64 in "tokens" mode), each its own block, and a
     second kernel merges the pieces (in "heads" mode the sixteen waves of a block share a piece, so
     ``split_keys`` is a multiple of 256).  Returns False (nothing launched) if the shape
@@ -726,8 +728,9 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     _need(positions.dtype == torch.int32 and req_of_token.dtype == torch.int32 and block_tables.dtype == torch.int32
           and item_token.dtype == torch.int32 and block_tables.dim() == 2, "descriptor arrays are int32")
     _need(item_token.numel() >= num_items and 0 < num_items <= 65535, "bad item list")
-    _need(mode in ("heads", "tokens", "tokens_dense", "tokens_wide"), "mode is heads, tokens, tokens_dense or tokens_wide")
-    _need(mode != "tokens_wide" or num_splits == 1, "the wide form does not split keys")
+    _need(mode in ("heads", "tokens", "tokens_dense", "tokens_wide", "tokens_group"),
+          "mode is heads, tokens, tokens_dense, tokens_wide or tokens_group")
+    _need(mode not in ("tokens_wide", "tokens_group") or num_splits == 1, "the wide and group forms do not split keys over blocks")
     _need(mode != "heads" or num_splits == 1 or split_keys % 256 == 0, "heads mode splits keys in multiples of 256")
     if mode != "heads":
         _need(item_count is not None and item_count.dtype == torch.int32 and item_count.numel() >= num_items,
@@ -740,7 +743,7 @@ def attention_mfma(mode: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
         part_o = torch.empty((rows, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((rows, 2), dtype=torch.float32, device=q.device)
     status = _fn("attention_mfma", "tk_attention_mfma")(
-        {"heads": 0, "tokens": 1, "tokens_dense": 2, "tokens_wide": 3}[mode], _p(q), _p(k_cache), _p(v_cache), _p(block_tables),
+        {"heads": 0, "tokens": 1, "tokens_dense": 2, "tokens_wide": 3, "tokens_group": 4}[mode], _p(q), _p(k_cache), _p(v_cache), _p(block_tables),
         block_tables.shape[1], _p(positions), _p(req_of_token), _p(item_token), _p(item_count),
         num_items, _p(out), _p(part_o), _p(part_ml), num_splits, split_keys, num_heads, num_kv_heads,
         head_dim, page_size, float(scale), _stream())
