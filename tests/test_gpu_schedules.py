@@ -301,18 +301,31 @@ def test_layers_launched_from_a_recorded_layer_give_the_same_bits(dtype):
         cache = [a.clone() for slot in sorted(runner.storage._slots) for a in runner.storage.slot(slot).arrays.values()]
         return [o.cpu() for o in out], cache
 
+    packed = []
+
     def counted(self, tensors, then):
         launched.append(len(self.calls))
+        packed.append(self.packed is not None and len(self.packed.expected) == len(self.calls))
         return launch(self, tensors, then)
 
     plainly, cache_plain = run(False)
     try:
         layer_replay.LayerRecording.launch = counted
         replayed, cache_replayed = run(True)
+        # ... and once more with the lists issued call by call from Python (what a recording falls
+        # back to when an entry point has no slot form)
+        layer_replay.LayerRecording.launch = lambda self, tensors, then: (
+            setattr(self, "packed", None), launch(self, tensors, then))[1]
+        by_call, cache_by_call = run(True)
     finally:
         layer_replay.LayerRecording.launch = launch
     assert len(launched) == 5 * (cfg.num_layers - 2), "three of five layers of every step are launched from the list"
     assert min(launched) >= 5
+    assert all(packed), "every list was issued by one foreign call (csrc/replay.hip)"
+    for a, b in zip(replayed, by_call):
+        assert torch.equal(a, b)
+    for a, b in zip(cache_replayed, cache_by_call):
+        assert torch.equal(a, b)
     for step, (a, b) in enumerate(zip(plainly, replayed)):
         assert torch.equal(a, b), f"step {step}: {float((a - b).abs().max())}"
     for a, b in zip(cache_plain, cache_replayed):

@@ -17,6 +17,7 @@
 //
 // Cache pages: K [nkv][hd/8][ps][8], V [nkv][hd/16][ps/4][16][4] (see elementwise.hip).
 #include "common.h"
+#include "slots.h"
 
 using namespace tk;
 
@@ -262,3 +263,6 @@ TK_API int tk_paged_attention_generic(int dtype, const void* q, const void* k_ca
 #undef TK_GENERIC
   return launch_status();
 }
+
+// the same entry points in slot form (slots.h), for launch lists
+TK_SLOTS(tk_paged_attention_generic)

@@ -18,6 +18,7 @@
 // With more than one split the block writes an unnormalised partial (o, m, l) and
 // a second kernel merges the splits of each (token, head).
 #include "common.h"
+#include "slots.h"
 
 using namespace tk;
 
@@ -1465,3 +1466,7 @@ TK_API int tk_attention_decode_fused(const void* qkv, int in_f32, int parts, lon
 #undef TK_FARGS
   return -2;
 }
+
+// the same entry points in slot form (slots.h), for launch lists
+TK_SLOTS(tk_attention_mfma)
+TK_SLOTS(tk_attention_decode_fused)

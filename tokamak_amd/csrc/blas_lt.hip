@@ -25,6 +25,7 @@
 #include <mutex>
 #include <tuple>
 #include <vector>
+#include "slots.h"
 
 #define TK_API extern "C" __attribute__((visibility("default")))
 
@@ -181,3 +182,6 @@ TK_API long tk_lt_tuned_classes() {
   std::lock_guard<std::mutex> guard(g_lock);
   return g_tuned;
 }
+
+// the same entry points in slot form (slots.h), for launch lists
+TK_SLOTS(tk_lt_gemm)

@@ -3,6 +3,7 @@
 // The residual stream is float32 in both dtypes; norm statistics, rotation
 // angles and the residual sum are float32.
 #include "common.h"
+#include "slots.h"
 
 using namespace tk;
 
@@ -558,3 +559,9 @@ TK_API int tk_silu_mul(int dtype, const void* gu, void* out, int N, int I, hipSt
     silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
   return launch_status();
 }
+
+// the same entry points in slot form (slots.h), for launch lists
+TK_SLOTS(tk_add_rmsnorm)
+TK_SLOTS(tk_rope_tables)
+TK_SLOTS(tk_qknorm_rope_store)
+TK_SLOTS(tk_silu_mul)

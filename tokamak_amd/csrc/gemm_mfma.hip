@@ -14,6 +14,7 @@
 // waves' partial sums are added in wave order through LDS (a fixed order, so
 // the result is deterministic) and written as bf16 or float32.
 #include "common.h"
+#include "slots.h"
 
 using namespace tk;
 
@@ -337,14 +338,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
       TK_FETCH_W(next_)                                                                             \
       TK_FETCH_X(next_)                                                                             \
     }                                                                                               \
-    _Pragma("unroll") for (int s = 0; s < SBK / 32; ++s) {                                          \
-      Frag8 wf;                                                                                     \
-      wf.u = *reinterpret_cast<const uint4*>(&ws[wave][r][s * 32 + kb * 8]);                        \
-      _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                              \
-        Frag8 xf;                                                                                   \
-        xf.u = *reinterpret_cast<const uint4*>(&xs[xb_][j * 16 + r][s * 32 + kb * 8]);              \
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf.v, acc[j], 0, 0, 0);              \
+    {                                                                                               \
+      /* the fragments of a step of 32 k are asked for while the step before is multiplied: a    */ \
+      /* wave that waits for each fragment in turn spends its time on round trips to LDS         */ \
+      Frag8 wf[SBK / 32], xf[SBK / 32][MT];                                                         \
+      _Pragma("unroll") for (int s = 0; s < SBK / 32; ++s) {                                        \
+        wf[s].u = *reinterpret_cast<const uint4*>(&ws[wave][r][s * 32 + kb * 8]);                   \
+        _Pragma("unroll") for (int j = 0; j < MT; ++j)                                              \
+            xf[s][j].u = *reinterpret_cast<const uint4*>(&xs[xb_][j * 16 + r][s * 32 + kb * 8]);    \
       }                                                                                             \
+      _Pragma("unroll") for (int s = 0; s < SBK / 32; ++s)                                          \
+        _Pragma("unroll") for (int j = 0; j < MT; ++j)                                              \
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[s].v, xf[s][j].v, acc[j], 0, 0, 0); \
+      /* order asked of the scheduler: two steps' reads, then a product and a read in turn */       \
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * (1 + MT), 0);                                 \
+      _Pragma("unroll") for (int i = 0; i < (SBK / 32 - 2) * (1 + MT); ++i) {                       \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                          \
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                          \
+      }                                                                                             \
+      __builtin_amdgcn_sched_group_barrier(0x008, SBK / 32 * MT - (SBK / 32 - 2) * (1 + MT), 0);    \
     }                                                                                               \
   }
 
@@ -492,3 +504,8 @@ TK_API int tk_gemm_stream_swiglu(const void* A, const void* W, void* C, int M, i
   return launch_stream<bf16_t, true>(waves, A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0,
                                      RowScale{sumsq, slabs, eps}, stream);
 }
+
+// the same entry points in slot form (slots.h), for launch lists
+TK_SLOTS(tk_gemm_stream)
+TK_SLOTS(tk_gemm_stream_swiglu)
+TK_SLOTS(tk_gemm_skinny)

@@ -7,6 +7,7 @@
 // keep the rounding error of a sum over K terms near sqrt(kPiece) + sqrt(K / kPiece)
 // units instead of sqrt(K) (K is 25,600 in the widest feed-forward).
 #include "common.h"
+#include "slots.h"
 
 using namespace tk;
 
@@ -211,3 +212,7 @@ TK_API int tk_gemm_tiled(int in_dtype, int out_dtype, const void* A, const void*
 #undef TK_TILED
   return launch_status();
 }
+
+// the same entry points in slot form (slots.h), for launch lists
+TK_SLOTS(tk_gemm_tiled)
+TK_SLOTS(tk_gemm_fewrows)

@@ -25,6 +25,7 @@
 // So a decode layer of few rows runs q/k/v product, attention, o product, gate/up product and
 // down product with no kernel in between.
 #include "common.h"
+#include "slots.h"
 
 using namespace tk;
 
@@ -318,3 +319,7 @@ TK_API int tk_gemm_wholek_add(const void* A, const void* W, int M, int N, int K,
   if (waves >= 8) return launch_wholek<EPI_ADD, float, 8>(A, W, nullptr, M, N, K, lda, ldw, 0, none, sum, stream);
   return launch_wholek<EPI_ADD, float, 4>(A, W, nullptr, M, N, K, lda, ldw, 0, none, sum, stream);
 }
+
+// the same entry points in slot form (slots.h), for launch lists
+TK_SLOTS(tk_gemm_wholek)
+TK_SLOTS(tk_gemm_wholek_add)

@@ -20,8 +20,9 @@ from __future__ import annotations
 import bisect
 import dataclasses
 from ctypes import c_void_p
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
+import numpy as np
 import torch
 
 from tokamak_amd.kernels import ops
@@ -86,22 +87,80 @@ def call_tensors(own: dict, pending, then) -> dict[tuple, torch.Tensor]:
     return out
 
 
+class PackedCalls:
+    """A recording's calls laid out for ``ops.replay_calls``: the slot forms' addresses, every
+    call's arguments as 64-bit slots in one array, and the patches (slot, index of the tensor
+    in ``keys``, offset inside it).  One foreign call then issues a whole layer."""
+
+    def __init__(self, calls: list[tuple]) -> None:
+        fns, first, slots, expected = [], [], [], []
+        patch_slot, patch_key, patch_offset = [], [], []
+        self.keys: list[tuple] = []
+        index: dict[tuple, int] = {}
+        self.ok = True
+        for fn, args, patches, status in calls:
+            packed = ops.slots_of(fn, args)
+            if packed is None:
+                self.ok = False
+                return
+            fns.append(fn.slots_address)
+            first.append(len(slots))
+            for at, key, offset in patches:
+                if key not in index:
+                    index[key] = len(self.keys)
+                    self.keys.append(key)
+                patch_slot.append(len(slots) + at)
+                patch_key.append(index[key])
+                patch_offset.append(offset)
+            slots.extend(packed)
+            expected.append(status)
+        self.fns = np.array(fns, dtype=np.uint64)
+        self.first = np.array(first, dtype=np.int32)
+        self.slots = np.array(slots, dtype=np.uint64)
+        self.expected = np.array(expected, dtype=np.int32)
+        self.patch_slot = np.array(patch_slot, dtype=np.int32)
+        self.patch_key = np.array(patch_key, dtype=np.int32)
+        self.patch_offset = np.array(patch_offset, dtype=np.int64)
+        self.addresses = np.zeros(max(1, len(self.keys)), dtype=np.uint64)
+        self.got = np.zeros(1, dtype=np.int32)
+        self.pointers = tuple(a.ctypes.data for a in (self.fns, self.first, self.slots))
+        self.patch_pointers = tuple(a.ctypes.data for a in (self.patch_slot, self.patch_key, self.patch_offset,
+                                                            self.addresses, self.expected, self.got))
+
+    def launch(self, tensors: dict[tuple, torch.Tensor]) -> None:
+        addresses = self.addresses
+        for i, key in enumerate(self.keys):
+            addresses[i] = tensors[key].data_ptr()
+        bad = ops.replay_calls(len(self.expected), *self.pointers, len(self.patch_slot), *self.patch_pointers)
+        if bad >= 0:
+            raise ops.KernelError(f"replayed launch {bad} returned {int(self.got[0])}, the recorded one "
+                                  f"{int(self.expected[bad])}")
+
+
 @dataclass
 class LayerRecording:
     calls: list[tuple]          # (function, arguments, ((argument index, tensor key, byte offset), ...), status)
     keep: list[torch.Tensor]
     result: object
+    packed: PackedCalls | None = field(default=None, repr=False)
+
+    def __post_init__(self) -> None:
+        packed = PackedCalls(self.calls)
+        self.packed = packed if packed.ok else None
 
     def launch(self, tensors: dict[tuple, torch.Tensor], then):
-        address = {key: t.data_ptr() for key, t in tensors.items()}     # once a layer, not once a patch
-        for fn, args, patches, status in self.calls:
-            if patches:
-                args = list(args)
-                for index, key, offset in patches:
-                    args[index] = address[key] + offset     # a plain int is taken for a pointer argument
-            got = fn(*args)
-            if got != status:
-                raise ops.KernelError(f"a replayed launch returned {got}, the recorded one {status}")
+        if self.packed is not None:
+            self.packed.launch(tensors)         # the whole layer in one foreign call
+        else:
+            address = {key: t.data_ptr() for key, t in tensors.items()}     # once a layer, not once a patch
+            for fn, args, patches, status in self.calls:
+                if patches:
+                    args = list(args)
+                    for index, key, offset in patches:
+                        args[index] = address[key] + offset     # a plain int is taken for a pointer argument
+                got = fn(*args)
+                if got != status:
+                    raise ops.KernelError(f"a replayed launch returned {got}, the recorded one {status}")
         result = self.result
         if isinstance(result, Added) and result.gamma is not None:
             # the stream times the weight of the norm that follows THIS layer

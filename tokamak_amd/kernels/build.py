@@ -29,7 +29,7 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
 ]
 LIBRARIES = ("elementwise", "gemm_tiled", "attention_generic", "sampling", "gemm_mfma",
-             "gemm_wholek", "attention_mfma", "blas_lt", "peaks")
+             "gemm_wholek", "attention_mfma", "blas_lt", "peaks", "replay")
 # libraries a source links against (blas_lt is host code around hipBLASLt)
 LINK_FLAGS = {"blas_lt": ["-lhipblaslt"]}
 

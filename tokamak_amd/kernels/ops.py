@@ -74,6 +74,43 @@ class recording:
         return False
 
 
+def slots_of(fn, args: tuple) -> list[int] | None:
+    """The arguments of a recorded call as 64-bit slots (csrc/slots.h): integers and
+    addresses as they are (negative ones in two's complement), a float by its bits.  None if
+    the entry point has no slot form."""
+    import struct
+
+    if getattr(fn, "slots_address", None) is None or len(args) != len(fn.argtypes):
+        return None
+    out = []
+    for kind, arg in zip(fn.argtypes, args):
+        value = getattr(arg, "value", arg)
+        if kind is c_float:
+            out.append(struct.unpack("<I", struct.pack("<f", float(value)))[0])
+        elif kind is c_void_p:
+            out.append(int(value or 0))
+        else:
+            out.append(int(value) & 0xFFFFFFFFFFFFFFFF)
+    return out
+
+
+_replay_fn = None
+
+
+def replay_calls(ncalls, fns, first_slot, slots, npatches, patch_slot, patch_key, patch_offset, addresses, expected, got) -> int:
+    """Issue a packed list of recorded launches (csrc/replay.hip): every argument is the
+    address of a host array.  Returns -1, or the index of the first call whose status
+    differs from the recorded one."""
+    global _replay_fn
+    if _replay_fn is None:
+        lib = load_library("replay")
+        _replay_fn = lib.tk_replay_calls
+        _replay_fn.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p]
+        _replay_fn.restype = c_int
+    return _replay_fn(ncalls, fns, first_slot, slots, npatches, patch_slot, patch_key, patch_offset, addresses, expected, got)
+
+
 def not_replayable() -> None:
     """Called where work is launched past this module (a library routine of torch): a
     recording that is being made does not hold it and must not be replayed."""
@@ -254,6 +291,11 @@ def _fn(library: str, name: str):
         fn = getattr(lib, name)
         fn.argtypes = _SIGS[library][name]
         fn.restype = c_int
+        # the same entry point with its arguments as slots, if the library has it (csrc/slots.h)
+        try:
+            fn.slots_address = ctypes.cast(getattr(lib, name + "_slots"), c_void_p).value
+        except AttributeError:
+            fn.slots_address = None
         _fns[name] = fn
     if _profile is not None and name not in ("tk_argmax_segments",):
         profile = _profile
