@@ -635,8 +635,9 @@ def main() -> int:
     max_batch = max(64 if want_points else 1, args.batch)
     peaks = None if args.no_peaks else measure_peaks()
     ops.set_library_tuning(not args.no_tune)
-    pool = max_batch * (-(-(final_context + 1) // PAGE_SIZE) * PAGE_SIZE + PAGE_SIZE)
-    longest = max(final_context + 1, PREFILL_TOKENS + 1)
+    deepest = max(final_context, prompt_tokens + 129) if args.profile else final_context   # (the profiled step sits 129 tokens in)
+    pool = max_batch * (-(-(deepest + 1) // PAGE_SIZE) * PAGE_SIZE + PAGE_SIZE)
+    longest = max(deepest + 1, PREFILL_TOKENS + 1)
     llm = make_llm(cfg, args.dtype, max(pool, PREFILL_TOKENS + PAGE_SIZE, longest), max_batch, longest)
     runner = llm.runner
     cost = StepCost(runner)

@@ -27,6 +27,37 @@ static_assert(kWaves * kWave >= kMaxHd, "the merge gives every dimension a threa
 constexpr int kTileTokens = 16;  // tokens of a tile in the work list
 constexpr int kQueries = 8;      // queries a block of the tile kernel takes
 
+// four consecutive elements (four keys of one dimension in a V page) as one load
+__device__ __forceinline__ void load_four(const float* p, float (&v)[4]) {
+  const float4 x = *reinterpret_cast<const float4*>(p);
+  v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+}
+__device__ __forceinline__ void load_four(const bf16_t* p, float (&v)[4]) {
+  const uint2 x = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(x.x << 16); v[1] = __uint_as_float(x.x & 0xffff0000u);
+  v[2] = __uint_as_float(x.y << 16); v[3] = __uint_as_float(x.y & 0xffff0000u);
+}
+
+// eight consecutive elements (a key's piece of a K page)
+__device__ __forceinline__ void load_eight(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load_eight(const bf16_t* p, float (&v)[8]) {
+  const uint4 x = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+// pieces of a key (8 dimensions each) asked for together: many for a query alone, whose walk
+// is a chain of memory round trips; few where eight queries share the key and the
+// multiply-adds fill the time (and the registers)
+template <int QT> constexpr int key_pieces() { return QT == 1 ? 8 : QT <= 4 ? 4 : 2; }
+
 struct GenericItems {
   const int* single;      // token rows that run alone (null: every token of the step does)
   const int* tile_first;  // first token row of each tile
@@ -44,7 +75,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
     int hd, int ps, int max_pages, float scale, int window) {
   __shared__ __attribute__((aligned(16))) float q_s[QT][kMaxHd];
   __shared__ __attribute__((aligned(16))) float p_s[kWaves][kWave][QT];
-  __shared__ long base_s[kWaves][kWave];
+  __shared__ long base_s[kWaves][kWave];  // where a key's values lie (a quad's, for tokens that run alone), or -1
   __shared__ float m_s[kWaves], l_s[kWaves];
   __shared__ float acc_s[kWaves][kMaxHd];
 
@@ -103,23 +134,53 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
     float dot[QT];
 #pragma unroll
     for (int t = 0; t < QT; ++t) dot[t] = 0.f;
+    // Tokens that run alone (decode) are bound by round trips to memory, not by arithmetic: they
+    // ask for eight pieces of a key at once and for the values of four keys in one piece (four
+    // such pieces at once).  Tiles of a prompt portion, eight queries to a key, are bound by
+    // their multiply-adds and keep the plain loops.  The order of every sum is the same.
+    constexpr bool BATCHED = HEADS;
     long vbase = -1;
+    if (BATCHED && (lane & 3) == 0 && c <= hi && c + 3 >= lo) {
+      // the values of four consecutive keys of a dimension are one piece of a page
+      const int page = table[c / ps];
+      vbase = (long)((size_t)page * page_elems + head_off + (size_t)((c % ps) >> 2) * 64);
+    }
     if (loaded) {
       const int page = table[c / ps];
       const int off = c % ps;
       const T* kp = k_cache + (size_t)page * page_elems + head_off;
-      for (int j = 0; j < hd / 8; ++j) {
-        const T* kk = kp + ((size_t)j * ps + off) * 8;
-        float k8[8];
+      if constexpr (BATCHED) {
+        constexpr int kKeyPieces = key_pieces<QT>();
+        for (int j0 = 0; j0 < hd / 8; j0 += kKeyPieces) {
+          float k8[kKeyPieces][8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) k8[e] = Elem<T>::load(kk + e);
+          for (int u = 0; u < kKeyPieces; ++u) {
+            const int j = min(j0 + u, hd / 8 - 1);      // (a piece past the head is loaded again and not used)
+            load_eight(kp + ((size_t)j * ps + off) * 8, k8[u]);
+          }
 #pragma unroll
-        for (int t = 0; t < QT; ++t) {
+          for (int u = 0; u < kKeyPieces; ++u) {
+            if (j0 + u < hd / 8) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) dot[t] = fmaf(q_s[t][j * 8 + e], k8[e], dot[t]);
+              for (int t = 0; t < QT; ++t) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) dot[t] = fmaf(q_s[t][(j0 + u) * 8 + e], k8[u][e], dot[t]);
+              }
+            }
+          }
         }
+      } else {
+        for (int j = 0; j < hd / 8; ++j) {
+          float k8[8];
+          load_eight(kp + ((size_t)j * ps + off) * 8, k8);
+#pragma unroll
+          for (int t = 0; t < QT; ++t) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dot[t] = fmaf(q_s[t][j * 8 + e], k8[e], dot[t]);
+          }
+        }
+        vbase = (long)((size_t)page * page_elems + head_off + (size_t)(off >> 2) * 64 + (off & 3));
       }
-      vbase = (long)((size_t)page * page_elems + head_off + (size_t)(off >> 2) * 64 + (off & 3));
     }
     float alpha[QT], p[QT];
 #pragma unroll
@@ -141,7 +202,8 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
     wave_lds_sync();   // the wave has read its last round's probabilities
 #pragma unroll
     for (int t = 0; t < QT; ++t) p_s[wave][lane][t] = p[t];
-    base_s[wave][lane] = vbase;
+    if (!BATCHED) base_s[wave][lane] = vbase;
+    else if ((lane & 3) == 0) base_s[wave][lane >> 2] = vbase;
     wave_lds_sync();
     const int count = (hi - c0 + 1 < kWave) ? hi - c0 + 1 : kWave;
 #pragma unroll
@@ -152,12 +214,39 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
         float a[QT];
 #pragma unroll
         for (int t = 0; t < QT; ++t) a[t] = acc[i][t] * alpha[t];
-        for (int key = 0; key < count; ++key) {
-          const long b = base_s[wave][key];
-          if (b >= 0) {
-            const float v = Elem<T>::load(v_cache + b + v_dim_off);
+        if constexpr (BATCHED) {
+          // four keys a load (16 bytes of float32) and four such loads asked for together, added
+          // key by key in ascending order: the same sums as one key at a time.  A key out of
+          // range adds a probability times 0.
+          for (int quad0 = 0; quad0 * 4 < count; quad0 += 4) {
+            float v4[4][4];
+            bool there[4];
 #pragma unroll
-            for (int t = 0; t < QT; ++t) a[t] = fmaf(p_s[wave][key][t], v, a[t]);
+            for (int u = 0; u < 4; ++u) {
+              const long b = base_s[wave][quad0 + u];
+              there[u] = (quad0 + u) * 4 < count && b >= 0;
+              load_four(v_cache + (there[u] ? b : 0) + v_dim_off, v4[u]);   // (absent: the cache's first page, not used)
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const int key = (quad0 + u) * 4 + e;
+                const bool in = there[u] && c0 + key >= lo && c0 + key <= hi;
+                const float v = in ? v4[u][e] : 0.f;   // (the probabilities of such a key are finite: 0 * p adds nothing)
+#pragma unroll
+                for (int t = 0; t < QT; ++t) a[t] = fmaf(p_s[wave][key][t], v, a[t]);
+              }
+            }
+          }
+        } else {
+          for (int key = 0; key < count; ++key) {
+            const long b = base_s[wave][key];
+            if (b >= 0) {
+              const float v = Elem<T>::load(v_cache + b + v_dim_off);
+#pragma unroll
+              for (int t = 0; t < QT; ++t) a[t] = fmaf(p_s[wave][key][t], v, a[t]);
+            }
           }
         }
 #pragma unroll
