@@ -387,11 +387,27 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(
   }
   const size_t row = (size_t)blockIdx.x * nh + head;  // partial row
   const size_t orow = (size_t)n * nh + head;          // output row (by token)
-  const int used = min(nsplit, positions[n] / split_keys + 1);
+  // Where the partials lie follows from the block alone, how many of them count from the
+  // token's position: the first splits' partials are asked for before the position is known
+  // (one memory round trip instead of three in a row; what a split that does not count left
+  // there is not used).
+  constexpr int kAhead = 8;
   const float* ml = part_ml + row * nsplit * 2;
+  const float* po0 = part_o + row * nsplit * HD;
+  float m_first = -INFINITY, l_first = 0.f;
+  if (lane < nsplit) {
+    m_first = ml[lane * 2];
+    l_first = ml[lane * 2 + 1];
+  }
+  float ahead[kAhead][HD / 64];
+#pragma unroll
+  for (int t = 0; t < kAhead; ++t)
+#pragma unroll
+    for (int i = 0; i < HD / 64; ++i) ahead[t][i] = t < nsplit ? po0[(size_t)t * HD + lane + i * 64] : 0.f;
+  const int used = min(nsplit, positions[n] / split_keys + 1);
   // lane s holds split s's (m, l): one load each, then the maximum over the wave
-  float mx = -INFINITY;
-  for (int s = lane; s < used; s += kWave) mx = fmaxf(mx, ml[s * 2]);
+  float mx = lane < used ? m_first : -INFINITY;
+  for (int s = lane + kWave; s < used; s += kWave) mx = fmaxf(mx, ml[s * 2]);
   mx = wave_max(mx);
   float denom = 0.f;
   float o[HD / 64];
@@ -399,12 +415,24 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(
   for (int i = 0; i < HD / 64; ++i) o[i] = 0.f;
   for (int s0 = 0; s0 < used; s0 += kWave) {
     const int mine = s0 + lane;
-    const float w_mine = mine < used ? fast_exp2(ml[mine * 2] - mx) : 0.f;
-    denom += mine < used ? w_mine * ml[mine * 2 + 1] : 0.f;
+    const float m_mine = s0 == 0 ? m_first : (mine < used ? ml[mine * 2] : 0.f);
+    const float l_mine = s0 == 0 ? l_first : (mine < used ? ml[mine * 2 + 1] : 0.f);
+    const float w_mine = mine < used ? fast_exp2(m_mine - mx) : 0.f;
+    denom += mine < used ? w_mine * l_mine : 0.f;
     const int count = min(kWave, used - s0);
-    const float* po = part_o + (row * nsplit + s0) * HD;
+    const float* po = po0 + (size_t)s0 * HD;
+    int t = 0;
+    if (s0 == 0) {
+#pragma unroll
+      for (; t < kAhead; ++t) {
+        if (t >= count) break;
+        const float w = __shfl(w_mine, t, kWave);
+#pragma unroll
+        for (int i = 0; i < HD / 64; ++i) o[i] = fmaf(w, ahead[t][i], o[i]);
+      }
+    }
 #pragma unroll 4
-    for (int t = 0; t < count; ++t) {
+    for (; t < count; ++t) {
       const float w = __shfl(w_mine, t, kWave);
 #pragma unroll
       for (int i = 0; i < HD / 64; ++i) o[i] = fmaf(w, po[(size_t)t * HD + lane + i * 64], o[i]);
