@@ -100,8 +100,15 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
   const size_t row = rows ? (size_t)rows[m] : (size_t)m;
   float* x = resid + row * H;
   const TD* dl = delta ? delta + row * H : nullptr;
-  float4 xv[kNormGroups];
+  float4 xv[kNormGroups], wv[kNormGroups];
   float ss = 0.f;
+  // the norm's weight is asked for with the stream, not after the rows' sums are known (a
+  // memory round trip less in a kernel that is little else)
+#pragma unroll
+  for (int g = 0; g < kNormGroups; ++g) {
+    const int d = (g * blockDim.x + threadIdx.x) * 4;
+    wv[g] = d < H ? *reinterpret_cast<const float4*>(weight + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
 #pragma unroll
   for (int g = 0; g < kNormGroups; ++g) {
     const int d = (g * blockDim.x + threadIdx.x) * 4;
@@ -110,6 +117,18 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
       float4 v = *reinterpret_cast<const float4*>(x + d);
       if (dl) {
         int p = 0;
+        for (; p + 8 <= parts; p += 8) {   // eight partial sums in flight, added in split order
+          float4 q[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) q[u] = Load4<TD>::at(dl + (size_t)(p + u) * part_stride + d);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            v.x += q[u].x;
+            v.y += q[u].y;
+            v.z += q[u].z;
+            v.w += q[u].w;
+          }
+        }
         for (; p + 4 <= parts; p += 4) {
           const float4 a = Load4<TD>::at(dl + (size_t)p * part_stride + d);
           const float4 b = Load4<TD>::at(dl + (size_t)(p + 1) * part_stride + d);
@@ -140,7 +159,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(
   for (int g = 0; g < kNormGroups; ++g) {
     const int d = (g * blockDim.x + threadIdx.x) * 4;
     if (d < H) {
-      const float4 w = *reinterpret_cast<const float4*>(weight + d);
+      const float4 w = wv[g];
       Store4<T>::at(o + d, make_float4(xv[g].x * rstd * w.x, xv[g].y * rstd * w.y,
                                        xv[g].z * rstd * w.z, xv[g].w * rstd * w.w));
     }
