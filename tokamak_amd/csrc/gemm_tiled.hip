@@ -98,6 +98,116 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const TI* __restrict__ 
   }
 }
 
+// The same product on the matrix cores: v_mfma_f32_32x32x2_f32 multiplies and adds in full
+// float32 and, for every output element, gives exactly the bits of fmaf over its two k in
+// ascending order (measured against the chain on random operands: every output of every
+// step equal), so a walk over k in steps of two is the chain of the kernels above and below,
+// bit for bit, and the pieces of kPiece are kept as they are.  A block of four waves owns
+// 64H x 64H outputs, a wave 32H x 32H of them (H x H tiles of 32 x 32, each 16 accumulators a
+// lane and as many for the total).  The tiles of A and W lie in LDS k-major as above; a lane's
+// operand of a step is one float: A[row lane % 32][k + lane / 32].
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+template <typename TO, int H>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_tiled_mfma_kernel(const float* __restrict__ A,
+                                                              const float* __restrict__ W,
+                                                              TO* __restrict__ C, int M, int N, int K,
+                                                              long lda, long ldw, long ldc) {
+  constexpr int BM = 64 * H, BN = 64 * H;
+  __shared__ __attribute__((aligned(16))) float As[BK][BM + PAD];
+  __shared__ __attribute__((aligned(16))) float Ws[BK][BN + PAD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, g = lane >> 5;
+  const int wm = (wave & 1) * 32 * H, wn = (wave >> 1) * 32 * H;   // this wave's corner of the block's tile
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int lrow = tid / 4, lk = (tid % 4) * 4;   // loader: rows lrow (and lrow + 64), four k from lk
+  // rows whose four k are one aligned 16-byte piece are loaded as one
+  const bool a_wide = lda % 4 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0;
+  const bool w_wide = ldw % 4 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0;
+
+  float16v acc[H][H], total[H][H];
+#pragma unroll
+  for (int i = 0; i < H; ++i)
+#pragma unroll
+    for (int j = 0; j < H; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = total[i][j][e] = 0.f;
+
+  float ar[H][4], wr[H][4];
+  auto fetch = [&](int k0) {
+    const int k = k0 + lk;
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const int m = m0 + lrow + 64 * h, n = n0 + lrow + 64 * h;
+      if (a_wide && m < M && k + 3 < K) {
+        const float4 v = *reinterpret_cast<const float4*>(A + (size_t)m * lda + k);
+        ar[h][0] = v.x; ar[h][1] = v.y; ar[h][2] = v.z; ar[h][3] = v.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ar[h][i] = (m < M && k + i < K) ? A[(size_t)m * lda + k + i] : 0.f;
+      }
+      if (w_wide && n < N && k + 3 < K) {
+        const float4 v = *reinterpret_cast<const float4*>(W + (size_t)n * ldw + k);
+        wr[h][0] = v.x; wr[h][1] = v.y; wr[h][2] = v.z; wr[h][3] = v.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wr[h][i] = (n < N && k + i < K) ? W[(size_t)n * ldw + k + i] : 0.f;
+      }
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    if (k0 > 0 && k0 % kPiece == 0) {
+#pragma unroll
+      for (int i = 0; i < H; ++i)
+#pragma unroll
+        for (int j = 0; j < H; ++j) {
+          total[i][j] += acc[i][j];
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < H; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        As[lk + i][lrow + 64 * h] = ar[h][i];
+        Ws[lk + i][lrow + 64 * h] = wr[h][i];
+      }
+    __syncthreads();
+    if (k0 + BK < K) fetch(k0 + BK);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      float a[H], w[H];
+#pragma unroll
+      for (int h = 0; h < H; ++h) {
+        a[h] = As[kk + g][wm + 32 * h + r];
+        w[h] = Ws[kk + g][wn + 32 * h + r];
+      }
+#pragma unroll
+      for (int i = 0; i < H; ++i)
+#pragma unroll
+        for (int j = 0; j < H; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], w[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  // acc[i][j][4 q + e] = C[m0 + wm + 32 i + 8 q + 4 g + e][n0 + wn + 32 j + r]
+#pragma unroll
+  for (int i = 0; i < H; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = m0 + wm + 32 * i + 8 * q + 4 * g + e;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < H; ++j) {
+          const int n = n0 + wn + 32 * j + r;
+          if (n < N) Elem<TO>::store(C + (size_t)m * ldc + n, total[i][j][4 * q + e] + acc[i][j][4 * q + e]);
+        }
+      }
+}
+
 // Few rows (M <= 16, float32): the tiles above leave most of a block idle.  Here a lane owns
 // one weight row and walks it with 16-byte loads, a cache line in eight loads one after the other; the activations are the same for every lane
 // (the compiler reads them through the scalar path).  The order of the sum is the one of the
@@ -205,7 +315,11 @@ TK_API int tk_gemm_tiled(int in_dtype, int out_dtype, const void* A, const void*
       gemm_tiled_kernel<TI_, TO_, 1><<<grid, 256, 0, stream>>>((const TI_*)A, (const TI_*)W,       \
                                                                (TO_*)C, M, N, K, lda, ldw, ldc);   \
   }
-  if (in_dtype == 0 && out_dtype == 0) TK_TILED(float, float)
+  if (in_dtype == 0 && out_dtype == 0) {
+    // float32 operands: the matrix-core form (the same bits)
+    if (H == 2) gemm_tiled_mfma_kernel<float, 2><<<grid, 256, 0, stream>>>((const float*)A, (const float*)W, (float*)C, M, N, K, lda, ldw, ldc);
+    else gemm_tiled_mfma_kernel<float, 1><<<grid, 256, 0, stream>>>((const float*)A, (const float*)W, (float*)C, M, N, K, lda, ldw, ldc);
+  }
   else if (in_dtype == 1 && out_dtype == 1) TK_TILED(bf16_t, bf16_t)
   else if (in_dtype == 1 && out_dtype == 0) TK_TILED(bf16_t, float)
   else return -1;
