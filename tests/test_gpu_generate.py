@@ -284,6 +284,55 @@ def test_captured_decode_steps_equal_eager_ones_on_every_replay(folders, dtype):
     assert sum(g.replays for g in graphed._graphs.values()) == 40 - len(graphed._graphs)
 
 
+def test_nothing_is_garbage_collected_while_a_step_is_recorded(folders):
+    """Cyclic garbage that owns GPU objects of its own (an older runner's recorded steps) may not
+    be destroyed in the middle of a recording: the HIP runtime ends the process when a recorded
+    step is destroyed then.  Collection is therefore off while a step is recorded.  Here every
+    allocation would start a collection (threshold 1), an older runner with recorded steps is
+    garbage in a cycle, and a new runner records a step: no collection starts while the stream
+    is being recorded, and the step gives the eager runner's logits."""
+    import gc
+
+    from tokamak_amd.engine.runner import ModelRunner, StepEntry
+
+    folder = folders["C"]
+    cfg, _ = plain.read_folder(folder)
+    kw = dict(dtype="bfloat16", page_size=16, kv_pool_tokens=512, max_requests=4)
+    prompt = random_ids(cfg["vocab_size"], 20, 5)
+
+    old = ModelRunner.from_folder(folder, use_graphs=True, **kw)
+    old.step([StepEntry("a", prompt, [])])
+    for token in (3, 4, 5):
+        old.step([StepEntry("a", [token], [0])])
+    assert old._graphs and sum(g.replays for g in old._graphs.values()) >= 2
+    old.myself = old            # only a collection can free it now
+    del old
+
+    new = ModelRunner.from_folder(folder, use_graphs=True, **kw)
+    eager = ModelRunner.from_folder(folder, use_graphs=False, **kw)
+    for runner in (new, eager):
+        runner.step([StepEntry("a", prompt, [])])
+    during = []
+
+    def watch(phase, info):
+        if phase == "start" and torch.cuda.is_current_stream_capturing():
+            during.append(info)
+
+    threshold = gc.get_threshold()
+    gc.callbacks.append(watch)
+    gc.set_threshold(1, 1, 1)
+    try:
+        got = [new.step([StepEntry("a", [token], [0])]).clone() for token in (3, 4, 5)]
+    finally:
+        gc.set_threshold(*threshold)
+        gc.callbacks.remove(watch)
+    assert new._graphs and not during, "a collection started while a step was being recorded"
+    assert gc.isenabled()
+    for token, have in zip((3, 4, 5), got):
+        assert torch.equal(have, eager.step([StepEntry("a", [token], [0])]))
+    gc.collect()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_captured_decode_steps_queued_without_a_host_sync(folders, dtype):
     """Forced tokens, nothing wanted, no synchronisation between steps: the host packs

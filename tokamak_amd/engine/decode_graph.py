@@ -15,6 +15,8 @@ token exactly once, whether its step was the recorded one or a replay.
 
 from __future__ import annotations
 
+import gc
+
 import torch
 
 from tokamak_amd.engine.batch import PackedBatch, batch_from_device
@@ -54,8 +56,20 @@ class DecodeGraph:
         torch.cuda.reset_peak_memory_stats(device)
         before = torch.cuda.memory_allocated(device)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self.logits = model.forward(self.batch, storage)
+        # No garbage collection while the stream is being recorded: a collection that starts in
+        # the middle of the step (any allocation may start one) can free cyclic garbage that
+        # owns GPU objects of its own, an older runner's recorded steps say, and destroying
+        # those is not allowed during a recording: the HIP runtime then ends the process.
+        # (torch collects once before the recording starts; what the step itself drops goes
+        # by reference count as always.)
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                self.logits = model.forward(self.batch, storage)
+        finally:
+            if collecting:
+                gc.enable()
         self.bytes = max(0, torch.cuda.max_memory_allocated(device) - before) + self.size * 4
         self.replays = 0
 
