@@ -521,17 +521,30 @@ def test_streaming_product_and_its_partial_sums(M, N, K):
     """The LDS-staged weight-streaming kernel, unsplit and split over K: the
     partial sums add up to the product, whoever adds them."""
     from tokamak_amd.kernels import ops
+    check_streaming_product(ops, M, N, K, 0)
+
+
+@pytest.mark.parametrize("M, N, K", [(64, 6144, 4096), (49, 200, 520), (40, 97, 264), (3, 96, 64), (24, 1000, 1024)])
+@pytest.mark.parametrize("waves", [4, 6, 8])
+def test_streaming_product_with_every_block_size(M, N, K, waves):
+    """Blocks of four, six and eight waves (64, 96 and 128 weight rows): with six, a chunk of
+    the activations does not divide evenly among the block's threads."""
+    from tokamak_amd.kernels import ops
+    check_streaming_product(ops, M, N, K, waves)
+
+
+def check_streaming_product(ops, M, N, K, waves):
 
     x = rand(M, K, seed=1).to(torch.bfloat16)
     w = rand(N, K, seed=2, scale=K ** -0.5).to(torch.bfloat16)
     want = x.double() @ w.double().T
     for out_dtype, tol in ((torch.float32, dict(rtol=1e-3, atol=1e-3)), (torch.bfloat16, dict(rtol=2e-2, atol=1e-2))):
         out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
-        assert ops.gemm_stream(x.to(DEV), w.to(DEV), out) == 1
+        assert ops.gemm_stream(x.to(DEV), w.to(DEV), out, waves=waves) == 1
         torch.testing.assert_close(out.cpu().double(), want, **tol)
     for splits in (2, 3, 8):
         parts = torch.full((splits, M, N), float("nan"), device=DEV)
-        used = ops.gemm_stream(x.to(DEV), w.to(DEV), parts, splits=splits)
+        used = ops.gemm_stream(x.to(DEV), w.to(DEV), parts, splits=splits, waves=waves)
         assert 1 <= used <= splits
         torch.testing.assert_close(parts[:used].sum(0).cpu().double(), want, rtol=1e-3, atol=1e-3)
         if used > 1:
@@ -603,8 +616,8 @@ def test_consumers_add_partial_sums():
     assert outs[0][2].abs().max() > 0
 
 
-@pytest.mark.parametrize("M, I, K", [(1, 64, 64), (8, 12288, 4096), (64, 200, 96), (33, 3072, 1024), (17, 136, 120)])
-@pytest.mark.parametrize("waves", [0, 2, 4, 8], ids=["chosen", "two waves", "four", "eight"])
+@pytest.mark.parametrize("M, I, K", [(1, 64, 64), (8, 12288, 4096), (64, 200, 96), (33, 3072, 1024), (17, 136, 120), (64, 12288, 4096), (50, 1000, 520)])
+@pytest.mark.parametrize("waves", [0, 2, 4, 6, 8], ids=["chosen", "two waves", "four", "six", "eight"])
 def test_fused_gate_up_silu_product(M, I, K, waves):
     from tokamak_amd.kernels import ops
 

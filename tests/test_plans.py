@@ -15,7 +15,7 @@ SHAPES = [(4096, 1024), (1024, 2048), (1024, 3072), (6144, 2560), (2560, 9728), 
 def test_splits_stay_within_the_chunks_and_fill_the_gpu_evenly(n, k, m):
     chunks = -(-k // 256)
     waves = ops.stream_waves(m, k, False, n)
-    assert waves in (4, 8)
+    assert waves in (4, 6, 8)
     splits = stream_splits(n, k, m)
     assert 1 <= splits <= max(1, chunks)
     blocks = -(-n // (16 * waves))
@@ -24,7 +24,12 @@ def test_splits_stay_within_the_chunks_and_fill_the_gpu_evenly(n, k, m):
         limit = STREAM_TARGET_BLOCKS * 9 // 8 if waves == 4 else STREAM_TARGET_BLOCKS // 2
         assert splits == 1 or splits * blocks <= limit
         assert splits == 1 or chunks // splits >= 2
-        assert waves == (8 if m > 32 and n <= 256 * 128 else 4)
+        if m > 32 and n <= 256 * 128:
+            # six waves only where one round of them covers a tenth more of the CUs than one of eight
+            six, eight = ops.stream_fill(n, k, 6)[0], ops.stream_fill(n, k, 8)[0]
+            assert waves == (6 if six >= 1.1 * eight else 8)
+        else:
+            assert waves == 4
     else:
         assert waves == 4
 
@@ -34,10 +39,20 @@ def test_the_gated_product_picks_its_block_size_by_rows_columns_and_row_length()
     cases = {
         (1, 1024, 3072): 2, (16, 1024, 3072): 2, (48, 1024, 3072): 2, (64, 1024, 3072): 4,       # 0.6B
         (8, 2048, 6144): 2, (32, 2048, 6144): 2, (48, 2048, 6144): 2, (64, 2048, 6144): 4,        # 1.7B
-        (8, 2560, 9728): 2, (32, 2560, 9728): 2, (48, 2560, 9728): 8,                             # 4B
-        (1, 4096, 12288): 4, (16, 4096, 12288): 4, (32, 4096, 12288): 4, (64, 4096, 12288): 8,    # 8B: rows of 8 KB
-        (8, 5120, 17408): 2, (24, 5120, 17408): 4, (64, 5120, 17408): 8,                          # 14B
+        (8, 2560, 9728): 2, (32, 2560, 9728): 2, (48, 2560, 9728): 6,                             # 4B
+        (1, 4096, 12288): 4, (16, 4096, 12288): 4, (32, 4096, 12288): 4, (64, 4096, 12288): 6,    # 8B: rows of 8 KB; 256 blocks of six
+        (8, 5120, 17408): 2, (24, 5120, 17408): 4, (64, 5120, 17408): 6,                          # 14B
         (8, 5120, 25600): 2, (32, 5120, 25600): 4, (33, 5120, 25600): 8,                          # 32B
     }
     for (rows, k, n), waves in cases.items():
         assert ops.stream_waves(rows, k, True, n) == waves, (rows, k, n)
+
+
+def test_six_waves_where_they_fill_the_gpu_better():
+    # q/k/v of an 8B-shaped layer: 64 row blocks of six waves x 4 shares of K = 256 blocks, of eight 48 x 4
+    assert ops.stream_fill(6144, 4096, 6) == (1.0, 4) and ops.stream_fill(6144, 4096, 8) == (0.75, 4)
+    assert ops.stream_waves(64, 4096, False, 6144) == 6 and stream_splits(6144, 4096, 64) == 4
+    # o and down of the same layer are 256 blocks of eight already
+    assert ops.stream_waves(64, 4096, False, 4096) == 8 and ops.stream_waves(64, 12288, False, 4096) == 8
+    # the gated product at 32B: three rounds of six lose to two of eight
+    assert ops.stream_waves(64, 5120, True, 25600) == 8

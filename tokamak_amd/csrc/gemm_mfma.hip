@@ -249,14 +249,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, TO* __restrict__ C, int M, int N,
     int K, long lda, long ldw, long ldc, int chunks_per_split, long split_stride, RowScale scale) {
   constexpr int THREADS = WAVES * 64;
-  constexpr int XP = 16 * MT * 32 / THREADS;  // 16-byte pieces of the activations a thread loads per chunk
-  static_assert(XP * THREADS == 16 * MT * 32, "the activations' chunk divides among the threads");
+  constexpr int XP = (16 * MT * 32 + THREADS - 1) / THREADS;  // 16-byte pieces of the activations a thread loads per chunk
+  constexpr bool XWHOLE = XP * THREADS == 16 * MT * 32;       // else the last piece of some threads lies past the chunk
+  static_assert(WAVES % 2 == 0, "waves load the weights' pieces in pairs of rows and the gated form halves them");
   constexpr int HALF = WAVES / 2;
   // XBUF: copies of the activations' chunk.  A wave reads weights from its own tile only, so with
   // two copies written in turn one barrier a chunk is enough (a wave may start to write chunk
   // i + 1 while others still read chunk i): 3-6 % for blocks of eight waves, which have a CU to
   // themselves anyway; nothing at up to 16 rows, and blocks of four would lose a place on the CU.
-  constexpr int XBUF = (WAVES == 8 && MT >= 2) ? 2 : 1;
+  constexpr int XBUF = (WAVES >= 6 && MT >= 2) ? 2 : 1;
   __shared__ __attribute__((aligned(16))) bf16_t ws[WAVES][16][SLD];
   __shared__ __attribute__((aligned(16))) bf16_t xs[XBUF][16 * MT][SLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -330,6 +331,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
     {                                                                                               \
       const bool inside_ = cur_ * SBK + x_col < K;                                                  \
       _Pragma("unroll") for (int i = 0; i < XP; ++i)                                                \
+        if (XWHOLE || i * (THREADS / 32) + x_row0 < 16 * MT)                                        \
           *reinterpret_cast<u32x4*>(&xs[xb_][i * (THREADS / 32) + x_row0][x_col]) = inside_ ? xreg[i] : zero; \
     }                                                                                               \
     __syncthreads();                                                                                \
@@ -456,13 +458,16 @@ static int launch_stream_shape(const void* A, const void* W, void* C, int M, int
   return launch_status();
 }
 
-// waves: 4 or 8 a block; the gated product also 2.
+// waves: 4, 6 or 8 a block; the gated product also 2.
 template <typename TO, bool GATED>
 static int launch_stream(int waves, const void* A, const void* W, void* C, int M, int N, int K,
                          long lda, long ldw, long ldc, int cps, int KS, long split_stride, RowScale scale,
                          hipStream_t stream) {
   if (waves >= 8)
     return launch_stream_shape<TO, GATED, 8>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, scale, stream);
+  // six waves (96 weight rows a block): for matrices whose rows divide over the CUs that way
+  if (waves == 6)
+    return launch_stream_shape<TO, GATED, 6>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, scale, stream);
   if constexpr (GATED) {
     // two waves (one gate tile, one up tile: 16 output columns a block): more, smaller blocks
     if (waves == 2)
@@ -481,7 +486,7 @@ TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, 
                           const float* sumsq, int slabs, float eps, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535) return -1;
-  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 8)) return -1;
+  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 6)) return -1;
   const RowScale scale{sumsq, slabs, eps};
   if (splits > 1 && out_dtype != 0) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
@@ -499,7 +504,7 @@ TK_API int tk_gemm_stream_swiglu(const void* A, const void* W, void* C, int M, i
                                  hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
-  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 8)) return -1;
+  if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 6)) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
   return launch_stream<bf16_t, true>(waves, A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0,
                                      RowScale{sumsq, slabs, eps}, stream);

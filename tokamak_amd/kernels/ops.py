@@ -484,7 +484,15 @@ def stream_waves(rows: int, k: int, gated: bool = False, n: int = 0) -> int:
     take four waves where two would do: twice as many row tiles in flight at equal offsets
     meet the same memory channels (gate/up of an 8B-shaped layer, K = 4096, at 8 rows: 38 us
     with two waves, 34 with four; with K = 3840 or 4352 two waves are 9 % ahead).  Measured on
-    the shapes of 0.6B to 32B models at 1 to 64 rows: two waves gain 5 to 20 % where chosen."""
+    the shapes of 0.6B to 32B models at 1 to 64 rows: two waves gain 5 to 20 % where chosen.
+
+    Where eight waves are the rule, six (96 weight rows a block) are taken instead if the blocks
+    then fill the CUs better: one block of either size runs on a CU at a time, so the gated
+    product takes the size whose rounds of blocks times rows a block is smaller (gate/up of an
+    8B-shaped layer: 192 blocks of eight leave a quarter of the CUs idle, 256 blocks of six none:
+    44 -> 42 us at 64 rows; 4B 29.6 -> 26.9, 14B 107 -> 94; at 32B three rounds of six lose to two
+    of eight), and the plain product six only if, with the best split of K for each, one round of
+    them covers a tenth more of the CUs (q/k/v of 8B: 64 x 4 blocks against 48 x 4)."""
     if gated:
         if rows <= 16:
             waves = 2
@@ -496,8 +504,33 @@ def stream_waves(rows: int, k: int, gated: bool = False, n: int = 0) -> int:
             waves = 4 if n < 8192 else 8
         if waves == 2 and (2 * k) % 8192 == 0:
             waves = 4
+        if waves == 8 and _rounds(n, 8 * 6) * 6 < _rounds(n, 8 * 8) * 8:
+            waves = 6
         return waves
-    return 8 if rows > 32 and n <= 256 * 128 and 2 * n * k >= STREAM_SMALL_MATRIX_BYTES else 4
+    if rows > 32 and n <= 256 * 128 and 2 * n * k >= STREAM_SMALL_MATRIX_BYTES:
+        return 6 if stream_fill(n, k, 6)[0] >= 1.1 * stream_fill(n, k, 8)[0] else 8
+    return 4
+
+
+STREAM_CUS = 256    # blocks of six or eight waves that run at once: one a CU
+
+
+def _rounds(n: int, columns: int) -> int:
+    return -(-(-(-n // columns)) // STREAM_CUS)
+
+
+def stream_fill(n: int, k: int, waves: int) -> tuple[float, int]:
+    """(share of the CUs that one round of ``waves``-wave blocks covers, shares of K that do it):
+    the split of K, of at least two chunks of 256 a share, whose blocks come closest to one a CU
+    without exceeding it."""
+    blocks = -(-n // (16 * waves))
+    chunks = -(-k // 256)
+    best, best_splits = min(blocks, STREAM_CUS), 1
+    for per in range(2, chunks + 1):
+        splits = -(-chunks // per)
+        if best < blocks * splits <= STREAM_CUS:
+            best, best_splits = blocks * splits, splits
+    return best / STREAM_CUS, best_splits
 
 
 def _row_scale(sumsq: torch.Tensor | None, m: int, what: str) -> int:
@@ -514,7 +547,7 @@ def _row_scale(sumsq: torch.Tensor | None, m: int, what: str) -> int:
 def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: int = 1, waves: int = 0,
                 sumsq: torch.Tensor | None = None, eps: float = 0.0) -> int:
     """out = a[M, K] @ w[N, K]^T for M <= 64 with the LDS-staged weight-streaming
-    MFMA kernel (``waves``: 4 or 8 waves a block; 0 chooses by M).  ``splits == 1``: out is
+    MFMA kernel (``waves``: 4, 6 or 8 waves a block; 0 chooses by the shape).  ``splits == 1``: out is
     [M, N], bfloat16 or float32.  More:
     out is float32 [splits, M, N] and receives partial sums; returns how many of
     them were written (the reader adds out[:returned]).  ``sumsq`` [slabs, M] (M <= 16): row m
