@@ -216,6 +216,10 @@ TK_API int tk_gemm_skinny(int out_dtype, const void* A, const void* W, void* C, 
 // the copies in split order.  No block waits for, or signals, another.
 // ---------------------------------------------------------------------------
 constexpr int SBK = 256;        // k per chunk
+// Row tiles of activations from which a chunk's operand reads are asked for ahead of the
+// products (sched_group_barrier below).  With one row tile the plain loop is kept: the read-ahead
+// gains nothing there and cost the two-wave gated product of a 14B-shaped layer 8 % (63 -> 68 us).
+constexpr int READ_AHEAD_FROM = 2;
 constexpr int SLD = SBK + 8;    // LDS row stride in elements
 
 // GATED: W is [2N, K], gate rows then up rows; the block owns 8*WAVES output columns, the
@@ -340,7 +344,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
       TK_FETCH_W(next_)                                                                             \
       TK_FETCH_X(next_)                                                                             \
     }                                                                                               \
-    {                                                                                               \
+    if constexpr (MT < READ_AHEAD_FROM) {                                                           \
+      _Pragma("unroll") for (int s = 0; s < SBK / 32; ++s) {                                        \
+        Frag8 wf, xf[MT];                                                                           \
+        wf.u = *reinterpret_cast<const uint4*>(&ws[wave][r][s * 32 + kb * 8]);                      \
+        _Pragma("unroll") for (int j = 0; j < MT; ++j)                                              \
+            xf[j].u = *reinterpret_cast<const uint4*>(&xs[xb_][j * 16 + r][s * 32 + kb * 8]);       \
+        _Pragma("unroll") for (int j = 0; j < MT; ++j)                                              \
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf[j].v, acc[j], 0, 0, 0);       \
+      }                                                                                             \
+    } else {                                                                                        \
       /* the fragments of a step of 32 k are asked for while the step before is multiplied: a    */ \
       /* wave that waits for each fragment in turn spends its time on round trips to LDS         */ \
       Frag8 wf[SBK / 32], xf[SBK / 32][MT];                                                         \
