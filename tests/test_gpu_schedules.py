@@ -315,13 +315,15 @@ def test_layers_launched_from_a_recorded_layer_give_the_same_bits(dtype):
         # ... and once more with the lists issued call by call from Python (what a recording falls
         # back to when an entry point has no slot form)
         layer_replay.LayerRecording.launch = lambda self, tensors, then: (
-            setattr(self, "packed", None), launch(self, tensors, then))[1]
+            setattr(self, "pack_tried", True), launch(self, tensors, then))[1]
         by_call, cache_by_call = run(True)
     finally:
         layer_replay.LayerRecording.launch = launch
     assert len(launched) == 5 * (cfg.num_layers - 2), "three of five layers of every step are launched from the list"
     assert min(launched) >= 5
-    assert all(packed), "every list was issued by one foreign call (csrc/replay.hip)"
+    # a list is issued call by call at its first replay and packed behind it: of the three replayed
+    # layers of a step the second and third go out in one foreign call each (csrc/replay.hip)
+    assert packed == [False, True, True] * 5, packed
     for a, b in zip(replayed, by_call):
         assert torch.equal(a, b)
     for a, b in zip(cache_replayed, cache_by_call):
