@@ -497,7 +497,7 @@ def test_float32_product_is_true_32_bit_and_row_independent():
 
 
 @pytest.mark.parametrize("M, N, K", [(1, 64, 64), (3, 331, 200), (8, 1000, 4096), (16, 77, 1028), (17, 130, 516),
-                                     (40, 200, 260), (64, 65, 12), (5, 70000, 264)])
+                                     (40, 200, 260), (64, 65, 12), (5, 70000, 264), (50, 16500, 264), (24, 66000, 40)])
 def test_float32_product_of_few_rows_equals_the_tiled_one_bit_for_bit(M, N, K):
     """Up to 64 rows the float32 product streams the weights (a lane a weight row, a wave a
     piece of K or all of them); it sums in the tiled kernel's order, so the same rows inside
@@ -514,6 +514,9 @@ def test_float32_product_of_few_rows_equals_the_tiled_one_bit_for_bit(M, N, K):
             out = torch.full((M, N), float("nan"), device=DEV)
             ops.gemm_tiled(x[at:at + M].to(DEV), w.to(DEV), out, fewrows_split=split)
             assert torch.equal(out, whole[at:at + M]), (at, split)
+    # many rows of activations over a matrix with a tile for every CU take the tiled kernel itself
+    assert ops.fewrows_pays(64, 4096) and ops.fewrows_pays(16, 200000) and ops.fewrows_pays(40, 16000)
+    assert not ops.fewrows_pays(48, 16384) and not ops.fewrows_pays(24, 65536)
 
 
 @pytest.mark.parametrize("M, N, K", [(1, 64, 64), (8, 6144, 4096), (64, 4096, 4096), (33, 331, 200), (17, 4096, 12288), (64, 1000, 264)])

@@ -436,10 +436,25 @@ FEWROWS_GROUP = 16             # this many rows a pass over the weights
 FEWROWS_SPLIT_BELOW = 65536    # weight rows below which every piece of 256 k gets a wave of its own
 
 
+def fewrows_pays(m: int, n: int) -> bool:
+    """Whether ``m`` rows stream the weights (one pass per FEWROWS_GROUP rows) rather than take
+    the tiled kernel in tiles of 64 x 64, which reads the weights once but needs a block for
+    every CU to be worth it: measured on the shapes of an 8B-shaped layer, the tiled kernel wins
+    from 24 rows where it has a thousand tiles (the logits head at 64 rows: 4.7 -> 1.6 ms) and
+    from 48 where it has one a CU (gate/up: 546 -> 303 us); a matrix of 4,096 rows never."""
+    tiles = -(-n // 64)
+    if m >= 48 and tiles >= 256:
+        return False
+    if m >= 24 and tiles >= 1024:
+        return False
+    return True
+
+
 def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, fewrows_split: bool | None = None) -> None:
     """out[M, N] = a[M, K] @ w[N, K]^T, float32 multiply-add (rows may be strided).  float32
-    operands of up to 64 rows go to the weight-streaming kernel, which gives the same bits
-    (``fewrows_split``: a wave per piece of K or not; None chooses by the matrix's rows)."""
+    operands of up to 64 rows go to the weight-streaming kernel where that pays
+    (``fewrows_pays``), which gives the same bits (``fewrows_split``: that kernel with a wave
+    per piece of K or not; None chooses the kernel and the split by the shape)."""
     for t in (a, w, out):
         _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1, "gemm operands are 2-D GPU tensors with unit inner stride")
     m, k = a.shape
@@ -448,7 +463,8 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, fewrows_spli
     _need(a.dtype == w.dtype, "gemm inputs must share a dtype")
     _need(m <= 64 * 65535, "too many rows for one launch")
     _note(f"{m}x{n}x{k}", (n * k + m * k) * a.element_size() + m * n * out.element_size(), 2.0 * m * n * k)
-    if (m <= FEWROWS_MAX_ROWS and a.dtype == torch.float32 and out.dtype == torch.float32 and k % 4 == 0 and k >= 4
+    if (m <= FEWROWS_MAX_ROWS and (fewrows_split is not None or fewrows_pays(m, n))
+            and a.dtype == torch.float32 and out.dtype == torch.float32 and k % 4 == 0 and k >= 4
             and a.stride(0) % 4 == 0 and w.stride(0) % 4 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
         # the same sums in the same order, by a kernel that streams the weights; a wave for every
         # piece of K where the matrix has too few rows to fill the GPU with a wave per 64 of them
