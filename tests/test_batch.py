@@ -47,6 +47,9 @@ def test_the_attention_kernels_lists_are_made_by_their_planner():
     rows = lists["attention.single"] + [f + i for f, c in zip(lists["attention.tile_first"], lists["attention.tile_count"])
                                         for i in range(c)]
     assert sorted(rows) == list(range(batch.num_tokens))
+    # single tokens are listed longest context first (blocks start in that order), ties in step order
+    mixed = unpack(pack_batch(spans_of((1, 7), (1, 300), (2, 5), (1, 300), (1, 41)), 1, [ATTENTION_WORK]))
+    assert mixed.lists["attention.single"].tolist() == [1, 4, 5, 0]
 
 
 def test_a_recorded_step_rounds_the_facts_as_the_planner_asks():

@@ -40,7 +40,7 @@ def quarter_octave_at_least(n: int, floor: int) -> int:
 
 class AttentionWork(StepPlanner):
     """The attention kernels' cut of a step: spans of one token run alone (``single``: their
-    token rows), longer spans are cut into tiles of up to 16 consecutive tokens
+    token rows, the one with the longest context first), longer spans are cut into tiles of up to 16 consecutive tokens
     (``tile_first``, ``tile_count``) and, for the wide kernel, of up to 32 (``wide_first``,
     ``wide_count``).  Facts: how many of each, the tokens in tiled spans, the longest
     context among the single tokens (it fixes how their keys are split), the longest
@@ -51,13 +51,17 @@ class AttentionWork(StepPlanner):
     def lists(self, q_lens, ctx_lens):
         single, tiles, wide = [], [], []
         at = 0
-        for q in q_lens:
+        for q, ctx in zip(q_lens, ctx_lens):
             if q == 1:
-                single.append(at)
+                single.append((-ctx, at))
             else:
                 tiles.extend((at + t, min(TILE_TOKENS, q - t)) for t in range(0, q, TILE_TOKENS))
                 wide.extend((at + t, min(WIDE_TOKENS, q - t)) for t in range(0, q, WIDE_TOKENS))
             at += q
+        # Longest context first: blocks start in the list's order, and a long walk that starts
+        # last is what the whole kernel waits for (50 requests of 48 to 1,280 keys, 16 query heads
+        # over 8 kv heads: 33 us in the order of the requests, 25 longest first).
+        single = [row for _, row in sorted(single)]
         arrays = {"single": single, "tile_first": [t[0] for t in tiles], "tile_count": [t[1] for t in tiles],
                   "wide_first": [t[0] for t in wide], "wide_count": [t[1] for t in wide]}
         tiled = [(q, c) for q, c in zip(q_lens, ctx_lens) if q > 1]
