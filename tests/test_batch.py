@@ -38,8 +38,9 @@ def test_the_attention_kernels_lists_are_made_by_their_planner():
     batch = unpack(packed)
     lists = {k: v.tolist() for k, v in batch.lists.items()}
     assert lists["attention.single"] == [40, 41]
-    assert lists["attention.tile_first"] == [0, 16, 32, 42, 58] and lists["attention.tile_count"] == [16, 16, 8, 16, 1]
-    assert lists["attention.wide_first"] == [0, 32, 42] and lists["attention.wide_count"] == [32, 8, 17]
+    # tiles by the keys they walk, shortest first (the kernels start from the list's end)
+    assert lists["attention.tile_first"] == [42, 58, 0, 16, 32] and lists["attention.tile_count"] == [16, 1, 16, 16, 8]
+    assert lists["attention.wide_first"] == [42, 0, 32] and lists["attention.wide_count"] == [17, 32, 8]
     assert batch.facts == {"attention.num_single": 2, "attention.num_tiles": 5, "attention.num_wide": 3,
                            "attention.num_tile_tokens": 57, "attention.max_single_len": 301,
                            "attention.max_tile_len": 140, "attention.min_tile_ctx": 0}

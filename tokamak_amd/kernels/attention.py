@@ -55,13 +55,18 @@ class AttentionWork(StepPlanner):
             if q == 1:
                 single.append((-ctx, at))
             else:
-                tiles.extend((at + t, min(TILE_TOKENS, q - t)) for t in range(0, q, TILE_TOKENS))
-                wide.extend((at + t, min(WIDE_TOKENS, q - t)) for t in range(0, q, WIDE_TOKENS))
+                tiles.extend((ctx + t, at + t, min(TILE_TOKENS, q - t)) for t in range(0, q, TILE_TOKENS))
+                wide.extend((ctx + t, at + t, min(WIDE_TOKENS, q - t)) for t in range(0, q, WIDE_TOKENS))
             at += q
         # Longest context first: blocks start in the list's order, and a long walk that starts
         # last is what the whole kernel waits for (50 requests of 48 to 1,280 keys, 16 query heads
         # over 8 kv heads: 33 us in the order of the requests, 25 longest first).
         single = [row for _, row in sorted(single)]
+        # Tiles by the keys they walk, shortest first: the kernels take the list from its end (as
+        # they do for one prompt from position zero, whose later tiles walk further), so that the
+        # tiles of several requests' portions start longest first too.
+        tiles = [t[1:] for t in sorted(tiles)]
+        wide = [t[1:] for t in sorted(wide)]
         arrays = {"single": single, "tile_first": [t[0] for t in tiles], "tile_count": [t[1] for t in tiles],
                   "wide_first": [t[0] for t in wide], "wide_count": [t[1] for t in wide]}
         tiled = [(q, c) for q, c in zip(q_lens, ctx_lens) if q > 1]
