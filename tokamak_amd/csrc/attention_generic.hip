@@ -199,7 +199,7 @@ __global__ __launch_bounds__(kWaves * kWave) void paged_attention_generic_kernel
         m[t] = m_new;
       }
     }
-    wave_lds_sync();   // the wave has read its last round's probabilities
+    wave_lds_sync();   // the wave has read the probabilities of the 64 keys before
 #pragma unroll
     for (int t = 0; t < QT; ++t) p_s[wave][lane][t] = p[t];
     if (!BATCHED) base_s[wave][lane] = vbase;
