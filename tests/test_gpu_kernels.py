@@ -157,7 +157,7 @@ def test_tiles_of_32_tokens_for_long_walks(nh, nkv, hd, ps, monkeypatch):
     from tokamak_amd.kernels import attention
 
     monkeypatch.setattr(attention, "WIDE_FROM_KEYS", 64)
-    monkeypatch.setattr(attention, "GROUP_FROM_KEYS", 64)
+    monkeypatch.setattr(attention, "group_form_pays", lambda group, *rest: group >= 3)
     requests = [(0, 200), (37, 150), (900, 33), (5, 32), (300, 1), (0, 450)]
     tiles = [q for _, q in requests if q > 1]
     assert sum(tiles) >= attention.WIDE_FROM_TOKENS * sum(-(-q // 32) for q in tiles)
@@ -172,13 +172,18 @@ def test_tiles_of_32_tokens_for_long_walks(nh, nkv, hd, ps, monkeypatch):
 
 
 @pytest.mark.parametrize("nh, nkv", [(8, 2), (4, 2), (5, 1)])
-def test_tiles_of_32_tokens_find_a_far_key_and_respect_the_causal_edge(nh, nkv):
+def test_tiles_of_32_tokens_find_a_far_key_and_respect_the_causal_edge(nh, nkv, monkeypatch):
     """The group form (and for groups of two the wide form) on inputs made to show faults: one key far back dominates one query's
     softmax (its value must come out), and the key right after a query's position is made
-    enormous (reading it would show)."""
+    enormous (reading it would show).  (Three tiles are too few for these forms to be chosen: they are asked for.)"""
     from tokamak_amd.kernels import attention
 
     hd = 128
+    launched = []
+    real = attention.ops.attention_mfma
+    monkeypatch.setattr(attention, "group_form_pays", lambda group, *rest: group >= 3)
+    monkeypatch.setattr(attention, "tile_split", lambda *sizes: (1 << 30, 1))    # (so few tiles would have their keys split)
+    monkeypatch.setattr(attention.ops, "attention_mfma", lambda mode, *a, **k: (launched.append(mode), real(mode, *a, **k))[1])
     seen = {}
 
     def boost(q, k, v, ctx, qlen):
@@ -193,6 +198,7 @@ def test_tiles_of_32_tokens_find_a_far_key_and_respect_the_causal_edge(nh, nkv):
 
     got, want = run_attention(torch.bfloat16, nh, nkv, hd, 16, [(4100, 96)], boost=boost, seed=5)
     assert attention.WIDE_FROM_KEYS <= 4196
+    assert launched == ["tokens_group" if nh // nkv >= 3 else "tokens_wide"]
     torch.testing.assert_close(got[0], want[0], **TOL[torch.bfloat16])
     expected = seen["far"].repeat_interleave(nh // nkv, dim=0)
     torch.testing.assert_close(got[0][40], expected, rtol=0, atol=2e-2)

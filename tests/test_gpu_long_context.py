@@ -121,11 +121,14 @@ def test_a_long_portion_over_the_longest_context(dtype, keys, monkeypatch):
 
 @pytest.mark.parametrize("keys", [32768, 40960])
 def test_a_long_portion_of_pairs_of_heads_over_the_longest_context(keys, monkeypatch):
-    """The same with two query heads a kv head: the wide form."""
+    """The same with two query heads a kv head: the wide form when the tiles are more than the CUs
+    (eight kv heads), the group form with four shares of the keys a block when they are not (four)."""
     ctx = keys - 2048
     targets = [(0, 0), (31, 63), (32, 64), (1000, ctx - 1), (1500, ctx + 1499), (2047, ctx // 3)]
-    launched = run(torch.bfloat16, 8, 4, ctx, 2048, seed=keys + 4, targets=targets, monkeypatch=monkeypatch)
+    launched = run(torch.bfloat16, 16, 8, ctx, 2048, seed=keys + 4, targets=targets, monkeypatch=monkeypatch)
     assert launched == [("tokens_wide", 1)]
+    launched = run(torch.bfloat16, 8, 4, ctx, 2048, seed=keys + 5, targets=targets, monkeypatch=monkeypatch)
+    assert launched == [("tokens_group", 1)]
 
 
 @pytest.mark.parametrize("keys", [32768, 40960])

@@ -56,3 +56,21 @@ def test_six_waves_where_they_fill_the_gpu_better():
     assert ops.stream_waves(64, 4096, False, 4096) == 8 and ops.stream_waves(64, 12288, False, 4096) == 8
     # the gated product at 32B: three rounds of six lose to two of eight
     assert ops.stream_waves(64, 5120, True, 25600) == 8
+
+
+def test_the_group_form_of_prefill_attention_is_taken_where_it_was_measured_to_pay():
+    from tokamak_amd.kernels.attention import group_form_pays
+
+    wide = lambda tokens: -(-tokens // 32)
+    # (query heads a kv head, kv heads, tokens of the portion, longest context) -> group form
+    cases = {
+        (4, 8, 2048, 2048): True, (4, 8, 2048, 32768): True, (4, 8, 256, 1280): True, (4, 8, 128, 5000): False,   # 8B, 4B
+        (4, 8, 2048, 1000): False,                                                                               # short walks
+        (5, 8, 2048, 2048): True, (5, 8, 512, 1536): True, (5, 8, 256, 4352): False, (5, 8, 128, 16512): False,   # 14B: too few blocks
+        (8, 8, 2048, 2048): True, (8, 8, 1024, 1024): False, (8, 8, 1024, 2048): True, (8, 8, 512, 1536): False,  # 32B
+        (8, 8, 512, 4608): True, (8, 8, 256, 16640): False,
+        (2, 8, 512, 4608): True, (2, 8, 1024, 17408): True, (2, 8, 1024, 1024): False, (2, 8, 2048, 6144): False,  # 0.6B, 1.7B
+        (3, 1, 2048, 2048): True, (16, 2, 2048, 2048): True,
+    }
+    for (group, nkv, tokens, longest), want in cases.items():
+        assert group_form_pays(group, nkv, wide(tokens), longest) == want, (group, nkv, tokens, longest)

@@ -22,8 +22,8 @@ DENSE_TILES_FROM = 2048         # every tiled span starts at least this deep: th
 WIDE_FROM_KEYS = 4096           # longest context from which the 32-token tiles of the wide kernel pay (+15-20 %;
                                 # for shorter walks the narrow one's smaller tiles balance better)
 WIDE_FROM_TOKENS = 20           # ... if a 32-token tile holds at least this many tokens on average
-GROUP_FROM_KEYS = 1024          # longest context from which the group form (a block a CU, all heads of a kv head) pays ...
-GROUP_FROM_HEADS = 3            # ... for groups of at least this many query heads a kv head (fewer: too few waves a block)
+GROUP_FROM_KEYS = 1024          # longest context from which the group form (a block a CU, all heads of a kv head) pays
+GROUP_FILL = 128                # ... if its blocks times their shares of the keys are at least this many (half the CUs)
 
 
 def quarter_octave_at_least(n: int, floor: int) -> int:
@@ -165,6 +165,28 @@ def tile_split(num_tiles: int, blocks_per_tile: int, max_len: int) -> tuple[int,
     return split, -(-max_len // split)
 
 
+def group_form_pays(group: int, num_kv_heads: int, num_wide: int, max_len: int) -> bool:
+    """Whether the tiles of a step's portions take the group form (csrc/attention_mfma.hip: a block
+    holds a CU, the query heads of a kv head times 4, 2 or 1 shares of each stage of keys).  Measured
+    against the other forms for 2, 4, 5 and 8 heads a kv head, 64 to 2,048 tokens over 0 to 16,384
+    cached ones: it needs enough blocks to fill the GPU (with few tiles the narrow form, whose
+    tiles are half as long and whose keys can be split over blocks, is up to 40 % ahead); with an
+    odd group it wins from there on (the narrow form computes on one wave of four then); with one
+    share a block it needs the longer walks the fewer its blocks; with two heads a kv head it wins
+    (by 27-35 %) while its blocks are no more than the CUs, beyond that the wide form does."""
+    nblk = -(-group // 8)
+    heads = -(-group // nblk)                   # heads a block
+    shares = 4 if heads <= 2 else 2 if heads <= 4 else 1
+    blocks = num_wide * num_kv_heads * nblk
+    if blocks * shares < GROUP_FILL:
+        return False
+    if group <= 2:
+        return blocks <= 256 and max_len >= 2 * GROUP_FROM_KEYS
+    if group % 2 == 1 or shares >= 2:
+        return max_len >= GROUP_FROM_KEYS
+    return max_len >= 2 * GROUP_FROM_KEYS * max(1, 256 // blocks)
+
+
 def fused_decode_fits(dtype, head_dim, page_size, group, window, rotary_dim, batch) -> bool:
     """A step of decode tokens only, at shapes the one-kernel form takes."""
     work = work_of(batch)
@@ -248,8 +270,8 @@ def _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, *
         group = num_heads // num_kv_heads
         per_tile = num_kv_heads * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
         split, nsplit = tile_split(work.num_tiles, per_tile, work.max_tile_len)
-        if (nsplit == 1 and work.max_tile_len >= GROUP_FROM_KEYS and group >= GROUP_FROM_HEADS
-                and work.num_tile_tokens >= WIDE_FROM_TOKENS * work.num_wide):
+        if (nsplit == 1 and work.num_tile_tokens >= WIDE_FROM_TOKENS * work.num_wide
+                and group_form_pays(group, num_kv_heads, work.num_wide, work.max_tile_len)):
             # tiles of 32 tokens mostly full: the group form, whose blocks hold a CU each
             if note is not None:
                 ops._note(f"portions {work.num_wide} wide tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
