@@ -80,15 +80,19 @@ def test_a_decode_token_over_the_longest_context(dtype, keys, far, monkeypatch):
     """One token over ``keys`` keys (itself the last), pointed at one far key: the first, the
     last of the first split's first wave share, both sides of a split's edge, the one before
     itself."""
-    from tokamak_amd.kernels.attention import decode_split
+    from tokamak_amd.kernels import attention
 
     ctx = keys - 1
     key = far if far >= 0 else ctx + far + 1
-    launched = run(dtype, 8, 2, ctx, 1, seed=keys + (far % 997), targets=[(0, key)],
-                   monkeypatch=monkeypatch if dtype == torch.bfloat16 else None)
-    if dtype == torch.bfloat16:
-        split, nsplit = decode_split(1, 2, keys)
-        assert nsplit > 64 and launched == [("heads", nsplit)]       # the merge walks more than 64 splits
+    chosen = attention.decode_split(1, 2, keys, HD)[1]
+    assert 32 <= chosen <= 64            # as priced: two blocks a split, each split a merge read
+    for finest in (False, True):
+        if finest:                       # and the finest split there is: the merge walks more than 64 splits
+            monkeypatch.setattr(attention, "decode_split", lambda *sizes: (256, keys // 256))
+        launched = run(dtype, 8, 2, ctx, 1, seed=keys + (far % 997), targets=[(0, key)],
+                       monkeypatch=monkeypatch if dtype == torch.bfloat16 else None)
+        if dtype == torch.bfloat16:
+            assert launched == [("heads", keys // 256 if finest else chosen)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])

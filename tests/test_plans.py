@@ -74,3 +74,22 @@ def test_the_group_form_of_prefill_attention_is_taken_where_it_was_measured_to_p
     }
     for (group, nkv, tokens, longest), want in cases.items():
         assert group_form_pays(group, nkv, wide(tokens), longest) == want, (group, nkv, tokens, longest)
+
+
+def test_decode_splits_follow_how_the_blocks_fill_the_rounds():
+    from tokamak_amd.kernels.attention import DECODE_WAVES, decode_split
+
+    for requests in (1, 2, 7, 8, 16, 17, 31, 32, 33, 40, 64):
+        for kv_heads in (1, 2, 8):
+            for longest in (1, 255, 256, 257, 600, 2049, 2560, 8192, 40960):
+                split, nsplit = decode_split(requests, kv_heads, longest)
+                assert split % (16 * DECODE_WAVES) == 0 and nsplit >= 1 and split * nsplit >= longest
+                assert split * (nsplit - 1) < longest            # no split past the longest request
+    # 32 requests x 8 kv heads are one block a CU: no split; one request more is 264 blocks, whose
+    # last eight would take as long again: split, so that the last round is short
+    assert decode_split(32, 8, 2560)[1] == 1 and decode_split(64, 8, 2560)[1] == 1
+    assert decode_split(33, 8, 2560)[1] >= 3
+    # few requests: as many splits as fill the GPU, fewer when each split is only a few tiles long
+    assert decode_split(8, 8, 2560)[1] == 4 and decode_split(1, 8, 2560)[1] >= 8
+    assert decode_split(8, 8, 300)[1] <= 2
+    assert decode_split(1, 2, 32768)[1] >= 32

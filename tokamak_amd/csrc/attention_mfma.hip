@@ -44,6 +44,15 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 constexpr int kDecodeWaves = 16;
 
+// The keys of one split of a decode token whose keys are cut in nsplit: the token's own keys
+// cut evenly (a whole number of 16 keys for every wave of a block), whatever the longest
+// request of the step holds, so that the blocks of a token walk equal shares; splits past the
+// token's last key hold nothing.
+__device__ __forceinline__ int decode_share(int keys, int nsplit) {
+  constexpr int unit = 16 * kDecodeWaves;
+  return ((keys + nsplit - 1) / nsplit + unit - 1) / unit * unit;
+}
+
 // What the fused form of the decode kernel takes instead of finished queries: the q/k/v
 // projection's output as it left the product (`parts` float32 partial sums of a split-K
 // product, part_stride elements apart, or one bfloat16 matrix), rows of (nh + 2 nkv_in)
@@ -129,14 +138,18 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
   // LDS: the waves' accumulators of the group's heads [WAVES][G][HD], then their (m, l) [WAVES][16] each
   extern __shared__ __attribute__((aligned(16))) float s_dyn[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, kb = lane >> 4;
-  const int split = blockIdx.x, item = blockIdx.z;
+  // splits are the slowest index of the grid: blocks start in the grid's order, so a token's
+  // last split (the shortest, or one that holds no key) starts behind every first one
+  const int split = blockIdx.z, item = blockIdx.y;
   const int G = nh / nkv;
-  const int kvh = blockIdx.y;
+  const int kvh = blockIdx.x;
 
   const int n0 = item_token[item];
   const int pos0 = positions[n0];  // the token's position: it sees keys 0 .. pos0
-  const int k_begin = split * split_keys;
-  const int k_end = min(pos0 + 1, k_begin + split_keys);
+  static_assert(WAVES == kDecodeWaves, "decode_share cuts for blocks of kDecodeWaves waves");
+  const int share = nsplit > 1 ? decode_share(pos0 + 1, nsplit) : split_keys;
+  const int k_begin = split * share;
+  const int k_end = min(pos0 + 1, k_begin + share);
   if (k_begin >= k_end) return;  // the whole block: this split holds no key of the token
   const int* table = block_tables + (size_t)req_of_token[n0] * max_pages;
   const size_t page_elems = (size_t)nkv * HD * ps;
@@ -207,7 +220,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_kernel(
     }
     __syncthreads();
     // the block that holds the token's position writes its key and value to the page
-    if (stores && wave == 0 && lane < HD / 2 && k_begin <= pos0 && pos0 < k_begin + split_keys) {
+    if (stores && wave == 0 && lane < HD / 2 && k_begin <= pos0 && pos0 < k_begin + share) {
       const int page = table[pos0 / ps], off = pos0 % ps, d = 2 * lane;
       bf16_t* kp = const_cast<bf16_t*>(k_cache_in) + (size_t)page * page_elems + head_off;
       bf16_t* vp = const_cast<bf16_t*>(v_cache_in) + (size_t)page * page_elems + head_off;
@@ -404,7 +417,9 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(
   for (int t = 0; t < kAhead; ++t)
 #pragma unroll
     for (int i = 0; i < HD / 64; ++i) ahead[t][i] = t < nsplit ? po0[(size_t)t * HD + lane + i * 64] : 0.f;
-  const int used = min(nsplit, positions[n] / split_keys + 1);
+  // splits that hold keys: of a decode token by its own even cut, of a tile by the step's
+  const int pos = positions[n];
+  const int used = min(nsplit, pos / (item_count == nullptr ? decode_share(pos + 1, nsplit) : split_keys) + 1);
   // lane s holds split s's (m, l): one load each, then the maximum over the wave
   float mx = lane < used ? m_first : -INFINITY;
   for (int s = lane + kWave; s < used; s += kWave) mx = fmaxf(mx, ml[s * 2]);
@@ -1354,7 +1369,8 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
                   const int* item_token, const int* item_count, int num_items, void* out,
                   float* part_o, float* part_ml, int nsplit, int split_keys, int nh, int nkv, int ps,
                   float scale, hipStream_t stream, DecodeInputs in = DecodeInputs{}) {
-  dim3 grid(nsplit, nkv, num_items);
+  if (num_items > 65535) return -1;
+  dim3 grid(nkv, num_items, nsplit);
   const int G = nh / nkv;
   // sixteen waves a block and one tile a wave in flight measured best at every batch size
   // (four or eight waves with two tiles: 12 % slower at batch 64, 15 % at batch 8)
@@ -1384,7 +1400,9 @@ static int launch(const void* q, const void* k_cache, const void* v_cache, const
 }
 
 // mode 0: heads (every item is one decode token; item_count is ignored; split_keys is a multiple of
-//         16 * tk_attention_decode_waves(), a tile for every wave of a block)
+//         16 * tk_attention_decode_waves(), a tile for every wave of a block, and nsplit of them
+//         cover the longest token; with nsplit > 1 every token's own keys are cut evenly in
+//         nsplit, see decode_share)
 // mode 1: tokens (item = up to 16 consecutive tokens of one request; with nsplit > 1 split_keys
 //         is a multiple of 64 and the partial buffers hold 16 rows per item)
 // mode 2: tokens, every tile over a long context (same results; the kernel built for four waves a SIMD)

@@ -3,6 +3,9 @@ those kernels read: how a step's spans are cut into single tokens and tiles."""
 
 from __future__ import annotations
 
+import functools
+import math
+
 import torch
 
 from tokamak_amd.kernels import ops
@@ -13,8 +16,6 @@ WIDE_TOKENS = 32   # and per tile of the wide matrix-core kernel
 
 MFMA_HEAD_DIMS = (64, 128)
 DECODE_WAVES = 16           # waves of a decode block (csrc/attention_mfma.hip: kDecodeWaves)
-TARGET_DECODE_WAVES = 4096  # waves wanted in flight; beyond that splits only cost a merge
-MERGE_WORTH_TILES = 2       # tiles of 16 keys a wave must save for a split of the keys to pay for its merge
 TILE_SPLIT_BELOW_BLOCKS = 256   # a portion with fewer blocks than this has its keys split ...
 TILE_SPLIT_MIN_KEYS = 512       # ... into pieces no shorter than this
 TARGET_TILE_BLOCKS = 1024
@@ -125,28 +126,55 @@ def mfma_fits(dtype, head_dim, page_size, group, window) -> bool:
             and page_size & (page_size - 1) == 0 and group <= 16 and window is None)
 
 
-def decode_split(num_decode: int, num_kv_heads: int, max_len: int) -> tuple[int, int]:
+# What the choice of the decode splits is priced with (seconds, bytes a second; fitted to 154
+# measured cases of 9 to 64 requests over 300 to 16,384 keys in 1 to 8 splits and checked on
+# 1 to 8 requests up to 32,768 keys: the cheapest split by this price is on average 1 % and at
+# worst 18 % slower than the best measured one; the rule it replaced, "as few splits as put
+# 4,096 waves on the GPU", 5 % and 49 % on such cases).
+DECODE_CUS = 256                 # blocks that run at once: a block of sixteen waves has a CU to itself
+DECODE_RATE = 5.8e12             # bytes a second of a round of DECODE_CUS blocks
+DECODE_BLOCK_RATE = 60e9         # ... and of one block with the GPU to itself
+DECODE_START = 3e-6              # a launch
+DECODE_ROUND = 3e-6              # a further round of blocks
+DECODE_MERGE = (2e-6, 0.1e-6)    # the merge kernel, and each split it reads
+DECODE_MOST_SPLITS = 64          # candidates looked at (beside the finest split)
+
+
+@functools.lru_cache(maxsize=4096)
+def decode_split(num_decode: int, num_kv_heads: int, max_len: int, head_dim: int = 128) -> tuple[int, int]:
     """(keys per split, number of splits) for the decode tokens of a step.  A block of
     DECODE_WAVES waves walks one split of one request and kv head, every wave a share of
-    it; the splits of a token are merged by a second kernel.  As few splits as put
-    TARGET_DECODE_WAVES waves on the GPU: more only add to the merge, and with one split
-    there is no merge.  A split is a whole number of 16 keys for every wave."""
+    it (a split is a whole number of 16 keys for every wave); the splits of a token are
+    merged by a second kernel.
+
+    The blocks run in rounds of one a CU, so what a split costs follows from how its blocks
+    fill the rounds: full rounds stream at the GPU's rate; the last, partial round at that
+    rate or, if its blocks are few, at the rate of a block alone (17 requests of 2,048 keys in
+    two splits are 272 blocks, 256 and then 16 that take as long again: 45 us against 34 in
+    three splits; 33 requests unsplit are 264 blocks: 71 us against 60 in three splits).  The
+    cheapest of the candidates by that price is taken; equal prices go to fewer splits.  The
+    kernel cuts every token's own keys evenly in that many splits (csrc/attention_mfma.hip:
+    decode_share), so a step's shorter requests, and lengths below the step's rounded longest
+    one, still give every block of a token the same share."""
     pairs = max(1, num_decode * num_kv_heads)
     least = 16 * DECODE_WAVES
     most = max(1, -(-max_len // least))
-    nsplit = min(most, max(1, -(-TARGET_DECODE_WAVES // (DECODE_WAVES * pairs))))
-    split = -(-(-(-max_len // nsplit)) // least) * least
-    nsplit = max(1, -(-max_len // split))
-    # A wave walks its tiles of 16 keys one after the other, about 2 us each from HBM, and the
-    # merge is a kernel of its own (4-5 us): splitting pays when it saves a wave two tiles or
-    # more (measured on a 0.6B-shaped model: 16 requests of some 600 keys, where two splits
-    # save one tile, +3 % a step without them; one request of 600 keys, where three splits
-    # save two, 3 % slower without them).
-    if nsplit > 1:
-        whole = -(-(-(-max_len // 16)) // DECODE_WAVES)
-        if whole - split // least < MERGE_WORTH_TILES:
-            return -(-max_len // least) * least, 1
-    return split, nsplit
+    key_bytes = 4 * head_dim          # a key and a value of one kv head, bfloat16
+    best = None
+    for want in list(range(1, min(most, DECODE_MOST_SPLITS) + 1)) + [most]:
+        split = -(-(-(-max_len // want)) // least) * least
+        nsplit = max(1, -(-max_len // split))
+        share = max_len / nsplit * key_bytes                       # bytes a block walks, on average
+        full, rest = divmod(pairs * nsplit, DECODE_CUS)
+        price = full * DECODE_CUS * share / DECODE_RATE
+        if rest:
+            price += math.hypot(rest * share / DECODE_RATE, share / DECODE_BLOCK_RATE)
+        price += DECODE_START + DECODE_ROUND * max(0, full + (rest > 0) - 1)
+        if nsplit > 1:
+            price += DECODE_MERGE[0] + DECODE_MERGE[1] * nsplit
+        if best is None or price < best[0] * (1 - 1e-9):
+            best = (price, split, nsplit)
+    return best[1], best[2]
 
 
 def tile_split(num_tiles: int, blocks_per_tile: int, max_len: int) -> tuple[int, int]:
@@ -200,7 +228,7 @@ def decode_attention_fused(qkv, q_weight, k_weight, cos, sin, k_cache, v_cache, 
     """q/k norm, rotation, cache write and attention of a decode-only step in one kernel
     (plus the merge of the splits, if a token's keys are split)."""
     work = work_of(batch)
-    split, nsplit = decode_split(work.num_single, num_kv_heads, work.max_single_len)
+    split, nsplit = decode_split(work.num_single, num_kv_heads, work.max_single_len, head_dim)
     if ops._profile is not None:
         keys = sum(c + 1 for c in batch.ctx_lens)
         ops._note(f"decode {work.num_single} tokens, fused", keys * 2 * num_kv_heads * head_dim * 2,
@@ -259,7 +287,7 @@ def _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, *
     if note is not None:
         decode_keys, tile_keys, tile_pairs, kv_token_bytes, flops_per_pair = note
     if work.num_single:
-        split, nsplit = decode_split(work.num_single, num_kv_heads, work.max_single_len)
+        split, nsplit = decode_split(work.num_single, num_kv_heads, work.max_single_len, head_dim)
         if note is not None:
             ops._note(f"decode {work.num_single} tokens", decode_keys * kv_token_bytes, decode_keys * flops_per_pair)
         if not ops.attention_mfma("heads", q, k_cache, v_cache, block_tables, batch.positions,
