@@ -128,17 +128,22 @@ def test_short_portions_over_long_contexts_split_their_keys(nh, nkv, hd, ps):
         torch.testing.assert_close(g, w, **TOL[torch.bfloat16])
 
 
-def test_many_tiles_over_long_contexts_use_the_four_wave_kernel():
-    """Two portions that both start beyond 2,048 cached tokens and fill the GPU without
-    splitting: the dispatcher takes the kernel variant built for four waves a SIMD
-    (checked by its conditions), with the same results."""
+def test_many_tiles_over_long_contexts_use_the_four_wave_kernel(monkeypatch):
+    """Two portions that both start beyond 2,048 cached tokens, with too many tiles for their
+    keys to be split and (pairs of heads, more blocks than CUs, under 4,096 keys) neither the
+    group nor the wide form: the dispatcher takes the kernel variant built for four waves a
+    SIMD (checked), with the same results."""
     from tokamak_amd.kernels import attention
 
-    nh, nkv, hd, ps = 32, 8, 128, 16
-    requests = [(2100, 300), (2500, 250)]
+    nh, nkv, hd, ps = 16, 8, 128, 16
+    requests = [(2100, 700), (2500, 650)]
     tiles = sum(-(-q // 16) for _, q in requests)
-    assert attention.tile_split(tiles, nkv, 2800)[1] == 1 and min(c for c, _ in requests) >= attention.DENSE_TILES_FROM
+    assert attention.tile_split(tiles, nkv, 3150)[1] == 1 and min(c for c, _ in requests) >= attention.DENSE_TILES_FROM
+    launched = []
+    real = attention.ops.attention_mfma
+    monkeypatch.setattr(attention.ops, "attention_mfma", lambda mode, *a, **k: (launched.append(mode), real(mode, *a, **k))[1])
     got, want = run_attention(torch.bfloat16, nh, nkv, hd, ps, requests, seed=13)
+    assert launched == ["tokens_dense"]
     for g, w in zip(got, want):
         assert torch.isfinite(g).all()
         torch.testing.assert_close(g, w, **TOL[torch.bfloat16])

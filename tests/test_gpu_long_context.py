@@ -113,14 +113,17 @@ def test_a_short_portion_over_the_longest_context(dtype, keys, monkeypatch):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 @pytest.mark.parametrize("keys", [32768, 40960])
 def test_a_long_portion_over_the_longest_context(dtype, keys, monkeypatch):
-    """2,048 tokens at the end of ``keys``: the group form (tiles of 32 tokens, a block a CU) at
-    its real threshold."""
+    """2,048 tokens at the end of ``keys``: with four kv heads the group form (tiles of 32 tokens,
+    a block a CU) at its real threshold; with two, too few blocks for it: the 16-token tiles with
+    their keys cut into pieces."""
     ctx = keys - 2048
     targets = [(0, 0), (31, 63), (32, 64), (1000, ctx - 1), (1500, ctx + 1499), (2047, ctx // 3), (777, 4095), (778, 4096)]
-    launched = run(dtype, 8, 2, ctx, 2048, seed=keys + 2, targets=targets,
+    launched = run(dtype, 16, 4, ctx, 2048, seed=keys + 2, targets=targets,
                    monkeypatch=monkeypatch if dtype == torch.bfloat16 else None)
     if dtype == torch.bfloat16:
         assert launched == [("tokens_group", 1)]
+        launched = run(dtype, 8, 2, ctx, 2048, seed=keys + 6, targets=targets, monkeypatch=monkeypatch)
+        assert len(launched) == 1 and launched[0][0] == "tokens" and launched[0][1] > 1
 
 
 @pytest.mark.parametrize("keys", [32768, 40960])

@@ -93,3 +93,20 @@ def test_decode_splits_follow_how_the_blocks_fill_the_rounds():
     assert decode_split(8, 8, 2560)[1] == 4 and decode_split(1, 8, 2560)[1] >= 8
     assert decode_split(8, 8, 300)[1] <= 2
     assert decode_split(1, 2, 32768)[1] >= 32
+
+
+def test_the_keys_of_few_tiles_are_split_over_blocks():
+    from tokamak_amd.kernels.attention import tile_split
+
+    none = (1 << 30, 1)
+    # (tiles of 16 tokens, blocks of the narrow form a tile, longest context)
+    assert tile_split(4, 2, 40960) == (512, 80)             # four tiles: pieces of 512 keys
+    assert tile_split(16, 16, 16640)[1] == 8                # 256 tokens, 64 query heads: eight pieces
+    assert tile_split(8, 40, 16512)[1] == 7                 # 128 tokens, five heads a kv head
+    assert tile_split(16, 16, 1280) == none                 # pieces would be shorter than 1,024 keys
+    assert tile_split(8, 8, 1100)[1] == 2                   # few blocks: pieces of 512 and more
+    assert tile_split(64, 16, 16384) == none                # 1,024 blocks fill the GPU unsplit
+    for tiles, per_tile, longest in ((4, 2, 40960), (16, 16, 16640), (35, 8, 5037), (3, 1, 1024)):
+        split, nsplit = tile_split(tiles, per_tile, longest)
+        if nsplit > 1:
+            assert split % 64 == 0 and (nsplit - 1) * split < longest <= nsplit * split

@@ -16,9 +16,11 @@ WIDE_TOKENS = 32   # and per tile of the wide matrix-core kernel
 
 MFMA_HEAD_DIMS = (64, 128)
 DECODE_WAVES = 16           # waves of a decode block (csrc/attention_mfma.hip: kDecodeWaves)
-TILE_SPLIT_BELOW_BLOCKS = 256   # a portion with fewer blocks than this has its keys split ...
-TILE_SPLIT_MIN_KEYS = 512       # ... into pieces no shorter than this
-TARGET_TILE_BLOCKS = 1024
+TILE_SPLIT_UP_TO_BLOCKS = 640   # a portion with no more blocks of the narrow form than this has its keys split ...
+TILE_SPLIT_MIN_KEYS = 512       # ... into pieces no shorter than this (twice this from TILE_SPLIT_FEW_BLOCKS blocks on) ...
+TILE_SPLIT_FEW_BLOCKS = 128
+TARGET_TILE_BLOCKS = 2048       # ... so that about this many blocks run
+GROUP_OVER_SPLIT_FILL = 512     # blocks times shares from which the group form is taken rather than split tiles
 DENSE_TILES_FROM = 2048         # every tiled span starts at least this deep: the four-wave kernel
 WIDE_FROM_KEYS = 4096           # longest context from which the 32-token tiles of the wide kernel pay (+15-20 %;
                                 # for shorter walks the narrow one's smaller tiles balance better)
@@ -179,18 +181,30 @@ def decode_split(num_decode: int, num_kv_heads: int, max_len: int, head_dim: int
 
 def tile_split(num_tiles: int, blocks_per_tile: int, max_len: int) -> tuple[int, int]:
     """(keys per split, number of splits) for the 16-token tiles of prompt portions.
-    A block walks its tile's keys 64 at a time, one after the other; a short portion
-    over a long context (the last piece of a long prompt, a small token budget) has
-    few tiles and would leave the GPU idle for hundreds of such steps, so its keys
-    are cut into pieces that run side by side and are merged afterwards."""
+    A block walks its tile's keys 64 at a time, one after the other; a portion of a few
+    hundred tokens over a long context (the last piece of a long prompt, a small token
+    budget) has few tiles, and a CU holds three such blocks, so up to some hundreds of
+    blocks the GPU is mostly idle for a long walk: the keys are cut into pieces that run
+    side by side, about TARGET_TILE_BLOCKS blocks in all, and merged afterwards (256 tokens
+    of a layer with 64 query heads over 16,384 keys: 447 us unsplit, 228 in eight pieces;
+    128 tokens with five heads a kv head over 16,384: 432 -> 220)."""
     blocks = num_tiles * blocks_per_tile
-    if blocks >= TILE_SPLIT_BELOW_BLOCKS or max_len < 2 * TILE_SPLIT_MIN_KEYS or num_tiles * 16 > 65535:
+    least = TILE_SPLIT_MIN_KEYS if blocks <= TILE_SPLIT_FEW_BLOCKS else 2 * TILE_SPLIT_MIN_KEYS
+    if blocks > TILE_SPLIT_UP_TO_BLOCKS or max_len < 2 * least or num_tiles * 16 > 65535:
         return 1 << 30, 1
-    nsplit = min(max_len // TILE_SPLIT_MIN_KEYS, -(-TARGET_TILE_BLOCKS // blocks))
+    nsplit = min(max_len // least, -(-TARGET_TILE_BLOCKS // blocks))
     if nsplit < 2:
         return 1 << 30, 1
     split = -(-(-(-max_len // nsplit)) // 64) * 64
     return split, -(-max_len // split)
+
+
+def group_fill(group: int, num_kv_heads: int, num_wide: int) -> int:
+    """Blocks of the group form times the shares of the keys a block holds."""
+    nblk = -(-group // 8)
+    heads = -(-group // nblk)                   # heads a block
+    shares = 4 if heads <= 2 else 2 if heads <= 4 else 1
+    return num_wide * num_kv_heads * nblk * shares
 
 
 def group_form_pays(group: int, num_kv_heads: int, num_wide: int, max_len: int) -> bool:
@@ -206,7 +220,7 @@ def group_form_pays(group: int, num_kv_heads: int, num_wide: int, max_len: int) 
     heads = -(-group // nblk)                   # heads a block
     shares = 4 if heads <= 2 else 2 if heads <= 4 else 1
     blocks = num_wide * num_kv_heads * nblk
-    if blocks * shares < GROUP_FILL:
+    if group_fill(group, num_kv_heads, num_wide) < GROUP_FILL:
         return False
     if group <= 2:
         return blocks <= 256 and max_len >= 2 * GROUP_FROM_KEYS
@@ -298,16 +312,19 @@ def _paged_attention_mfma(q, k_cache, v_cache, block_tables, batch, work, out, *
         group = num_heads // num_kv_heads
         per_tile = num_kv_heads * (group // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
         split, nsplit = tile_split(work.num_tiles, per_tile, work.max_tile_len)
-        if (nsplit == 1 and work.num_tile_tokens >= WIDE_FROM_TOKENS * work.num_wide
-                and group_form_pays(group, num_kv_heads, work.num_wide, work.max_tile_len)):
+        full = work.num_tile_tokens >= WIDE_FROM_TOKENS * work.num_wide
+        grouped = full and group_form_pays(group, num_kv_heads, work.num_wide, work.max_tile_len)
+        if (nsplit > 1 and grouped and work.num_tiles * per_tile > 2 * TILE_SPLIT_FEW_BLOCKS
+                and group_fill(group, num_kv_heads, work.num_wide) >= GROUP_OVER_SPLIT_FILL):
+            split, nsplit = 1 << 30, 1      # enough blocks for the group form: ahead of split tiles there
+        if nsplit == 1 and grouped:
             # tiles of 32 tokens mostly full: the group form, whose blocks hold a CU each
             if note is not None:
                 ops._note(f"portions {work.num_wide} wide tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
             return ops.attention_mfma("tokens_group", q, k_cache, v_cache, block_tables, batch.positions,
                                       batch.req_of_token, work.wide_first, work.wide_count, work.num_wide,
                                       out, **common)
-        if (nsplit == 1 and work.max_tile_len >= WIDE_FROM_KEYS
-                and work.num_tile_tokens >= WIDE_FROM_TOKENS * work.num_wide):
+        if nsplit == 1 and work.max_tile_len >= WIDE_FROM_KEYS and full:
             # long walks over the keys, tiles of 32 tokens mostly full: the wide kernel
             if note is not None:
                 ops._note(f"portions {work.num_wide} wide tiles", tile_keys * kv_token_bytes, tile_pairs * flops_per_pair)
