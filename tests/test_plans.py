@@ -4,7 +4,7 @@ the weight-streaming product keeps its own rules at every size."""
 import pytest
 
 from tokamak_amd.kernels import ops
-from tokamak_amd.kernels.gemm_bf16 import STREAM_TARGET_BLOCKS, stream_splits
+from tokamak_amd.kernels.gemm_bf16 import STREAM_TARGET_BLOCKS, _fill, stream_splits
 
 SHAPES = [(4096, 1024), (1024, 2048), (1024, 3072), (6144, 2560), (2560, 9728), (6144, 4096), (4096, 4096),
           (4096, 12288), (10240, 5120), (5120, 8192), (5120, 25600), (151936, 4096), (151936, 1024), (48, 264), (130, 8)]
@@ -19,19 +19,43 @@ def test_splits_stay_within_the_chunks_and_fill_the_gpu_evenly(n, k, m):
     splits = stream_splits(n, k, m)
     assert 1 <= splits <= max(1, chunks)
     blocks = -(-n // (16 * waves))
-    if m > 16 and 2 * n * k >= ops.STREAM_SMALL_MATRIX_BYTES:
-        # what runs at once: two blocks of four waves a CU (an eighth over is taken), one of eight
-        limit = STREAM_TARGET_BLOCKS * 9 // 8 if waves == 4 else STREAM_TARGET_BLOCKS // 2
-        assert splits == 1 or splits * blocks <= limit
+    large = 2 * n * k >= ops.STREAM_SMALL_MATRIX_BYTES
+    if m > 32 and large:
+        # one block of six or eight waves a CU
+        assert splits == 1 or splits * blocks <= STREAM_TARGET_BLOCKS // 2
         assert splits == 1 or chunks // splits >= 2
-        if m > 32 and n <= 256 * 128:
+        if n <= 256 * 128:
             # six waves only where one round of them covers a tenth more of the CUs than one of eight
             six, eight = ops.stream_fill(n, k, 6)[0], ops.stream_fill(n, k, 8)[0]
             assert waves == (6 if six >= 1.1 * eight else 8)
         else:
             assert waves == 4
-    else:
-        assert waves == 4
+        return
+    assert waves == 4
+    used = -(-chunks // -(-chunks // splits))       # the kernel's shares: none is empty
+    assert used == splits                           # the plan names the number that runs
+    if m > 16 and large and splits > 1:
+        assert -(-chunks // splits) >= 2
+    # no other number of shares fills the CUs more evenly
+    least = 1 if m <= 16 or not large else 2
+    if blocks < STREAM_TARGET_BLOCKS:
+        for share in range(least, chunks + 1):
+            other = -(-chunks // share)
+            assert other > 64 or _fill(blocks * other) <= _fill(blocks * splits)
+
+
+def test_splits_of_the_measured_shapes():
+    # (output columns, K, rows) -> shares of K that were the fastest, or within a few percent of it
+    cases = {
+        (6144, 4096, 8): 8, (4096, 4096, 8): 8, (4096, 12288, 8): 8, (6144, 4096, 24): 8, (4096, 12288, 32): 8,     # 8B
+        (7168, 5120, 8): 4, (5120, 5120, 8): 5, (5120, 17408, 8): 6, (5120, 17408, 32): 6,                          # 14B
+        (10240, 5120, 16): 3, (5120, 8192, 4): 6, (5120, 25600, 16): 6,                                             # 32B
+        (6144, 2560, 16): 5, (2560, 4096, 4): 16, (2560, 4096, 24): 16, (2560, 9728, 16): 19,                        # 4B
+        (2048, 6144, 4): 24, (2048, 6144, 32): 12,                                                                  # 1.7B
+        (151936, 4096, 8): 1,                                                                                       # a head
+    }
+    for (n, k, m), splits in cases.items():
+        assert stream_splits(n, k, m) == splits, (n, k, m)
 
 
 def test_the_gated_product_picks_its_block_size_by_rows_columns_and_row_length():

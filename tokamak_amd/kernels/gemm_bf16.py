@@ -38,30 +38,48 @@ def skinny_plan(m: int, n: int, k: int) -> tuple[int, int]:
     return row_tiles, waves
 
 
+def _fill(total: int) -> float:
+    """How well `total` blocks of four waves use the GPU: two a CU run at full rate, so up to 512
+    count by their number; beyond, the CUs that get one block more than the others set the time, so
+    a count just under the next multiple of 256 is good and one just over it is the worst (80 row
+    blocks of a 14B-shaped down projection: 480 blocks 29 us, 560 blocks 35 us, 720 blocks 32 us);
+    every further block a CU costs a little by itself (partial sums, shorter shares)."""
+    room = max(STREAM_TARGET_BLOCKS, -(-total // 256) * 256)
+    return total / room * 0.95 ** ((room - STREAM_TARGET_BLOCKS) // 256)
+
+
 def stream_splits(n: int, k: int, m: int = 1) -> int:
     """Shares of K for the LDS-staged kernel so that enough blocks exist, and no more.
 
-    Up to 16 rows, and for small matrices (the projections of a 0.6B-shaped model): about 512
-    blocks, down to one chunk of 256 a share: such a product is read in one memory round trip
-    then, and its time is round trips, not bytes.  With more rows every split also writes (and
-    the next kernel reads) float32 partial sums of all of them, a block holds more LDS and
-    fewer blocks fit a CU, so what counts is how evenly the blocks fill the 256 CUs: a few
-    blocks beyond what runs at once cost a whole further round (measured at 32B-shaped sizes
-    with 64 rows: 280 blocks of eight waves take 80 us where 240 take 57).  17 to 32 rows: two
-    blocks of four waves a CU, overshooting by an eighth at most; beyond: one block of eight
-    waves a CU; never fewer than two chunks a share.  Against the best of every split and block
-    size measured on the projection shapes of 0.6B to 32B models this is within 2 % on average
-    and 15 % at worst."""
+    Up to 32 rows (blocks of four waves): of the numbers of shares that K's chunks of 256 allow, the
+    one whose blocks fill the CUs most evenly (``_fill``): 512 blocks or a little less, else a
+    little less than 768.  17 to 32 rows of a large matrix: never fewer than two chunks a share,
+    since every split also writes (and the next kernel reads) float32 partial sums of all rows.
+    Small matrices (the projections of a 0.6B-shaped model) at any number of rows likewise, down
+    to one chunk a share: such a product is read in one memory round trip then, and its time is
+    round trips, not bytes.  More rows: a block holds more LDS and one block of six or eight waves
+    runs on a CU, so a few blocks beyond the 256 CUs cost a whole further round (measured at
+    32B-shaped sizes with 64 rows: 280 blocks of eight waves take 80 us where 240 take 57): at most
+    256 blocks, never fewer than two chunks a share.  Against the best of every split measured on
+    the projection shapes of 1.7B to 32B models at 4 to 32 rows this is within 1 % on average and
+    10 % at worst (a small matrix with 32 rows)."""
     chunks = -(-k // 256)
     blocks = -(-n // (16 * ops.stream_waves(m, k, False, n)))
-    if m <= 16 or 2 * n * k < ops.STREAM_SMALL_MATRIX_BYTES:
-        return max(1, min(chunks, -(-STREAM_TARGET_BLOCKS // blocks), 64))
-    if m <= 32:
-        splits = max(1, STREAM_TARGET_BLOCKS // blocks)
-        if (splits + 1) * blocks <= STREAM_TARGET_BLOCKS * 9 // 8:
-            splits += 1
-    else:
-        splits = max(1, STREAM_TARGET_BLOCKS // 2 // blocks)
+    small = 2 * n * k < ops.STREAM_SMALL_MATRIX_BYTES
+    if m <= 32 or small:
+        if blocks >= STREAM_TARGET_BLOCKS:
+            return 1
+        least_share = 1 if m <= 16 or small else min(2, chunks)
+        best, best_fill = 1, _fill(blocks)
+        for share in range(chunks, least_share - 1, -1):        # chunks a share, fewest splits first
+            splits = -(-chunks // share)
+            if splits > 64:
+                break
+            fill = _fill(blocks * splits)
+            if fill > best_fill:
+                best, best_fill = splits, fill
+        return best
+    splits = max(1, STREAM_TARGET_BLOCKS // 2 // blocks)
     return max(1, min(splits, chunks // 2))
 
 
