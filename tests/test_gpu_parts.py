@@ -174,6 +174,47 @@ def test_sampling_distribution_matches_plain(V):
     assert tokens[5].item() == logits[5].argmax().item()       # top_k = 1 is greedy at any temperature
 
 
+def _uniform(seed: int, draw: int) -> float:
+    """The sampler's uniform number of (request seed, draws so far): a splitmix64-style mix, its top 24 bits."""
+    mask = (1 << 64) - 1
+    z = (seed * 0x9E3779B97F4A7C15 + (draw + 1) * 0xBF58476D1CE4E5B9) & mask
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
+    z ^= z >> 31
+    return (z >> 40) / 16777216.0
+
+
+@pytest.mark.parametrize("V", [331, 1001, 151936])
+def test_the_drawn_token_is_where_the_uniform_number_falls_in_index_order(V):
+    """The draw is the inverse of the cumulative distribution over the kept tokens in index
+    order: with the request's uniform number u, the first token whose cumulative probability
+    exceeds u.  Checked against a float64 walk on the host, to the rounding of the float32 sums;
+    many seeds, so that targets fall in every part of the row (the first tokens, the last, the
+    edges of the chunks the kernel cuts the row into)."""
+    from tokamak_amd import SamplingParams
+    from tokamak_amd.sampling.sampler import sample_tokens
+
+    rows = 48
+    logits = torch.randn(rows, V, generator=torch.Generator().manual_seed(V + 1)) * 2
+    logits[1] = 0.0                                     # a uniform row: the target's place is the token's index
+    logits[2, : V // 2] = float("-inf")                 # nothing in the first half
+    logits[3, V // 3:] = float("-inf")                  # nothing after the first third
+    params = [SamplingParams(temperature=1.0) if i % 3 else SamplingParams(temperature=0.7, top_k=V // 2 + 1, top_p=0.95)
+              for i in range(rows)]
+    seeds = [1000 + 7 * i for i in range(rows)]
+    for draw in (0, 1, 2):
+        tokens, probs = sample_tokens(logits.to(DEV), params, seeds, [draw] * rows, return_probs=True)
+        tokens, probs = tokens.cpu().tolist(), probs.cpu().double()
+        for i in range(rows):
+            cum = probs[i].cumsum(0)
+            u = _uniform(seeds[i], draw) * cum[-1].item()
+            t = tokens[i]
+            assert probs[i, t] > 0
+            assert cum[t] > u - 2e-5 and cum[t] - probs[i, t] <= u + 2e-5, (i, draw, t, u, cum[t].item())
+    # the uniform row: token = floor(u V) to the same rounding
+    assert abs(tokens[1] - int(_uniform(seeds[1], 2) * V)) <= max(1, V // 20000)
+
+
 def test_sampling_vectors_and_seeds():
     """Vectors of reference tests/unit/test_sampler.py:26-56."""
     from tokamak_amd import SamplingParams
