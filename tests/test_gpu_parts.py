@@ -174,6 +174,31 @@ def test_sampling_distribution_matches_plain(V):
     assert tokens[5].item() == logits[5].argmax().item()       # top_k = 1 is greedy at any temperature
 
 
+@pytest.mark.parametrize("V", [20000, 151936])
+def test_sampling_thresholds_when_the_logits_are_nearly_all_alike(V):
+    """The threshold searches copy the values that may hold a threshold into LDS when they are
+    few.  Here they are not: every logit lies in [1, 1.06), one bin of the first level, so the
+    searches walk the row at every level; and a row with a few hundred values far above the
+    rest, where the copies are used.  Both against the plain distribution."""
+    from tokamak_amd import SamplingParams
+    from tokamak_amd.sampling.sampler import sample_tokens
+
+    gen = torch.Generator().manual_seed(V)
+    alike = 1.0 + 0.06 * torch.rand(3, V, generator=gen)
+    peaked = torch.randn(3, V, generator=gen)
+    peaked[:, torch.randperm(V, generator=gen)[:300]] += 12.0
+    logits = torch.cat([alike, peaked])
+    params = [SamplingParams(temperature=1.0, top_k=50), SamplingParams(temperature=0.9, top_p=0.5),
+              SamplingParams(temperature=1.1, top_k=9000, top_p=0.97)] * 2
+    tokens, probs = sample_tokens(logits.to(DEV), params, list(range(6)), [0] * 6, return_probs=True)
+    tokens, probs = tokens.cpu(), probs.cpu()
+    for i, p in enumerate(params):
+        want = plain.sampling_probs(logits[i], p.temperature, p.top_k, p.top_p).float()
+        torch.testing.assert_close(probs[i], want, rtol=2e-3, atol=1e-9)
+        assert (probs[i] > 0).sum() == (want > 0).sum()
+        assert probs[i][tokens[i]] > 0
+
+
 def _uniform(seed: int, draw: int) -> float:
     """The sampler's uniform number of (request seed, draws so far): a splitmix64-style mix, its top 24 bits."""
     mask = (1 << 64) - 1

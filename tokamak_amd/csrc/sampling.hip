@@ -285,22 +285,31 @@ __device__ __forceinline__ void for_row(const float* __restrict__ row, int V, F 
 // probs_out (optional, [M, V]) receives the final distribution, for tests.
 //
 // Both thresholds are found by radix selection over the ordered-integer image of the
-// scaled logits: three passes over the row (12, 12 and 8 bits), each filling a
-// histogram in LDS (counts for top-k, fixed-point probability mass for top-p) in
-// which the bin that holds the threshold is found; the next pass looks only at the
-// values of that bin.  The row (600 KB for a vocabulary of 152 k) stays in L2.
+// scaled logits: three levels (12, 12 and 8 bits), each filling a histogram in LDS (counts
+// for top-k, fixed-point probability mass for top-p) in which the bin that holds the
+// threshold is found; the next level looks only at the values of that bin.  A pass over the
+// row costs 14 us (one CU reads it alone), so the row is walked as rarely as possible: the
+// first pass fills the first level's histogram and tells in which of its bins the threshold
+// lies; if the values of that bin and the bins above it are few (up to kCandidates; they
+// are, unless the logits are nearly all alike), a second pass copies them into LDS, and every
+// further level of both searches reads those.  The third pass is the draw's.  (Without the
+// copies: seven passes with both thresholds.)
+constexpr int kCandidates = 16384;
+
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p,
     const unsigned long long* __restrict__ seeds, const unsigned long long* __restrict__ counters,
     const float* __restrict__ row_max, int* __restrict__ out, float* __restrict__ probs_out) {
   __shared__ float fs[16];
-  __shared__ unsigned long long hist64[kBins];       // counts use the same memory as 32-bit bins
+  __shared__ unsigned long long hist64[kBins];
+  __shared__ uint32_t hist32[kBins];
   __shared__ unsigned long long scan64[kSampleThreads];
+  __shared__ uint32_t cand[kCandidates];  // ordered images of the values that may hold a threshold
+  __shared__ uint32_t cand_count;
   __shared__ int found_bin;
   __shared__ int last_token;
   __shared__ unsigned long long found_above;
-  uint32_t* hist32 = reinterpret_cast<uint32_t*>(hist64);
   uint32_t* scan32 = reinterpret_cast<uint32_t*>(scan64);
   float* scanf_ = reinterpret_cast<float*>(scan64);
 
@@ -310,26 +319,88 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   const float inv_t = 1.f / temperature[r];
   const int k = top_k[r];
   const float p_keep = top_p[r];
+  const bool k_on = k > 0 && k < V, p_on = p_keep < 1.f;
 
   // the row's maximum comes from the argmax pass that ran before (temperature > 0
   // keeps the order); a row without any number has nothing to draw from
   const float mx = row_max[r] * inv_t;
   if (!(mx > -INFINITY)) return;
 
+  // First pass: the first level's histogram (counts; probability mass too if only top-p is
+  // asked for), the bin of the first threshold to be found, and the candidates.
+  uint32_t k_prefix = 0, k_remaining = (uint32_t)max(k, 0);
+  uint32_t p_prefix = 0;               // only top-p: its first level is found by the first pass
+  unsigned long long p_remaining = 0;
+  int ncand = -1;                      // >= 0: cand[0 .. ncand) hold every value that can be a threshold
+  if (k_on || p_on) {
+    for (int i = tid; i < kBins; i += nt) {
+      hist32[i] = 0;
+      hist64[i] = 0;
+    }
+    if (tid == 0) cand_count = 0;
+    __syncthreads();
+    for_row(row, V, [&](int, float logit) {
+      const float x = scaled(logit, inv_t);
+      const uint32_t bin = ordered(x) >> 20;
+      atomicAdd(&hist32[bin], 1u);
+      if (!k_on) atomicAdd(&hist64[bin], fixed_mass(x, mx));
+    });
+    __syncthreads();
+    int low_bin;
+    if (k_on) {
+      uint32_t above;
+      crossing_bin<uint32_t>(hist32, kBins, k_remaining, scan32, &found_bin,
+                             reinterpret_cast<uint32_t*>(&found_above), low_bin, above);
+      k_remaining -= above;
+      k_prefix = (uint32_t)low_bin;
+    } else {
+      // the whole mass, then the share of it that top_p allows (at least one unit)
+      unsigned long long mine = 0, upto, whole, above;
+      for (int i = tid; i < kBins; i += nt) mine += hist64[i];
+      block_scan<unsigned long long>(mine, scan64, upto, whole);
+      const double share = (double)p_keep * (double)whole;
+      p_remaining = share < 1.0 ? 1ull : (unsigned long long)share;
+      crossing_bin<unsigned long long>(hist64, kBins, p_remaining, scan64, &found_bin, &found_above, low_bin, above);
+      p_remaining -= above;
+      p_prefix = (uint32_t)low_bin;
+    }
+    // the values in that bin and above it
+    uint32_t mine = 0, upto, total;
+    for (int i = tid; i < kBins; i += nt) mine += i >= low_bin ? hist32[i] : 0u;
+    block_scan<uint32_t>(mine, scan32, upto, total);
+    if (total <= (uint32_t)kCandidates) {
+      for_row(row, V, [&](int, float logit) {
+        const uint32_t o = ordered(scaled(logit, inv_t));
+        if ((int)(o >> 20) >= low_bin) cand[atomicAdd(&cand_count, 1u)] = o;  // (in any order: the sums below are of integers)
+      });
+      ncand = (int)total;
+    }
+    __syncthreads();
+  }
+  // f(ordered image, scaled logit) for every value that may still hold a threshold
+  const auto each = [&](auto f) {
+    if (ncand >= 0) {
+      for (int i = tid; i < ncand; i += nt) f(cand[i], unordered(cand[i]));
+    } else {
+      for_row(row, V, [&](int, float logit) {
+        const float x = scaled(logit, inv_t);
+        f(ordered(x), x);
+      });
+    }
+  };
+
   // top-k: kth = the k-th largest scaled logit (everything >= it survives)
   uint32_t kth = 0;  // ordered(-inf) is > 0, so 0 keeps everything
-  if (k > 0 && k < V) {
-    uint32_t prefix = 0, remaining = (uint32_t)k;
-    // (shift, bits): 20/12, 8/12, 0/8
-    for (int level = 0; level < 3; ++level) {
-      const int shift = level == 0 ? 20 : level == 1 ? 8 : 0;
+  if (k_on) {
+    uint32_t prefix = k_prefix, remaining = k_remaining;
+    // (shift, bits): 20/12 (done above), 8/12, 0/8
+    for (int level = 1; level < 3; ++level) {
+      const int shift = level == 1 ? 8 : 0;
       const int nbins = level == 2 ? 256 : kBins;
       for (int i = tid; i < kBins; i += nt) hist32[i] = 0;
       __syncthreads();
-      for_row(row, V, [&](int, float logit) {
-        const uint32_t o = ordered(scaled(logit, inv_t));
-        const bool in_bin = level == 0 || (o >> (shift + (level == 1 ? 12 : 8))) == prefix;
-        if (in_bin) atomicAdd(&hist32[(o >> shift) & (uint32_t)(nbins - 1)], 1u);
+      each([&](uint32_t o, float) {
+        if ((o >> (shift + (level == 1 ? 12 : 8))) == prefix) atomicAdd(&hist32[(o >> shift) & (uint32_t)(nbins - 1)], 1u);
       });
       __syncthreads();
       int bin;
@@ -345,23 +416,21 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   // top-p: keep x iff the mass of kept values strictly greater than x is < top_p of
   // the whole; the kept set is {x >= cut}
   uint32_t cut = kth;
-  if (p_keep < 1.f) {
-    uint32_t prefix = 0;
-    unsigned long long remaining = 0;
-    for (int level = 0; level < 3; ++level) {
+  if (p_on) {
+    uint32_t prefix = p_prefix;
+    unsigned long long remaining = p_remaining;
+    for (int level = k_on ? 0 : 1; level < 3; ++level) {  // (without top-k the first pass was the first level)
       const int shift = level == 0 ? 20 : level == 1 ? 8 : 0;
       const int nbins = level == 2 ? 256 : kBins;
       for (int i = tid; i < kBins; i += nt) hist64[i] = 0;
       __syncthreads();
-      for_row(row, V, [&](int, float logit) {
-        const float x = scaled(logit, inv_t);
-        const uint32_t o = ordered(x);
+      each([&](uint32_t o, float x) {
         const bool in_bin = level == 0 || (o >> (shift + (level == 1 ? 12 : 8))) == prefix;
         if (in_bin && o >= kth) atomicAdd(&hist64[(o >> shift) & (uint32_t)(nbins - 1)], fixed_mass(x, mx));
       });
       __syncthreads();
       if (level == 0) {
-        // the whole mass, then the share of it that top_p allows (at least one unit)
+        // the whole mass of what top-k keeps (the candidates hold all of it)
         unsigned long long mine = 0, upto, whole;
         for (int i = tid; i < kBins; i += nt) mine += hist64[i];
         block_scan<unsigned long long>(mine, scan64, upto, whole);
