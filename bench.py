@@ -103,13 +103,13 @@ def measure_peaks() -> dict:
 # ---------------------------------------------------------------------------
 # the model and what a step has to move and compute, from the plan
 # ---------------------------------------------------------------------------
-def make_llm(cfg, dtype, pool_tokens, max_requests, max_seq_len, seed=0):
+def make_llm(cfg, dtype, pool_tokens, max_requests, max_seq_len, seed=0, tune=True):
     """The engine's entry point over seeded random weights of ``cfg``'s shape, drawn on the GPU."""
     from tokamak_amd import LLM
 
     return LLM(cfg, seed=seed, random_weights_on_gpu=True, dtype=dtype, block_size=PAGE_SIZE,
                kv_pool_tokens=pool_tokens, max_batch_size=max_requests, max_seq_len=max_seq_len,
-               max_num_batched_tokens=PREFILL_TOKENS)
+               max_num_batched_tokens=PREFILL_TOKENS, tune_library_products=tune)
 
 
 def make_runner(arch, cfg, dtype, pool_tokens, max_requests, seed=0):
@@ -634,11 +634,11 @@ def main() -> int:
     want_points = not args.no_points and args.phase == "all"
     max_batch = max(64 if want_points else 1, args.batch)
     peaks = None if args.no_peaks else measure_peaks()
-    ops.set_library_tuning(not args.no_tune)
     deepest = max(final_context, prompt_tokens + 129) if args.profile else final_context   # (the profiled step sits 129 tokens in)
     pool = max_batch * (-(-(deepest + 1) // PAGE_SIZE) * PAGE_SIZE + PAGE_SIZE)
     longest = max(deepest + 1, PREFILL_TOKENS + 1)
-    llm = make_llm(cfg, args.dtype, max(pool, PREFILL_TOKENS + PAGE_SIZE, longest), max_batch, longest)
+    llm = make_llm(cfg, args.dtype, max(pool, PREFILL_TOKENS + PAGE_SIZE, longest), max_batch, longest,
+                   tune=not args.no_tune)
     runner = llm.runner
     cost = StepCost(runner)
     vocab = runner.plan.vocab_size

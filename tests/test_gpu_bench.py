@@ -20,6 +20,10 @@ def test_timed_decoding_is_the_generation_loop(tmp_path, monkeypatch):
     batch, prompt_tokens, steps = 3, 40, 6
     built = bench.make_llm(cfg, "bfloat16", pool_tokens=256, max_requests=4, max_seq_len=64)
     assert built.runner.page_size == 8 and built.max_num_batched_tokens == 16 and built.max_seq_len == 64
+    from tokamak_amd.kernels import ops
+    assert ops._lt_tune == ops.LT_TUNE_CANDIDATES     # what the record calls tuned_products is on in this engine
+    bench.make_llm(cfg, "bfloat16", pool_tokens=256, max_requests=4, max_seq_len=64, tune=False)
+    assert ops._lt_tune == 1
     del built
     folder = make_folder(tmp_path, "B")       # weights the plain implementation can read
     llm = LLM(folder, dtype="float32", block_size=8, kv_pool_tokens=256, max_batch_size=4, max_seq_len=64,
