@@ -547,6 +547,50 @@ def test_streaming_product_with_every_block_size(M, N, K, waves):
     check_streaming_product(ops, M, N, K, waves)
 
 
+@pytest.mark.parametrize("M, N, K", [(65, 4096, 4096), (80, 331, 200), (96, 6144, 1024), (113, 1000, 2056), (128, 4096, 12288),
+                                     (128, 130, 264), (127, 64, 64)])
+def test_streaming_product_of_65_to_128_rows(M, N, K):
+    """Five to eight tiles of 16 rows in blocks of eight waves: one copy of the activations'
+    chunk in LDS, fragments read step by step."""
+    from tokamak_amd.kernels import ops
+    check_streaming_product(ops, M, N, K, 8)
+    check_streaming_product(ops, M, N, K, 0)        # eight waves are what is chosen for these rows
+    x = rand(M, K, seed=1).to(torch.bfloat16).to(DEV)
+    w = rand(N, K, seed=2, scale=K ** -0.5).to(torch.bfloat16).to(DEV)
+    with pytest.raises(ops.KernelError):            # blocks of four or six waves are not built for them
+        ops.gemm_stream(x, w, torch.empty((M, N), device=DEV), waves=4)
+    if N % 2 == 0:                                  # the gated product of the same operands
+        out = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.gemm_stream_swiglu(x, w, out)
+        g = x.cpu().double() @ w[:N // 2].cpu().double().T
+        u = x.cpu().double() @ w[N // 2:].cpu().double().T
+        torch.testing.assert_close(out.cpu().double(), g / (1 + torch.exp(-g)) * u, rtol=2e-2, atol=1e-2)
+
+
+def test_products_of_65_to_128_rows_whose_reader_adds_partial_sums_stream_the_weights():
+    """q/k/v, o and down of a step of 65 to 128 tokens: split over K by the streaming kernel where
+    that was measured to pay (up to 96 rows; to 128 for matrices of 64 MB and more); a caller
+    that wants the product itself gets the library's."""
+    from tokamak_amd.kernels import gemm_bf16, ops
+
+    x = rand(90, 1024, seed=1).to(torch.bfloat16).to(DEV)
+    w = rand(2048, 1024, seed=2, scale=1 / 32).to(torch.bfloat16).to(DEV)
+    want = x.cpu().double() @ w.cpu().double().T
+    with ops.KernelProfile() as seen:
+        parts = gemm_bf16.gemm(x, w, torch.bfloat16, allow_partials=True)
+        whole = gemm_bf16.gemm(x, w, torch.bfloat16)
+    assert parts.dim() == 3 and parts.shape[0] > 1 and parts.dtype == torch.float32
+    torch.testing.assert_close(parts.sum(0).cpu().double(), want, rtol=1e-3, atol=1e-3)
+    assert whole.shape == (90, 2048) and whole.dtype == torch.bfloat16
+    torch.testing.assert_close(whole.cpu().double(), want, rtol=2e-2, atol=1e-2)
+    assert [name.split()[0] for name, *_ in seen.calls] == ["gemm_stream", "lt_gemm"]
+    pays = gemm_bf16.stream_pays_beyond_64_rows
+    assert pays(65, 4096, 4096) and pays(96, 2048, 2048) and not pays(97, 4096, 4096) and not pays(64, 4096, 4096)
+    assert pays(128, 5120, 17408) and pays(112, 4096, 12288) and not pays(129, 5120, 25600) and not pays(80, 48, 4096)
+    more = rand(100, 1024, seed=3).to(torch.bfloat16).to(DEV)
+    assert gemm_bf16.gemm(more, w, torch.bfloat16, allow_partials=True).dim() == 2      # a small matrix: the library
+
+
 def check_streaming_product(ops, M, N, K, waves):
 
     x = rand(M, K, seed=1).to(torch.bfloat16)

@@ -261,7 +261,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
   // two copies written in turn one barrier a chunk is enough (a wave may start to write chunk
   // i + 1 while others still read chunk i): 3-6 % for blocks of eight waves, which have a CU to
   // themselves anyway; nothing at up to 16 rows, and blocks of four would lose a place on the CU.
-  constexpr int XBUF = (WAVES >= 6 && MT >= 2) ? 2 : 1;
+  constexpr int XBUF = (WAVES >= 6 && MT >= 2 && MT <= 4) ? 2 : 1;  // (five row tiles and more: one copy fits beside the weights)
   __shared__ __attribute__((aligned(16))) bf16_t ws[WAVES][16][SLD];
   __shared__ __attribute__((aligned(16))) bf16_t xs[XBUF][16 * MT][SLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -344,7 +344,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(
       TK_FETCH_W(next_)                                                                             \
       TK_FETCH_X(next_)                                                                             \
     }                                                                                               \
-    if constexpr (MT < READ_AHEAD_FROM) {                                                           \
+    if constexpr (MT < READ_AHEAD_FROM || MT > 4) { /* (more row tiles: no registers for two steps' fragments) */ \
       _Pragma("unroll") for (int s = 0; s < SBK / 32; ++s) {                                        \
         Frag8 wf, xf[MT];                                                                           \
         wf.u = *reinterpret_cast<const uint4*>(&ws[wave][r][s * 32 + kb * 8]);                      \
@@ -466,7 +466,14 @@ static int launch_stream_shape(const void* A, const void* W, void* C, int M, int
   if (mt == 1) TK_STREAM(1);
   else if (mt == 2) TK_STREAM(2);
   else if (mt == 3) TK_STREAM(3);
-  else TK_STREAM(4);
+  else if (mt == 4) TK_STREAM(4);
+  else if constexpr (WAVES == 8) {  // 65 to 128 rows: blocks of eight waves only
+    if (mt == 5) TK_STREAM(5);
+    else if (mt == 6) TK_STREAM(6);
+    else if (mt == 7) TK_STREAM(7);
+    else if (mt == 8) TK_STREAM(8);
+    else return -1;
+  } else return -1;
 #undef TK_STREAM
   return launch_status();
 }
@@ -489,7 +496,7 @@ static int launch_stream(int waves, const void* A, const void* W, void* C, int M
   return launch_stream_shape<TO, GATED, 4>(A, W, C, M, N, K, lda, ldw, ldc, cps, KS, split_stride, scale, stream);
 }
 
-// out_dtype: 0 float32, 1 bfloat16.  M <= 64; K a multiple of 8; rows 16-byte aligned.
+// out_dtype: 0 float32, 1 bfloat16.  M <= 64 (<= 128 with eight waves); K a multiple of 8; rows 16-byte aligned.
 // waves: 4 or 8 waves a block.  splits: shares of K.  With splits > 1 the output must be float32 and C holds
 // `splits` partial results, split_stride elements apart, that the reader adds.
 // sumsq (may be null), slabs, eps: the rows' scale, see RowScale; then M <= 16.
@@ -498,7 +505,7 @@ TK_API int tk_gemm_stream(int out_dtype, const void* A, const void* W, void* C, 
                           long lda, long ldw, long ldc, int splits, long split_stride, int waves,
                           const float* sumsq, int slabs, float eps, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535) return -1;
+  if (M > (waves >= 8 ? 128 : 64) || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0 || splits < 1 || splits > 65535) return -1;
   if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 6)) return -1;
   const RowScale scale{sumsq, slabs, eps};
   if (splits > 1 && out_dtype != 0) return -1;
@@ -516,7 +523,7 @@ TK_API int tk_gemm_stream_swiglu(const void* A, const void* W, void* C, int M, i
                                  long ldw, long ldc, int waves, const float* sumsq, int slabs, float eps,
                                  hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
+  if (M > (waves >= 8 ? 128 : 64) || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
   if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 6)) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
   return launch_stream<bf16_t, true>(waves, A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0,

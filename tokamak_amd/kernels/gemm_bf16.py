@@ -66,7 +66,7 @@ def stream_splits(n: int, k: int, m: int = 1) -> int:
     chunks = -(-k // 256)
     blocks = -(-n // (16 * ops.stream_waves(m, k, False, n)))
     small = 2 * n * k < ops.STREAM_SMALL_MATRIX_BYTES
-    if m <= 32 or small:
+    if m <= 32 or (small and m <= SKINNY_MAX_ROWS):
         if blocks >= STREAM_TARGET_BLOCKS:
             return 1
         least_share = 1 if m <= 16 or small else min(2, chunks)
@@ -83,6 +83,24 @@ def stream_splits(n: int, k: int, m: int = 1) -> int:
     return max(1, min(splits, chunks // 2))
 
 
+STREAM_PARTIALS_ROWS = 96           # rows up to which the split streaming product beats the library at every size
+STREAM_PARTIALS_BIG = 64 << 20      # ... and the bytes of a matrix from which it does up to 128 rows
+
+
+def stream_pays_beyond_64_rows(m: int, n: int, k: int) -> bool:
+    """Whether a product of 65 to 128 rows whose reader adds partial sums goes to the streaming
+    kernel (five to eight tiles of 16 rows, eight waves a block) rather than to the library.
+    Against the library's fastest candidate, q/k/v, o and down of 1.7B- to 32B-shaped layers are
+    10 to 40 % faster at 65 to 96 rows; at 128 rows the large matrices still are (down of a
+    32B-shaped layer 82 against 119 us) and the small ones are level or behind, and the partial
+    sums cost their reader a few microseconds more.  Whole decode steps: batch 80 at 1.7B / 8B /
+    14B / 32B widths +1 / +4 / +13 / +7 %, batch 128 -4 / -3 / +4 / +5 % if every product
+    took this path, hence the limit on small matrices."""
+    if not SKINNY_MAX_ROWS < m <= ops.STREAM_MAX_ROWS or n < STREAM_MIN_ROWS_OUT:
+        return False
+    return m <= STREAM_PARTIALS_ROWS or 2 * n * k >= STREAM_PARTIALS_BIG
+
+
 def gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype, allow_partials: bool = False) -> torch.Tensor:
     """x[M, K] @ weight[N, K]^T -> [M, N] in ``out_dtype``; or, if the caller can
     add them (``allow_partials``), float32 partial sums [P, M, N] of a split-K product.
@@ -90,20 +108,23 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype, allow_pa
     Up to 64 rows (decode batches, wanted logits rows): hand-written
     weight-streaming MFMA kernels: the LDS-staged one, split over K into partial
     sums when the matrix has few rows and the caller adds them; the
-    direct-operand one for very small matrices.  More than 64 rows
+    direct-operand one for very small matrices.  65 to 128 rows, if the caller adds partial
+    sums: the same kernel with five to eight tiles of 16 rows where it was measured to pay
+    (``stream_pays_beyond_64_rows``).  Else more than 64 rows
     with bfloat16 output: the library product (hipBLASLt, as the reference's
     nn.Linear ends in a library; csrc/blas_lt.hip); with float32 output: 64 rows at a time.
     """
     m = x.shape[0]
     n, k = weight.shape
     dev = x.device
-    if skinny_fits(x, weight) and (m <= SKINNY_MAX_ROWS or out_dtype == torch.float32):
-        if m <= SKINNY_MAX_ROWS and allow_partials:
-            splits = stream_splits(n, k, m)
-            if splits > 1:
-                out = torch.empty((splits, m, n), dtype=torch.float32, device=dev)
-                used = ops.gemm_stream(x, weight, out, splits=splits)
-                return out[:used]
+    fits = skinny_fits(x, weight)
+    if fits and allow_partials and (m <= SKINNY_MAX_ROWS or stream_pays_beyond_64_rows(m, n, k)):
+        splits = stream_splits(n, k, m)
+        if splits > 1:
+            out = torch.empty((splits, m, n), dtype=torch.float32, device=dev)
+            used = ops.gemm_stream(x, weight, out, splits=splits)
+            return out[:used]
+    if fits and (m <= SKINNY_MAX_ROWS or out_dtype == torch.float32):
         out = torch.empty((m, n), dtype=out_dtype, device=dev)
         for at in range(0, m, SKINNY_MAX_ROWS):
             xs, os_ = x[at:at + SKINNY_MAX_ROWS], out[at:at + SKINNY_MAX_ROWS]

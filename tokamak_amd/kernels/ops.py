@@ -482,6 +482,7 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, fewrows_spli
                                               _stream()), "gemm_tiled")
 
 
+STREAM_MAX_ROWS = 128     # rows of activations the streaming product takes (more than 64: eight-wave blocks)
 STREAM_SMALL_MATRIX_BYTES = 24 << 20   # below this a product's time is memory round trips, not bytes
 
 
@@ -509,6 +510,8 @@ def stream_waves(rows: int, k: int, gated: bool = False, n: int = 0) -> int:
     44 -> 42 us at 64 rows; 4B 29.6 -> 26.9, 14B 107 -> 94; at 32B three rounds of six lose to two
     of eight), and the plain product six only if, with the best split of K for each, one round of
     them covers a tenth more of the CUs (q/k/v of 8B: 64 x 4 blocks against 48 x 4)."""
+    if rows > 64:
+        return 8        # five to eight tiles of 16 rows: only blocks of eight waves are built for them
     if gated:
         if rows <= 16:
             waves = 2
@@ -576,8 +579,10 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
     n = w.shape[0]
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "the streaming product takes bfloat16 inputs")
     _need(w.shape[1] == k, "gemm shapes disagree")
-    _need(0 < m <= 64 and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
-          and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "streaming product needs M <= 64 and 16-byte aligned rows")
+    waves = waves or stream_waves(m, k, False, n)
+    _need(0 < m <= (STREAM_MAX_ROWS if waves == 8 else 64) and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0
+          and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0,
+          "streaming product needs M <= 64 (128 with eight waves) and 16-byte aligned rows")
     _need(out.is_cuda and out.stride(-1) == 1, "output must be a GPU tensor with unit inner stride")
     if splits == 1:
         _need(out.shape == (m, n), "output must be [M, N]")
@@ -589,7 +594,7 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, splits: 
     slabs = _row_scale(sumsq, m, "gemm_stream")
     _note(f"{m}x{n}x{k}", (n * k + m * k) * 2 + splits * m * n * out.element_size(), 2.0 * m * n * k)
     used = _fn("gemm_mfma", "tk_gemm_stream")(_code(out.dtype), _p(a), _p(w), _p(out), m, n, k, a.stride(0),
-                                              w.stride(0), ldc, splits, stride, waves or stream_waves(m, k, False, n),
+                                              w.stride(0), ldc, splits, stride, waves,
                                               _p(sumsq), slabs, float(eps), _stream())
     if used < 1:
         raise KernelError(f"gemm_stream failed with status {used}")
@@ -606,12 +611,14 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, w
     m, k = a.shape
     _need(w.shape[0] % 2 == 0 and w.shape[1] == k and out.shape == (m, w.shape[0] // 2), "gated product shapes disagree")
     _need(a.dtype == w.dtype == out.dtype == torch.bfloat16, "the gated product is bfloat16")
-    _need(0 < m <= 64 and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
-          and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gated product needs M <= 64 and 16-byte aligned rows")
+    waves = waves or stream_waves(m, k, True, w.shape[0] // 2)
+    _need(0 < m <= (STREAM_MAX_ROWS if waves == 8 else 64) and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0
+          and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0,
+          "gated product needs M <= 64 (128 with eight waves) and 16-byte aligned rows")
     slabs = _row_scale(sumsq, m, "gemm_stream_swiglu")
     _note(f"{m}x{w.shape[0]}x{k}", (w.shape[0] * k + m * k) * 2 + m * w.shape[0], 2.0 * m * w.shape[0] * k)
     _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
-                                                     w.stride(0), out.stride(0), waves or stream_waves(m, k, True, w.shape[0] // 2),
+                                                     w.stride(0), out.stride(0), waves,
                                                      _p(sumsq), slabs, float(eps), _stream()), "gemm_stream_swiglu")
 
 
