@@ -559,12 +559,9 @@ def test_streaming_product_of_65_to_128_rows(M, N, K):
     w = rand(N, K, seed=2, scale=K ** -0.5).to(torch.bfloat16).to(DEV)
     with pytest.raises(ops.KernelError):            # blocks of four or six waves are not built for them
         ops.gemm_stream(x, w, torch.empty((M, N), device=DEV), waves=4)
-    if N % 2 == 0:                                  # the gated product of the same operands
-        out = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
-        ops.gemm_stream_swiglu(x, w, out)
-        g = x.cpu().double() @ w[:N // 2].cpu().double().T
-        u = x.cpu().double() @ w[N // 2:].cpu().double().T
-        torch.testing.assert_close(out.cpu().double(), g / (1 + torch.exp(-g)) * u, rtol=2e-2, atol=1e-2)
+    if N % 2 == 0:                                  # the gated product stops at 64 rows
+        with pytest.raises(ops.KernelError):
+            ops.gemm_stream_swiglu(x, w, torch.empty((M, N // 2), dtype=torch.bfloat16, device=DEV))
 
 
 def test_products_of_65_to_128_rows_whose_reader_adds_partial_sums_stream_the_weights():

@@ -467,7 +467,7 @@ static int launch_stream_shape(const void* A, const void* W, void* C, int M, int
   else if (mt == 2) TK_STREAM(2);
   else if (mt == 3) TK_STREAM(3);
   else if (mt == 4) TK_STREAM(4);
-  else if constexpr (WAVES == 8) {  // 65 to 128 rows: blocks of eight waves only
+  else if constexpr (WAVES == 8 && !GATED) {  // 65 to 128 rows: blocks of eight waves, the plain product only
     if (mt == 5) TK_STREAM(5);
     else if (mt == 6) TK_STREAM(6);
     else if (mt == 7) TK_STREAM(7);
@@ -523,7 +523,7 @@ TK_API int tk_gemm_stream_swiglu(const void* A, const void* W, void* C, int M, i
                                  long ldw, long ldc, int waves, const float* sumsq, int slabs, float eps,
                                  hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (M > (waves >= 8 ? 128 : 64) || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
+  if (M > 64 || K < 8 || K % 8 != 0 || lda % 8 != 0 || ldw % 8 != 0) return -1;
   if (sumsq != nullptr && (M > 16 || slabs < 1 || slabs > kRowScaleSlabs || waves >= 6)) return -1;
   const int total_chunks = (K + SBK - 1) / SBK;
   return launch_stream<bf16_t, true>(waves, A, W, C, M, N, K, lda, ldw, ldc, total_chunks, 1, 0,

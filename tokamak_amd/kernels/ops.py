@@ -482,7 +482,7 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, fewrows_spli
                                               _stream()), "gemm_tiled")
 
 
-STREAM_MAX_ROWS = 128     # rows of activations the streaming product takes (more than 64: eight-wave blocks)
+STREAM_MAX_ROWS = 128     # rows of activations the streaming product takes (more than 64: eight-wave blocks, not the gated form)
 STREAM_SMALL_MATRIX_BYTES = 24 << 20   # below this a product's time is memory round trips, not bytes
 
 
@@ -612,9 +612,8 @@ def gemm_stream_swiglu(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, w
     _need(w.shape[0] % 2 == 0 and w.shape[1] == k and out.shape == (m, w.shape[0] // 2), "gated product shapes disagree")
     _need(a.dtype == w.dtype == out.dtype == torch.bfloat16, "the gated product is bfloat16")
     waves = waves or stream_waves(m, k, True, w.shape[0] // 2)
-    _need(0 < m <= (STREAM_MAX_ROWS if waves == 8 else 64) and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0
-          and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0,
-          "gated product needs M <= 64 (128 with eight waves) and 16-byte aligned rows")
+    _need(0 < m <= 64 and k >= 8 and k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+          and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "gated product needs M <= 64 and 16-byte aligned rows")
     slabs = _row_scale(sumsq, m, "gemm_stream_swiglu")
     _note(f"{m}x{w.shape[0]}x{k}", (w.shape[0] * k + m * k) * 2 + m * w.shape[0], 2.0 * m * w.shape[0] * k)
     _check(_fn("gemm_mfma", "tk_gemm_stream_swiglu")(_p(a), _p(w), _p(out), m, w.shape[0] // 2, k, a.stride(0),
