@@ -259,7 +259,7 @@ __device__ __forceinline__ unsigned long long fixed_mass(float x, float mx) {
 
 // f(index, value) for every element of a row, each by one thread of the block.  A block reads
 // its row alone, so what counts is the bytes it has in flight: 16-byte loads where the row's
-// address allows them (a pass over 152 k logits: 9 us instead of 29).
+// address allows them (a pass over 152 k logits: 14 us instead of 29 and more).
 template <typename F>
 __device__ __forceinline__ void for_row(const float* __restrict__ row, int V, F f) {
   const int tid = threadIdx.x;
