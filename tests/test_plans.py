@@ -134,3 +134,19 @@ def test_the_keys_of_few_tiles_are_split_over_blocks():
         split, nsplit = tile_split(tiles, per_tile, longest)
         if nsplit > 1:
             assert split % 64 == 0 and (nsplit - 1) * split < longest <= nsplit * split
+
+
+def test_the_streaming_product_takes_65_to_128_rows_where_it_was_measured_to_pay():
+    from tokamak_amd.kernels.gemm_bf16 import stream_pays_beyond_64_rows as pays
+
+    # up to 96 rows at every width; to 128 for matrices of 64 MB and more; never the tiny ones
+    for n, k in ((4096, 1024), (2048, 6144), (6144, 4096), (5120, 25600)):
+        assert not pays(64, n, k) and pays(65, n, k) and pays(96, n, k) and not pays(129, n, k)
+    assert not pays(97, 6144, 4096) and not pays(128, 4096, 4096)            # q/k/v and o of 8B: 50 and 34 MB
+    assert pays(128, 4096, 12288) and pays(97, 7168, 5120) and pays(128, 5120, 25600)
+    assert not pays(80, 48, 4096)                                            # fewer output columns than a block
+    # the plan of such a product: blocks of eight waves, one a CU, at least two chunks a share
+    for n, k, m in ((6144, 4096, 80), (4096, 12288, 128), (5120, 25600, 96), (2048, 6144, 70)):
+        assert ops.stream_waves(m, k, False, n) == 8
+        splits = stream_splits(n, k, m)
+        assert splits > 1 and splits * -(-n // 128) <= 256 and -(-k // 256) // splits >= 2
