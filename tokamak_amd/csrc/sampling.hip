@@ -31,9 +31,13 @@ __device__ __forceinline__ void argmax_take(float& bv, int& bi, float v, int i) 
   }
 }
 
+// temperature, top_k, top_p, part_mass (all or none): for a row with temperature > 0 and no
+// threshold the block also leaves the sum of e^((x - its segment's maximum) / temperature) over its segment, from which
+// the sampler has the mass of every segment without a pass of its own over the row.
 __global__ __launch_bounds__(kArgmaxThreads) void argmax_segments_kernel(
     const float* __restrict__ logits, float* __restrict__ part_v, int* __restrict__ part_i, int V,
-    long ld) {
+    long ld, const float* __restrict__ temperature, const int* __restrict__ top_k,
+    const float* __restrict__ top_p, float* __restrict__ part_mass) {
   __shared__ float best_v[kArgmaxThreads / kWave];
   __shared__ int best_i[kArgmaxThreads / kWave];
   const int seg = blockIdx.x, r = blockIdx.y;
@@ -71,10 +75,43 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_segments_kernel(
     best_i[wave] = bi;
   }
   __syncthreads();
+  for (int w = 0; w < kArgmaxThreads / kWave; ++w) argmax_take(bv, bi, best_v[w], best_i[w]);  // every thread: the segment's
   if (threadIdx.x == 0) {
-    for (int w = 1; w < kArgmaxThreads / kWave; ++w) argmax_take(bv, bi, best_v[w], best_i[w]);
     part_v[r * kArgmaxSegments + seg] = bv;
     part_i[r * kArgmaxSegments + seg] = bi;
+  }
+  if (part_mass == nullptr || !(temperature[r] > 0.f)) return;
+  if ((top_k[r] > 0 && top_k[r] < V) || top_p[r] < 1.f) return;  // a row with a threshold: the sampler sums what it keeps
+  // the segment again (it is in the cache): its mass relative to its own maximum
+  const float scale = 1.4426950408889634f / temperature[r];  // e^(y / t) = 2^(y log2 e / t)
+  float mass = 0.f;
+  const auto add = [&](float x) {
+    const float y = (x - bv) * scale;
+    if (y == y) mass += __builtin_amdgcn_exp2f(y);  // a NaN (also -inf - -inf of a segment without a number) adds nothing
+  };
+  if (vec) {
+    for (int i = begin + threadIdx.x * 4; i < end; i += kArgmaxThreads * 4) {
+      if (i + 4 <= end) {
+        const float4 v = *reinterpret_cast<const float4*>(row + i);
+        add(v.x);
+        add(v.y);
+        add(v.z);
+        add(v.w);
+      } else {
+        for (int j = i; j < end; ++j) add(row[j]);
+      }
+    }
+  } else {
+    for (int i = begin + threadIdx.x; i < end; i += kArgmaxThreads) add(row[i]);
+  }
+  mass = wave_sum(mass);
+  __syncthreads();  // best_v has been read
+  if (lane == 0) best_v[wave] = mass;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float total = 0.f;
+    for (int w = 0; w < kArgmaxThreads / kWave; ++w) total += best_v[w];
+    part_mass[r * kArgmaxSegments + seg] = total;
   }
 }
 
@@ -105,7 +142,21 @@ TK_API int tk_argmax(const float* logits, int* out, float* out_value, float* par
                      int V, long ld, hipStream_t stream) {
   if (M <= 0) return 0;
   if (V <= 0 || M > 65535) return -1;
-  argmax_segments_kernel<<<dim3(kArgmaxSegments, M), kArgmaxThreads, 0, stream>>>(logits, part_v, part_i, V, ld);
+  argmax_segments_kernel<<<dim3(kArgmaxSegments, M), kArgmaxThreads, 0, stream>>>(logits, part_v, part_i, V, ld,
+                                                                                   nullptr, nullptr, nullptr, nullptr);
+  argmax_pick_kernel<<<M, kWave, 0, stream>>>(part_v, part_i, out, out_value);
+  return launch_status();
+}
+
+// The same, and for the rows with temperature[m] > 0 and no threshold the mass of every segment
+// relative to its maximum at that temperature (part_mass: M * tk_argmax_segments() floats), for tk_sample.
+TK_API int tk_argmax_masses(const float* logits, int* out, float* out_value, float* part_v, int* part_i,
+                            const float* temperature, const int* top_k, const float* top_p, float* part_mass,
+                            int M, int V, long ld, hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (V <= 0 || M > 65535 || !temperature || !top_k || !top_p || !part_mass) return -1;
+  argmax_segments_kernel<<<dim3(kArgmaxSegments, M), kArgmaxThreads, 0, stream>>>(
+      logits, part_v, part_i, V, ld, temperature, top_k, top_p, part_mass);
   argmax_pick_kernel<<<M, kWave, 0, stream>>>(part_v, part_i, out, out_value);
   return launch_status();
 }
@@ -149,7 +200,7 @@ TK_API int tk_argmax_no_alloc(const float* logits, int* out, float* out_value, i
   ArgmaxScratch* scratch = argmax_scratch_of_current_device();
   if (scratch == nullptr) return -4;
   argmax_segments_kernel<<<dim3(kArgmaxSegments, M), kArgmaxThreads, 0, stream>>>(
-      logits, scratch->value, scratch->index, V, ld);
+      logits, scratch->value, scratch->index, V, ld, nullptr, nullptr, nullptr, nullptr);
   argmax_pick_kernel<<<M, kWave, 0, stream>>>(scratch->value, scratch->index, out, out_value);
   return launch_status();
 }
@@ -300,8 +351,9 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p,
     const unsigned long long* __restrict__ seeds, const unsigned long long* __restrict__ counters,
-    const float* __restrict__ row_max, int* __restrict__ out, float* __restrict__ probs_out) {
-  __shared__ float fs[16];
+    const float* __restrict__ row_max, const float* __restrict__ seg_max, const float* __restrict__ seg_mass,
+    int* __restrict__ out, float* __restrict__ probs_out) {
+  __shared__ float fs[kArgmaxSegments];  // the masses of the row's chunks (16 of the waves, or the 32 segments of the argmax pass)
   __shared__ unsigned long long hist64[kBins];
   __shared__ uint32_t hist32[kBins];
   __shared__ unsigned long long scan64[kSampleThreads];
@@ -449,9 +501,15 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   // final distribution over {x >= cut}.  The draw walks the tokens in index order: each
   // wave sums a contiguous chunk of the row; the chunk that holds the target is then
   // walked again by the whole block.
+  // Without a threshold the chunks are the segments of the argmax pass, which has left their
+  // masses (relative to each segment's own maximum): no pass over the row here.
   const int lane = tid & (kWave - 1), wave = tid / kWave;
   constexpr int kWaves = kSampleThreads / kWave;
-  const int chunk = ((V + kWaves - 1) / kWaves + 4 * kWave - 1) / (4 * kWave) * (4 * kWave);
+  static_assert(kWaves <= kArgmaxSegments, "fs holds either kind of chunk");
+  const bool by_segments = cut == 0 && seg_mass != nullptr;
+  const int nchunks = by_segments ? kArgmaxSegments : kWaves;
+  const int chunk = by_segments ? (((V + kArgmaxSegments - 1) / kArgmaxSegments + 3) & ~3)
+                                : ((V + kWaves - 1) / kWaves + 4 * kWave - 1) / (4 * kWave) * (4 * kWave);
   const int c_begin = wave * chunk, c_end = min(V, c_begin + chunk);
   float mine = 0.f;
   const auto kept_mass = [&](float logit) {
@@ -459,7 +517,14 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     return ordered(x) >= cut ? exp_unit(x - mx) : 0.f;
   };
   const int c_len = max(0, c_end - c_begin);
-  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {  // (chunks begin at multiples of 256 tokens)
+  if (by_segments) {
+    __syncthreads();
+    if (tid < kArgmaxSegments) {
+      const float m = seg_max[r * kArgmaxSegments + tid];
+      fs[tid] = m > -INFINITY ? seg_mass[r * kArgmaxSegments + tid] * exp_unit(m * inv_t - mx) : 0.f;
+    }
+    __syncthreads();
+  } else if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {  // (chunks begin at multiples of 256 tokens)
     const int quads = c_len / 4;
 #pragma unroll 8
     for (int q = lane; q < quads; q += kWave) {
@@ -471,12 +536,14 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 #pragma unroll 8
     for (int i = lane; i < c_len; i += kWave) mine += kept_mass(row[c_begin + i]);
   }
-  mine = wave_sum(mine);
-  __syncthreads();
-  if (lane == 0) fs[wave] = mine;
-  __syncthreads();
+  if (!by_segments) {
+    mine = wave_sum(mine);
+    __syncthreads();
+    if (lane == 0) fs[wave] = mine;
+    __syncthreads();
+  }
   float total = 0.f;
-  for (int w = 0; w < kWaves; ++w) total += fs[w];
+  for (int w = 0; w < nchunks; ++w) total += fs[w];
 
   if (probs_out) {
     float* po = probs_out + (size_t)r * V;
@@ -495,7 +562,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   {
     float run = 0.f;
     bool found = false;
-    for (int w = 0; w < kWaves; ++w) {
+    for (int w = 0; w < nchunks; ++w) {
       const float next = run + fs[w];
       if (!found && (target < next || w == sel)) {
         found = true;
@@ -548,14 +615,15 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
 // `out` must already hold each row's argmax and `row_max` its maximum (tk_argmax): greedy
 // rows keep the argmax, and so does a row whose search falls through (rounding at an edge).
+// seg_max, seg_mass (both or neither): what tk_argmax_masses left, [M][tk_argmax_segments()].
 TK_API int tk_sample(const float* logits, long ld, int M, int V, const float* temperature,
                      const int* top_k, const float* top_p, const unsigned long long* seeds,
-                     const unsigned long long* counters, const float* row_max, int* out,
-                     float* probs_out, hipStream_t stream) {
+                     const unsigned long long* counters, const float* row_max, const float* seg_max,
+                     const float* seg_mass, int* out, float* probs_out, hipStream_t stream) {
   if (M <= 0) return 0;
   if (V <= 0) return -1;
-  if (row_max == nullptr) return -1;
+  if (row_max == nullptr || (seg_max == nullptr) != (seg_mass == nullptr)) return -1;
   sample_kernel<<<M, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, seeds, counters,
-                                                  row_max, out, probs_out);
+                                                  row_max, seg_max, seg_mass, out, probs_out);
   return launch_status();
 }

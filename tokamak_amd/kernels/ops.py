@@ -219,9 +219,11 @@ _SIGS = {
     },
     "sampling": {
         "tk_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+        "tk_argmax_masses": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                             c_int, c_int, c_long, c_void_p],
         "tk_argmax_segments": [],
         "tk_sample": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     },
 }
 _LIBRARY_FILE = {"attention_fused": "attention_mfma"}   # signature group -> library that holds it
@@ -939,8 +941,18 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
         _need(t.numel() >= m, "one sampling parameter per row is required")
     _need(out.dtype == torch.int32, "sample output is int32")
     _need(probs_out is None or (probs_out.dtype == torch.float32 and probs_out.shape == (m, v)), "probs_out is float32 [M, V]")
-    row_max = torch.empty((m,), dtype=torch.float32, device=logits.device)
-    argmax(logits, out, row_max)  # greedy rows are done with this; the others overwrite it
+    _need(m <= 65535, "at most 65535 rows")
+    # the argmax pass: greedy rows are done with it, the others overwrite it; it also leaves every
+    # row's maximum and, segment by segment, the maxima and the masses at the row's temperature,
+    # from which a row without thresholds is drawn without another pass over its logits
+    segments = _fn("sampling", "tk_argmax_segments")()
+    floats = torch.empty((2 * segments + 1) * m, dtype=torch.float32, device=logits.device)
+    row_max, seg_max, seg_mass = floats[:m], floats[m:m + segments * m], floats[m + segments * m:]
+    seg_index = torch.empty(m * segments, dtype=torch.int32, device=logits.device)
+    _check(_fn("sampling", "tk_argmax_masses")(_p(logits), _p(out), _p(row_max), _p(seg_max), _p(seg_index),
+                                               _p(temperature), _p(top_k), _p(top_p), _p(seg_mass), m, v,
+                                               logits.stride(0), _stream()),
+           "argmax_masses")
     _check(_fn("sampling", "tk_sample")(_p(logits), logits.stride(0), m, v, _p(temperature), _p(top_k),
-                                        _p(top_p), _p(seeds), _p(counters), _p(row_max), _p(out),
-                                        _p(probs_out), _stream()), "sample")
+                                        _p(top_p), _p(seeds), _p(counters), _p(row_max), _p(seg_max), _p(seg_mass),
+                                        _p(out), _p(probs_out), _stream()), "sample")
