@@ -485,7 +485,7 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, fewrows_spli
 
 
 STREAM_MAX_ROWS = 128     # rows of activations the streaming product takes (more than 64: eight-wave blocks, not the gated form)
-STREAM_SMALL_MATRIX_BYTES = 24 << 20   # below this a product's time is memory round trips, not bytes
+STREAM_SMALL_MATRIX_BYTES = 20 << 20   # below this a product's time is memory round trips, not bytes
 
 
 def stream_waves(rows: int, k: int, gated: bool = False, n: int = 0) -> int:
@@ -522,7 +522,7 @@ def stream_waves(rows: int, k: int, gated: bool = False, n: int = 0) -> int:
         elif rows <= 48:
             waves = 2 if n < 8192 else 8
         else:
-            waves = 4 if n < 8192 else 8
+            waves = 2 if n < 4096 else 4 if n < 8192 else 8
         if waves == 2 and (2 * k) % 8192 == 0:
             waves = 4
         if waves == 8 and _rounds(n, 8 * 6) * 6 < _rounds(n, 8 * 8) * 8:
